@@ -1,0 +1,271 @@
+/*
+ * Tracea C ABI, MI355X (gfx950) implementation.
+ *
+ * Every declaration below keeps the name, argument order, field order and
+ * enumerator values of the interface it replaces in the reference, so that a
+ * program compiled against the reference's headers links against this
+ * library unchanged.  The reference file and line of each item is cited.
+ * Entry points that have no counterpart in the reference are grouped at the
+ * end and say so.
+ *
+ * Conventions shared by all calls
+ *   - pointers, shape arrays and stride arrays are borrowed for the duration
+ *     of the call and never freed by the library;
+ *   - strides are in ELEMENTS; a NULL stride array means contiguous row-major;
+ *   - device_id >= 0 names the HIP device that owns `ptr`; device_id == -1
+ *     (host memory) is rejected with TRACEA_CPU_ERROR: there is no CPU arm;
+ *   - `stream` is a hipStream_t passed through as void* (NULL = the default
+ *     stream); calls enqueue work and return without synchronising;
+ *   - a failing call returns a status other than TRACEA_SUCCESS and leaves a
+ *     human-readable message in a thread-local slot read with
+ *     tracea_get_last_error(); no C++ exception crosses the boundary.
+ */
+#ifndef TRACEA_H
+#define TRACEA_H
+
+#include <stdbool.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* reference: include/tracea.hpp:16-23.  TRACEA_CUDA_ERROR keeps its name for
+ * source compatibility; here it reports any HIP runtime / device failure. */
+typedef enum {
+  TRACEA_SUCCESS = 0,
+  TRACEA_INVALID_PARAMS = 1,
+  TRACEA_UNSUPPORTED_CONFIG = 2,
+  TRACEA_CUDA_ERROR = 3,
+  TRACEA_CPU_ERROR = 4,
+  TRACEA_UNKNOWN_ERROR = 99
+} TraceaStatus;
+
+/* reference: include/tracea.hpp:29-35 */
+typedef enum {
+  TRACEA_DTYPE_FLOAT32 = 0,
+  TRACEA_DTYPE_FLOAT16 = 1,
+  TRACEA_DTYPE_BFLOAT16 = 2,
+  TRACEA_DTYPE_INT32 = 3,
+  TRACEA_DTYPE_INT8 = 4
+} TraceaDType;
+
+/* reference: include/tracea.hpp:37-47; expansion into operator chains:
+ * src/interface/c_bindings.rs:144-197 */
+typedef enum {
+  TRACEA_EPILOGUE_IDENTITY = 0,
+  TRACEA_EPILOGUE_BIAS_ADD = 1,
+  TRACEA_EPILOGUE_RELU = 2,
+  TRACEA_EPILOGUE_GELU = 3,
+  TRACEA_EPILOGUE_SILU = 4,
+  TRACEA_EPILOGUE_BIAS_RELU = 5,
+  TRACEA_EPILOGUE_BIAS_SILU = 6,
+  TRACEA_EPILOGUE_RESIDUAL = 7,
+  TRACEA_EPILOGUE_RESIDUAL_RELU = 8
+} TraceaEpilogueKind;
+
+/* reference: include/tracea.hpp:49-53.  Accepted and ignored: the online
+ * softmax here always rescales once per key/value tile. */
+typedef enum {
+  TRACEA_SOFTMAX_AUTO = 0,
+  TRACEA_SOFTMAX_PER_TILE = 1,
+  TRACEA_SOFTMAX_PER_TWO_TILES = 2
+} TraceaSoftmaxGranularity;
+
+/* reference: include/tracea.hpp:59-66 */
+typedef struct {
+  void *ptr;
+  uint32_t rank;
+  const uint64_t *shape;
+  const int64_t *stride;
+  TraceaDType dtype;
+  int32_t device_id;
+} TraceaTensorView;
+
+/* reference: include/tracea.hpp:72-82 */
+typedef struct {
+  uint32_t stride_h;
+  uint32_t stride_w;
+  uint32_t padding_h;
+  uint32_t padding_w;
+  uint32_t dilation_h;
+  uint32_t dilation_w;
+  uint32_t groups;
+  TraceaEpilogueKind epilogue;
+  void *stream;
+} TraceaConv2dParams;
+
+/* reference: include/tracea.hpp:119-131 */
+typedef struct {
+  uint32_t stride_h;
+  uint32_t stride_w;
+  uint32_t padding_h;
+  uint32_t padding_w;
+  uint32_t output_padding_h;
+  uint32_t output_padding_w;
+  uint32_t dilation_h;
+  uint32_t dilation_w;
+  uint32_t groups;
+  TraceaEpilogueKind epilogue;
+  void *stream;
+} TraceaConvTranspose2dParams;
+
+/* reference: include/tracea.hpp:84-87 */
+typedef struct {
+  TraceaEpilogueKind epilogue;
+  void *stream;
+} TraceaGemmParams;
+
+/* reference: include/tracea.hpp:89-94.  scale == 0 selects 1/sqrt(D). */
+typedef struct {
+  uint8_t causal;
+  TraceaSoftmaxGranularity softmax_mode;
+  float scale;
+  void *stream;
+} TraceaAttentionParams;
+
+/* reference: include/tracea.h:15-20 */
+typedef struct {
+  bool success;
+  char *error_msg;
+  float score;      /* TFLOP/s of the winning configuration */
+  void *config_ptr; /* char*: PipelineConfig JSON; free with tracea_free_string */
+} TraceaResult;
+
+/* ---- lifecycle: reference include/tracea.h:26-31, src/interface/c_bindings.rs:105-125.
+ * tracea_init returns 0 on success.  It is idempotent.  Compute entry points
+ * called before it return TRACEA_UNKNOWN_ERROR (c_bindings.rs:212). */
+int tracea_init(void);
+void tracea_shutdown(void);
+void tracea_free_string(char *s);
+
+/* ---- implicit-GEMM convolution: reference include/tracea.hpp:107-110,
+ * src/interface/c_bindings.rs:206-290.
+ *   x   [N,H,W,C]   activations, channels innermost (NHWC)
+ *   w   [K,R,S,C]   filters as the reference reads the dims (c_bindings.rs:219-227);
+ *                   the physical order is taken from the strides, so both the
+ *                   K-major [K,R,S,C] and the [R,S,C,K] storage the reference's
+ *                   kernel indexes (src/emitter/cuda/conv.rs:253) are accepted
+ *   b   [K]         optional bias (f32, or the activation dtype)
+ *   residual        optional, shape of out
+ *   out [N,Ho,Wo,K] pre-allocated, Ho = (H + 2p - d(R-1) - 1)/s + 1
+ * groups must be 1; stride/padding/dilation may differ between h and w. */
+TraceaStatus tracea_conv2d(TraceaTensorView x, TraceaTensorView w, const TraceaTensorView *b,
+                           const TraceaTensorView *residual, TraceaTensorView *out,
+                           TraceaConv2dParams params);
+
+/* reference: include/tracea.hpp:133-137.  Outside the accelerated path:
+ * always returns TRACEA_UNSUPPORTED_CONFIG. */
+TraceaStatus tracea_conv_transpose2d(TraceaTensorView x, TraceaTensorView w,
+                                     const TraceaTensorView *b, const TraceaTensorView *residual,
+                                     TraceaTensorView *out, TraceaConvTranspose2dParams params);
+
+/* ---- GEMM C = epilogue(A.B): reference include/tracea.hpp:141-144,
+ * src/interface/c_bindings.rs:371-440.  a [M,K], b [K,N], c [M,N]; a
+ * column-major B is expressed through b's strides ({1, K}). */
+TraceaStatus tracea_gemm(TraceaTensorView a, TraceaTensorView b, const TraceaTensorView *bias,
+                         const TraceaTensorView *residual, TraceaTensorView *c,
+                         TraceaGemmParams params);
+
+/* ---- FlashAttention-2 forward: reference include/tracea.hpp:147-149,
+ * src/interface/c_bindings.rs:443-495.  q,k,v,o [B,H,S,D]. */
+TraceaStatus tracea_attention(TraceaTensorView q, TraceaTensorView k, TraceaTensorView v,
+                              TraceaTensorView *o, TraceaAttentionParams params);
+
+/* ---- errors and version: reference include/tracea.hpp:151-164,
+ * tracea-ffi/src/lib.rs:77-109, 244-251.  tracea_get_last_error copies at most
+ * len-1 bytes plus a NUL and returns the number of bytes copied, or -1 when
+ * buf is NULL or len is 0. */
+int32_t tracea_get_last_error(uint8_t *buf, size_t len);
+void tracea_clear_error(void);
+uint32_t tracea_version_major(void);
+uint32_t tracea_version_minor(void);
+uint32_t tracea_version_patch(void);
+
+/* ---- tuning: reference include/tracea.h:41-71 (the reference's bodies are
+ * stubs returning success=false, src/interface/c_bindings.rs:499-513).  Each
+ * call times every feasible kernel variant for the problem on synthetic
+ * device buffers, records the winner in the tuning cache and returns its
+ * PipelineConfig as JSON. */
+TraceaResult tracea_tune_gemm(size_t m, size_t n, size_t k);
+TraceaResult tracea_tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal);
+TraceaResult tracea_tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r,
+                                size_t s_kernel, size_t stride, size_t pad, size_t dilation);
+
+/* ======================================================================== */
+/* Additions.  None of these has a counterpart in the reference's headers.   */
+/* ======================================================================== */
+
+/* Operator vocabulary of the reference's EpilogueOp (src/core/op.rs:70-90)
+ * exposed one-to-one, plus the folded form of BatchNorm.  Applied to the fp32
+ * accumulator in list order before the conversion to the output dtype. */
+typedef enum {
+  TRACEA_EPI_OP_NONE = 0,
+  TRACEA_EPI_OP_BIAS_ADD = 1,      /* p0 = bias[channel] */
+  TRACEA_EPI_OP_RELU = 2,
+  TRACEA_EPI_OP_GELU = 3,
+  TRACEA_EPI_OP_SILU = 4,
+  TRACEA_EPI_OP_RESIDUAL_ADD = 5,  /* p0 = residual[row*ld + channel] */
+  TRACEA_EPI_OP_BIAS_ADD_SILU = 6, /* p0 = bias */
+  TRACEA_EPI_OP_BATCHNORM = 7,     /* p0..p3 = gamma, beta, mean, var (f32); epsilon */
+  TRACEA_EPI_OP_SCALE_SHIFT = 8    /* p0 = scale, p1 = shift (f32): folded BatchNorm */
+} TraceaEpilogueOpKind;
+
+typedef struct {
+  TraceaEpilogueOpKind kind;
+  TraceaDType dtype; /* element type of p0 for BIAS_ADD / RESIDUAL_ADD / BIAS_ADD_SILU */
+  const void *p0;
+  const void *p1;
+  const void *p2;
+  const void *p3;
+  float epsilon;
+  int64_t ld; /* RESIDUAL_ADD: row stride in elements; 0 = number of channels */
+} TraceaEpilogueOp;
+
+#define TRACEA_MAX_EPILOGUE_OPS 4
+
+/* tracea_conv2d / tracea_gemm with an explicit operator chain (at most
+ * TRACEA_MAX_EPILOGUE_OPS entries) instead of a TraceaEpilogueKind; the
+ * `epilogue` field of params is ignored.  This is how BatchNorm, which
+ * TraceaEpilogueKind cannot name, reaches the fused epilogue
+ * (fusion rules: src/core/optimizer.rs:122-150). */
+TraceaStatus tracea_conv2d_ex(TraceaTensorView x, TraceaTensorView w, TraceaTensorView *out,
+                              TraceaConv2dParams params, const TraceaEpilogueOp *ops,
+                              uint32_t n_ops);
+TraceaStatus tracea_gemm_ex(TraceaTensorView a, TraceaTensorView b, TraceaTensorView *c,
+                            TraceaGemmParams params, const TraceaEpilogueOp *ops, uint32_t n_ops);
+
+/* Kernel-variant control for tuners and benchmarks.  `op` is "gemm", "conv2d"
+ * or "attention".  A variant forced with tracea_force_variant (index >= 0) is
+ * used by every later call of that operator in the process whenever it is
+ * feasible for the problem; -1 restores automatic selection. */
+int32_t tracea_variant_count(const char *op);
+const char *tracea_variant_name(const char *op, int32_t index); /* library-owned */
+int32_t tracea_force_variant(const char *op, int32_t index);    /* 0 ok, -1 bad argument */
+
+/* The 80-byte ConvParams block of the reference (src/emitter/cuda/conv.rs:134-142;
+ * packing src/interface/python.rs:423-435) as this library computes it, for
+ * callers and tests that compare coordinate arithmetic bit for bit.  The
+ * shifts are those fast_divmod consumes (shift beyond 32). */
+typedef struct {
+  int32_t batch, h_in, w_in, c_in, k_out;
+  int32_t h_out, w_out, r_sz, s_sz;
+  int32_t stride, pad, dilation;
+  uint32_t hw_m, hw_s, w_m, w_s, sic_m, sic_s, c_m, c_s;
+} TraceaConvParamsBlock;
+TraceaStatus tracea_conv_params_pack(int32_t n, int32_t h, int32_t w, int32_t c, int32_t k,
+                                     int32_t r, int32_t s, int32_t stride, int32_t pad,
+                                     int32_t dilation, TraceaConvParamsBlock *out);
+
+/* Runs the device-side coordinate mapping of the convolution kernel for every
+ * GEMM row m and column k and writes {bn,ho,wo} per row, the batch base offset
+ * per row and {r,s,ci} per k into DEVICE buffers rows[M*3], base_off[M],
+ * cols[K*3]. */
+TraceaStatus tracea_conv_coords_device(const TraceaConvParamsBlock *p, int32_t *rows,
+                                       int64_t *base_off, int32_t *cols, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRACEA_H */

@@ -1,0 +1,120 @@
+"""Builds ``libtracea.so`` (HIP kernels for gfx950 + the C ABI) in-tree.
+
+Usage: ``python -m tracea_amd.build [--force] [-j N]``.  hipcc cross-compiles
+without a GPU, so this runs on any machine with ROCm installed.  Each line of
+``csrc/contraction_variants.def`` becomes one translation unit compiled from
+``csrc/contraction_variant.hip`` with the tile shape passed as -D flags.
+"""
+import argparse
+import concurrent.futures
+import hashlib
+import os
+import re
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "_obj")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB = os.path.join(LIB_DIR, "libtracea.so")
+
+ARCH = "gfx950"
+# -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.
+DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
+          "-Wno-pass-failed"]
+
+HOST_SOURCES = ["abi.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
+                "host/pipeline_config.cpp", "host/gaussian_process.cpp", "host/autotuner.cpp"]
+DEVICE_SOURCES = ["support_kernels.hip", "attention_kernels.hip"]
+
+
+def hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    return "hipcc"
+
+
+def variants():
+    text = open(os.path.join(CSRC, "contraction_variants.def")).read()
+    out = []
+    for m in re.finditer(r"^TRACEA_VARIANT\(([^)]*)\)", text, re.M):
+        f = [x.strip() for x in m.group(1).split(",")]
+        out.append(dict(name=f[0], bm=f[1], bn=f[2], bk=f[3], wm=f[4], wn=f[5], stages=f[6], direct=f[7]))
+    return out
+
+
+def _headers_digest():
+    h = hashlib.sha1()
+    for root, _, files in os.walk(CSRC):
+        for fn in sorted(files):
+            if fn.endswith((".hpp", ".h", ".def")):
+                h.update(open(os.path.join(root, fn), "rb").read())
+    h.update(open(os.path.join(HERE, "..", "include", "tracea.h"), "rb").read())
+    return h.hexdigest()
+
+
+def _jobs():
+    jobs = []
+    for v in variants():
+        defs = ["-DV_NAME=" + v["name"], "-DV_BM=" + v["bm"], "-DV_BN=" + v["bn"], "-DV_BK=" + v["bk"],
+                "-DV_WM=" + v["wm"], "-DV_WN=" + v["wn"], "-DV_STAGES=" + v["stages"],
+                "-DV_DIRECT=" + v["direct"]]
+        jobs.append((os.path.join(CSRC, "contraction_variant.hip"),
+                     os.path.join(OBJ, "variant_" + v["name"] + ".o"), DEVICE_FLAGS + defs))
+    for s in DEVICE_SOURCES:
+        jobs.append((os.path.join(CSRC, s), os.path.join(OBJ, s.replace("/", "_") + ".o"), DEVICE_FLAGS))
+    for s in HOST_SOURCES:
+        if os.path.exists(os.path.join(CSRC, s)):
+            jobs.append((os.path.join(CSRC, s), os.path.join(OBJ, s.replace("/", "_") + ".o"), []))
+    return jobs
+
+
+def _compile(job, digest, force):
+    src, obj, flags = job
+    stamp = obj + ".stamp"
+    key = hashlib.sha1((digest + open(src, "rb").read().hex() + " ".join(flags)).encode()).hexdigest()
+    if not force and os.path.exists(obj) and os.path.exists(stamp) and open(stamp).read() == key:
+        return obj, False
+    cmd = [hipcc()] + COMMON + flags + ["-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), r.stderr[-4000:]))
+    open(stamp, "w").write(key)
+    return obj, True
+
+
+def build(force=False, jobs=None, verbose=True):
+    """Compile every translation unit and link ``lib/libtracea.so``."""
+    os.makedirs(OBJ, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    digest = _headers_digest()
+    todo = _jobs()
+    jobs = jobs or min(8, os.cpu_count() or 4)
+    objs, rebuilt = [], 0
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        for obj, did in ex.map(lambda j: _compile(j, digest, force), todo):
+            objs.append(obj)
+            rebuilt += int(did)
+    if rebuilt or force or not os.path.exists(LIB):
+        cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o", LIB] + objs
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stderr[-4000:])
+    if verbose:
+        print("libtracea.so: %d of %d objects rebuilt -> %s" % (rebuilt, len(todo), LIB))
+    return LIB
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--force", action="store_true")
+    ap.add_argument("-j", type=int, default=None)
+    a = ap.parse_args()
+    try:
+        build(force=a.force, jobs=a.j)
+    except RuntimeError as e:
+        sys.stderr.write(str(e) + "\n")
+        sys.exit(1)

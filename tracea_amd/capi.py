@@ -1,0 +1,177 @@
+"""ctypes binding of the C ABI declared in ``include/tracea.h``.
+
+Nothing here computes: every call goes to ``libtracea.so``.  Loading fails
+loudly when the library has not been built (``python -m tracea_amd.build``).
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtracea.so")
+
+# TraceaStatus
+SUCCESS, INVALID_PARAMS, UNSUPPORTED_CONFIG, CUDA_ERROR, CPU_ERROR, UNKNOWN_ERROR = 0, 1, 2, 3, 4, 99
+# TraceaDType
+F32, F16, BF16, I32, I8 = 0, 1, 2, 3, 4
+# TraceaEpilogueKind
+(EPI_IDENTITY, EPI_BIAS_ADD, EPI_RELU, EPI_GELU, EPI_SILU, EPI_BIAS_RELU, EPI_BIAS_SILU,
+ EPI_RESIDUAL, EPI_RESIDUAL_RELU) = range(9)
+# TraceaEpilogueOpKind
+(OP_NONE, OP_BIAS_ADD, OP_RELU, OP_GELU, OP_SILU, OP_RESIDUAL_ADD, OP_BIAS_ADD_SILU, OP_BATCHNORM,
+ OP_SCALE_SHIFT) = range(9)
+MAX_EPILOGUE_OPS = 4
+
+
+class TensorView(C.Structure):
+    _fields_ = [("ptr", C.c_void_p), ("rank", C.c_uint32), ("shape", C.POINTER(C.c_uint64)),
+                ("stride", C.POINTER(C.c_int64)), ("dtype", C.c_int), ("device_id", C.c_int32)]
+
+
+class Conv2dParams(C.Structure):
+    _fields_ = [("stride_h", C.c_uint32), ("stride_w", C.c_uint32), ("padding_h", C.c_uint32),
+                ("padding_w", C.c_uint32), ("dilation_h", C.c_uint32), ("dilation_w", C.c_uint32),
+                ("groups", C.c_uint32), ("epilogue", C.c_int), ("stream", C.c_void_p)]
+
+
+class ConvTranspose2dParams(C.Structure):
+    _fields_ = [("stride_h", C.c_uint32), ("stride_w", C.c_uint32), ("padding_h", C.c_uint32),
+                ("padding_w", C.c_uint32), ("output_padding_h", C.c_uint32),
+                ("output_padding_w", C.c_uint32), ("dilation_h", C.c_uint32),
+                ("dilation_w", C.c_uint32), ("groups", C.c_uint32), ("epilogue", C.c_int),
+                ("stream", C.c_void_p)]
+
+
+class GemmParams(C.Structure):
+    _fields_ = [("epilogue", C.c_int), ("stream", C.c_void_p)]
+
+
+class AttentionParams(C.Structure):
+    _fields_ = [("causal", C.c_uint8), ("softmax_mode", C.c_int), ("scale", C.c_float),
+                ("stream", C.c_void_p)]
+
+
+class Result(C.Structure):
+    _fields_ = [("success", C.c_bool), ("error_msg", C.c_void_p), ("score", C.c_float),
+                ("config_ptr", C.c_void_p)]
+
+
+class EpilogueOp(C.Structure):
+    _fields_ = [("kind", C.c_int), ("dtype", C.c_int), ("p0", C.c_void_p), ("p1", C.c_void_p),
+                ("p2", C.c_void_p), ("p3", C.c_void_p), ("epsilon", C.c_float), ("ld", C.c_int64)]
+
+
+class ConvParamsBlock(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("batch", "h_in", "w_in", "c_in", "k_out", "h_out", "w_out", "r_sz", "s_sz",
+                 "stride", "pad", "dilation")] + \
+               [(n, C.c_uint32) for n in
+                ("hw_m", "hw_s", "w_m", "w_s", "sic_m", "sic_s", "c_m", "c_s")]
+
+
+# name -> (restype, argtypes); every symbol include/tracea.h declares
+SIGNATURES = {
+    "tracea_init": (C.c_int, []),
+    "tracea_shutdown": (None, []),
+    "tracea_free_string": (None, [C.c_void_p]),
+    "tracea_conv2d": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), C.POINTER(TensorView),
+                                C.POINTER(TensorView), Conv2dParams]),
+    "tracea_conv_transpose2d": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView),
+                                          C.POINTER(TensorView), C.POINTER(TensorView),
+                                          ConvTranspose2dParams]),
+    "tracea_gemm": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), C.POINTER(TensorView),
+                              C.POINTER(TensorView), GemmParams]),
+    "tracea_attention": (C.c_int, [TensorView, TensorView, TensorView, C.POINTER(TensorView),
+                                   AttentionParams]),
+    "tracea_get_last_error": (C.c_int32, [C.c_char_p, C.c_size_t]),
+    "tracea_clear_error": (None, []),
+    "tracea_version_major": (C.c_uint32, []),
+    "tracea_version_minor": (C.c_uint32, []),
+    "tracea_version_patch": (C.c_uint32, []),
+    "tracea_tune_gemm": (Result, [C.c_size_t, C.c_size_t, C.c_size_t]),
+    "tracea_tune_fa2": (Result, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_bool]),
+    "tracea_tune_conv2d": (Result, [C.c_size_t] * 10),
+    "tracea_conv2d_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), Conv2dParams,
+                                   C.POINTER(EpilogueOp), C.c_uint32]),
+    "tracea_gemm_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), GemmParams,
+                                 C.POINTER(EpilogueOp), C.c_uint32]),
+    "tracea_variant_count": (C.c_int32, [C.c_char_p]),
+    "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),
+    "tracea_force_variant": (C.c_int32, [C.c_char_p, C.c_int32]),
+    "tracea_conv_params_pack": (C.c_int, [C.c_int32] * 10 + [C.POINTER(ConvParamsBlock)]),
+    "tracea_conv_coords_device": (C.c_int, [C.POINTER(ConvParamsBlock), C.c_void_p, C.c_void_p,
+                                            C.c_void_p, C.c_void_p]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library; raises if it was not built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libtracea.so is missing (%s); run `python -m tracea_amd.build`"
+                               % LIB_PATH)
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def last_error():
+    buf = C.create_string_buffer(1024)
+    n = lib().tracea_get_last_error(buf, len(buf))
+    return buf.raw[:n].decode("utf-8", "replace") if n > 0 else ""
+
+
+class TraceaError(RuntimeError):
+    def __init__(self, what, status):
+        self.status = status
+        super().__init__("%s failed (status %d): %s" % (what, status, last_error()))
+
+
+def check(what, status):
+    if status != SUCCESS:
+        raise TraceaError(what, status)
+
+
+def init():
+    """tracea_init(); raises when no HIP device is usable."""
+    if lib().tracea_init() != 0:
+        raise RuntimeError("tracea_init failed: " + last_error())
+
+
+class View:
+    """Owns the shape/stride arrays a TraceaTensorView borrows."""
+
+    def __init__(self, ptr, shape, stride, dtype, device_id):
+        self._shape = (C.c_uint64 * len(shape))(*shape)
+        self._stride = (C.c_int64 * len(stride))(*stride) if stride is not None else None
+        self.c = TensorView(ptr, len(shape), self._shape,
+                            self._stride if stride is not None else None, dtype, device_id)
+
+
+def take_result(res):
+    """TraceaResult -> (success, score, config_json, error); frees the strings."""
+    cfg = C.string_at(res.config_ptr).decode() if res.config_ptr else None
+    err = C.string_at(res.error_msg).decode() if res.error_msg else None
+    if res.config_ptr:
+        lib().tracea_free_string(res.config_ptr)
+    if res.error_msg:
+        lib().tracea_free_string(res.error_msg)
+    return bool(res.success), float(res.score), cfg, err
+
+
+def variants(op):
+    n = lib().tracea_variant_count(op.encode())
+    return [lib().tracea_variant_name(op.encode(), i).decode() for i in range(max(n, 0))]
+
+
+def force_variant(op, index_or_name):
+    if isinstance(index_or_name, str):
+        index_or_name = variants(op).index(index_or_name)
+    if lib().tracea_force_variant(op.encode(), int(index_or_name)) != 0:
+        raise ValueError("bad variant %r for %s" % (index_or_name, op))

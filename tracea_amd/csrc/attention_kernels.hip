@@ -1,0 +1,333 @@
+// FlashAttention-2 forward for gfx950.
+//
+// Replaces flash_attention_v2_kernel of the reference
+// (src/kernels/attention/cuda_emitter.rs:69-238) and fa2_template_kernel
+// (src/kernels/gpu/templates_fa2.cu:41-388): O = softmax(scale Q K^T) V with
+// an online (running max / running sum) softmax in fp32, one pass over K/V.
+// Causal masking follows the reference's intent (keys strictly after the
+// query are excluded, cuda_emitter.rs.tmp:217-218); sequence-length bounds
+// masking follows templates_fa2.cu:201-206.  Masked scores are -inf instead of
+// the reference's -50000 sentinel, and the final division uses the exact l
+// (the reference adds 1e-9 / 1e-6): both differences are far below bf16
+// resolution.
+//
+// Work split: a workgroup of 4 waves owns 128 query rows of one (batch, head);
+// each wave owns 32 of them.  Per 64-key tile the wave computes the TRANSPOSED
+// score block S^T = K Q^T with v_mfma_f32_32x32x16 (A operand = 32 keys from
+// LDS, B operand = the wave's 32 queries, resident in registers).  In the
+// 32x32 accumulator layout lane l then holds scores of ONE query (l & 31) for
+// 32 of the 64 keys; its partner lane l^32 holds the other 32.  Row max and
+// row sum are therefore in-register reductions plus a single cross-lane
+// exchange per tile, and P^T is already laid out as the B operand of the
+// second product O^T += V^T P^T without touching LDS: accumulator registers
+// 8h..8h+7 of block b, converted to 16 bit, are exactly the 8 k-slots a lane
+// feeds to the MFMA that covers keys 32b+16h..+15, provided the A operand
+// (V^T) enumerates the keys in the same order.  That order is
+// key(slot j, half g) = 8*(j/4) + 4g + j%4, i.e. two runs of four consecutive
+// keys at a fixed head-dim column, which the LDS transpose load
+// ds_read_b64_tr_b16 delivers from a row-major [key][d] tile.
+// O^T accumulators of a lane all belong to the lane's query, so the online
+// rescale is a per-lane scalar multiply.
+#include "contraction_kernel.hpp"
+
+namespace tracea_amd {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ u32x4 pack8(const float (&p)[8]) {
+  if constexpr (DT == DT_F16) {
+    f16x8 h = {(_Float16)p[0], (_Float16)p[1], (_Float16)p[2], (_Float16)p[3],
+               (_Float16)p[4], (_Float16)p[5], (_Float16)p[6], (_Float16)p[7]};
+    return __builtin_bit_cast(u32x4, h);
+  } else {
+    bf16x8 h = {(__bf16)p[0], (__bf16)p[1], (__bf16)p[2], (__bf16)p[3],
+                (__bf16)p[4], (__bf16)p[5], (__bf16)p[6], (__bf16)p[7]};
+    return __builtin_bit_cast(u32x4, h);
+  }
+}
+
+constexpr int FA_BQ = 128;   // query rows per workgroup
+constexpr int FA_BKV = 64;   // keys per tile
+constexpr int FA_WAVES = 4;
+
+// V_TR: fetch the V^T operand with the LDS transpose load (fast); otherwise
+// with eight 16-bit LDS reads per operand (slow, instruction-for-instruction
+// obvious; kept as the cross-check of the transpose path).
+template <int DT, int D, bool V_TR>
+__global__ void __launch_bounds__(FA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+fa2_fwd_kernel(const AttentionArgs a) {
+  constexpr int NT = FA_WAVES * 64;
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CH = D / 8;                      // 16-byte pieces per row
+  constexpr int TILE_BYTES = FA_BKV * ROW_BYTES; // one K or V tile
+  constexpr int STAGE = 2 * TILE_BYTES;          // K + V
+  constexpr int NP = FA_BKV * CH / NT;           // pieces per thread per tensor per tile
+  constexpr int KS = D / 16;                     // k steps of the score product
+  constexpr int DB = D / 32;                     // 32-wide head-dim blocks of O^T
+  static_assert(D % 32 == 0 && (FA_BKV * CH) % NT == 0, "unsupported head dim");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 31, g = lane >> 5;
+
+  // workgroup -> (batch*head, query block); consecutive ids land on different
+  // XCDs, so regroup them to keep one head's K/V in one L2, and walk the query
+  // blocks from the last (most keys under a causal mask) to the first.
+  const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
+  const int total = nqb * a.B * a.H;
+  int vid = blockIdx.x;
+  if ((total & 7) == 0) vid = (vid & 7) * (total >> 3) + (vid >> 3);
+  const int bh = vid / nqb;
+  const int qb = nqb - 1 - (vid - bh * nqb);
+  const int b = bh / a.H, h = bh - b * a.H;
+  const int q0 = qb * FA_BQ;
+  const int S = a.S;
+
+  const unsigned short *Qg = (const unsigned short *)a.Q + (long long)b * a.q_sb + (long long)h * a.q_sh;
+  const unsigned short *Kg = (const unsigned short *)a.K + (long long)b * a.k_sb + (long long)h * a.k_sh;
+  const unsigned short *Vg = (const unsigned short *)a.V + (long long)b * a.v_sb + (long long)h * a.v_sh;
+  unsigned short *Og = (unsigned short *)a.O + (long long)b * a.o_sb + (long long)h * a.o_sh;
+
+  // ---- this wave's 32 queries, B operand of S^T: lane (q = lrow, g) holds
+  //      Q[q][16*ks + 8*g .. +7] for every k step ----
+  const int q_wave0 = q0 + wave * 32;
+  const int q_mine = q_wave0 + lrow;
+  u32x4 qf[KS];
+  {
+    const int qr = q_mine < S ? q_mine : S - 1;
+    const unsigned short *qp = Qg + (long long)qr * a.q_ss + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4 *)(qp + ks * 16);
+  }
+
+  // ---- key/value tile movement: piece p -> row p / CH, 16-byte column p % CH.
+  //      K rows are swizzled for 32 lanes reading the same column of 32 rows;
+  //      V rows are swizzled at 64-byte granularity for the transpose load,
+  //      whose 32 lanes read a 64-byte window of 4 consecutive rows. ----
+  auto k_piece = [&](int row, int c) -> int { return row * ROW_BYTES + ((c ^ (row & (CH - 1))) << 4); };
+  auto v_piece = [&](int row, int c) -> int { return row * ROW_BYTES + ((c ^ ((row & 3) << 2)) << 4); };
+
+  const int ntiles_all = (S + FA_BKV - 1) / FA_BKV;
+  int ntiles = ntiles_all;
+  if (a.causal) {
+    const int last_q = (q0 + FA_BQ - 1 < S ? q0 + FA_BQ - 1 : S - 1);
+    const int need = last_q / FA_BKV + 1;
+    ntiles = need < ntiles ? need : ntiles;
+  }
+
+  u32x4 rk[NP], rv[NP];
+  auto fetch = [&](int t) {
+    const int kv0 = t * FA_BKV;
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = tid + i * NT;
+      int row = kv0 + p / CH;
+      row = row < S ? row : S - 1;  // rows beyond S are masked in the scores
+      const int c = p % CH;
+      rk[i] = *(const u32x4 *)(Kg + (long long)row * a.k_ss + c * 8);
+      rv[i] = *(const u32x4 *)(Vg + (long long)row * a.v_ss + c * 8);
+    }
+  };
+  auto stash = [&](unsigned char *sK, unsigned char *sV) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = tid + i * NT;
+      const int row = p / CH, c = p % CH;
+      *(u32x4 *)(sK + k_piece(row, c)) = rk[i];
+      *(u32x4 *)(sV + v_piece(row, c)) = rv[i];
+    }
+  };
+
+  f32x16 o[DB];
+#pragma unroll
+  for (int d = 0; d < DB; ++d)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[d][e] = 0.0f;
+  float m_run = -1.0e30f;  // running max, log2 domain, finite so that exp2(m-m) is 1
+  float l_run = 0.0f;      // this lane's share of the running sum
+
+  fetch(0);
+  stash(smem, smem + TILE_BYTES);
+  __syncthreads();
+
+  for (int t = 0; t < ntiles; ++t) {
+    const unsigned char *sK = smem + (t & 1) * STAGE;
+    const unsigned char *sV = sK + TILE_BYTES;
+    unsigned char *nK = smem + ((t + 1) & 1) * STAGE;
+    const bool more = t + 1 < ntiles;
+    fetch(more ? t + 1 : t);
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int kv0 = t * FA_BKV;
+    // a wave whose every query precedes every key of the tile has nothing to add
+    const bool wave_active = !(a.causal && kv0 > q_wave0 + 31);
+    if (wave_active) {
+      // ---- S^T = K Q^T : two 32-key blocks ----
+      f32x16 s[2];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[blk][e] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+          const u32x4 kf = *(const u32x4 *)(sK + k_piece(blk * 32 + lrow, ks * 2 + g));
+          s[blk] = Mfma32<DT>::run(kf, qf[ks], s[blk]);
+        }
+      }
+
+      // ---- scale to the log2 domain, mask, running max ----
+      const bool edge = (kv0 + FA_BKV > S) || (a.causal && kv0 + FA_BKV - 1 > q_wave0);
+      float mx = -INFINITY;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          float x = s[blk][e] * a.scale_log2;
+          if (edge) {
+            const int kv = kv0 + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+            if (kv >= S || (a.causal && kv > q_mine)) x = -INFINITY;
+          }
+          s[blk][e] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = exp2f(m_run - m_new);
+      m_run = m_new;
+
+      // ---- P = exp2(S - m), row-sum share, B operands of the second product ----
+      float lsum = 0.0f;
+      u32x4 pf[4];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          float p[8];
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            p[j] = exp2f(s[blk][hh * 8 + j] - m_new);
+            lsum += p[j];
+          }
+          pf[blk * 2 + hh] = pack8<DT>(p);
+        }
+      l_run = l_run * alpha + lsum;
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
+
+      // ---- O^T += V^T P^T : 4 key groups of 16 x DB head-dim blocks ----
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+        for (int d = 0; d < DB; ++d) {
+          u32x4 vf;
+          if constexpr (V_TR) {
+            // 16-lane group: lane r supplies row (base + r/4), 4 columns at
+            // 4*(r%4) of its 16-column window; lane n receives column n of the
+            // 4 rows.
+            const int r = lane & 15;
+            const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
+            const int row_lo = kk * 16 + g * 4 + (r >> 2);
+            const int row_hi = row_lo + 8;
+            const unsigned char *p_lo = sV + v_piece(row_lo, col >> 3) + (col & 7) * 2;
+            const unsigned char *p_hi = sV + v_piece(row_hi, col >> 3) + (col & 7) * 2;
+            const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4 *)(p_lo));
+            const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4 *)(p_hi));
+            const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+            vf[0] = lo2[0]; vf[1] = lo2[1]; vf[2] = hi2[0]; vf[3] = hi2[1];
+          } else {
+            const int col = d * 32 + lrow;
+            unsigned short hv[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              const int row = kk * 16 + (j >> 2) * 8 + g * 4 + (j & 3);
+              hv[j] = *(const unsigned short *)(sV + v_piece(row, col >> 3) + (col & 7) * 2);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) vf[j] = (unsigned)hv[2 * j] | ((unsigned)hv[2 * j + 1] << 16);
+          }
+          o[d] = Mfma32<DT>::run(vf, pf[kk], o[d]);
+        }
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (more) stash(nK, nK + TILE_BYTES);
+    __syncthreads();
+  }
+
+  // ---- normalise, regroup through LDS, store 16 bytes per lane ----
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv_l = 1.0f / l_tot;
+  unsigned char *so = smem + wave * (32 * ROW_BYTES);  // [32 queries][D] of the output type
+#pragma unroll
+  for (int d = 0; d < DB; ++d)
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      float x[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = o[d][v4 * 4 + e] * inv_l;
+      u32x2 w;
+      if constexpr (DT == DT_F16) {
+        f16x4 hq = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+        w = __builtin_bit_cast(u32x2, hq);
+      } else {
+        bf16x4 hq = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
+        w = __builtin_bit_cast(u32x2, hq);
+      }
+      *(u32x2 *)(so + lrow * ROW_BYTES + (d * 32 + v4 * 8 + g * 4) * 2) = w;
+    }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 32 * CH / 64; ++i) {
+    const int p = lane + i * 64;
+    const int row = p / CH, c = p % CH;
+    const int q = q_wave0 + row;
+    if (q < S)
+      *(u32x4 *)(Og + (long long)q * a.o_ss + c * 8) = *(const u32x4 *)(so + row * ROW_BYTES + c * 16);
+  }
+}
+
+template <int D, bool V_TR>
+static int launch_fa2(const AttentionArgs &a, int dtype, hipStream_t stream) {
+  constexpr size_t lds = 2 * 2 * (size_t)FA_BKV * D * 2;
+  const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
+  const dim3 grid((unsigned)(nqb * a.B * a.H)), block(FA_WAVES * 64);
+#define TRACEA_FA_LAUNCH(DTV)                                                                  \
+  do {                                                                                         \
+    auto kfn = fa2_fwd_kernel<DTV, D, V_TR>;                                                   \
+    static bool attr_done = false;                                                             \
+    if (!attr_done) {                                                                          \
+      hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return (int)e;                                                      \
+      attr_done = true;                                                                        \
+    }                                                                                          \
+    hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                      \
+    return (int)hipGetLastError();                                                             \
+  } while (0)
+  if (dtype == DT_F16) TRACEA_FA_LAUNCH(DT_F16);
+  else TRACEA_FA_LAUNCH(DT_BF16);
+#undef TRACEA_FA_LAUNCH
+}
+
+static bool feasible_d128(const AttentionArgs &a) { return a.D == 128; }
+static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
+
+static const AttentionVariant kAttentionVariants[] = {
+    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, true>, &feasible_d128},
+    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, false>, &feasible_d128},
+    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<64, true>, &feasible_d64},
+    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<64, false>, &feasible_d64},
+};
+
+int attention_variant_count() { return (int)(sizeof(kAttentionVariants) / sizeof(kAttentionVariants[0])); }
+const AttentionVariant &attention_variant(int i) { return kAttentionVariants[i]; }
+
+}  // namespace tracea_amd

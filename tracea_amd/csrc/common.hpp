@@ -1,0 +1,103 @@
+// Shared host/device declarations of the MI355X Tracea library.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/tracea.h"
+
+namespace tracea_amd {
+
+// Element types the matrix-core kernels compute in (fp32 accumulate always).
+enum DataType : int { DT_F32 = 0, DT_F16 = 1, DT_BF16 = 2 };
+
+// One fused epilogue operator; mirrors TraceaEpilogueOp with device pointers.
+struct EpilogueOpDev {
+  int kind;   // TraceaEpilogueOpKind
+  int dtype;  // DataType of p0 when p0 is a bias or residual
+  const void *p0, *p1, *p2, *p3;
+  float epsilon;
+  long long ld;  // residual row stride, elements
+};
+
+struct EpilogueChain {
+  int n_ops;
+  EpilogueOpDev ops[TRACEA_MAX_EPILOGUE_OPS];
+};
+
+// Problem description handed to the contraction kernels.  For a convolution
+// the GEMM view is M = batch*h_out*w_out, N = k_out, K = r*s*c_in, A is the
+// NHWC activation tensor and B the filter bank.
+struct ContractionArgs {
+  const void *A;
+  const void *B;
+  void *C;
+  int M, N, K;
+  long long lda;       // A row stride (GEMM only), elements
+  long long ldb;       // B: stride between consecutive n (K-contiguous B) or k (N-contiguous B)
+  long long ldc;       // C row stride, elements
+  int out_dtype;       // DataType of C
+  int grid_m, grid_n;  // tiles along M and N
+  int group_m;         // tile-order group height
+  // convolution geometry (ConvParams of the reference, h/w split)
+  int h_in, w_in, c_in, h_out, w_out, s_sz;
+  int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+  unsigned hw_m, hw_s, w_m, w_s, sc_m, sc_s, c_m, c_s;
+  EpilogueChain epi;
+};
+
+struct AttentionArgs {
+  const void *Q, *K, *V;
+  void *O;
+  int B, H, S, D;
+  long long q_sb, q_sh, q_ss;  // element strides of batch, head, row (D contiguous)
+  long long k_sb, k_sh, k_ss;
+  long long v_sb, v_sh, v_ss;
+  long long o_sb, o_sh, o_ss;
+  float scale_log2;  // softmax scale * log2(e)
+  int causal;
+};
+
+// A precompiled kernel variant and the rule that says when it applies.
+struct ContractionVariant {
+  const char *name;
+  int bm, bn, bk, waves_m, waves_n, stages;
+  bool direct_to_lds;
+  size_t lds_bytes;
+  // launch: returns hipError_t as int
+  int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);
+};
+
+int contraction_variant_count();
+const ContractionVariant &contraction_variant(int i);
+
+// fp32 MFMA GEMM (row-major A [M,K], row-major B [K,N]).
+int launch_gemm_f32(const ContractionArgs &args, hipStream_t stream);
+// Any dtype/stride combination, no alignment requirement (VALU, slow).
+struct GenericGemmArgs {
+  const void *A, *B;
+  void *C;
+  int M, N, K;
+  long long sam, sak, sbk, sbn, scm, scn;
+  int a_dtype, b_dtype, c_dtype;
+  EpilogueChain epi;
+};
+int launch_gemm_generic(const GenericGemmArgs &args, hipStream_t stream);
+
+struct AttentionVariant {
+  const char *name;
+  int block_q, block_kv, waves;
+  int (*launch)(const AttentionArgs &, int dtype, hipStream_t);
+  bool (*feasible)(const AttentionArgs &);
+};
+int attention_variant_count();
+const AttentionVariant &attention_variant(int i);
+
+// Fills n elements with a counter-based pseudo-random sequence, uniform in
+// [-amplitude, amplitude] (synthetic operands for the tuner).
+int launch_fill_uniform(void *ptr, size_t n, int dtype, unsigned seed, float amplitude,
+                        hipStream_t stream);
+
+int launch_conv_coords(const TraceaConvParamsBlock &p, int32_t *rows, int64_t *base_off,
+                       int32_t *cols, hipStream_t stream);
+
+}  // namespace tracea_amd

@@ -1,0 +1,545 @@
+// MFMA contraction kernel for gfx950: one template covers the fp16/bf16 GEMM
+// and the implicit-GEMM convolution (they differ only in how a 16-byte piece
+// of the A operand is located in global memory).
+//
+// Behaviour it replaces in the reference: gemm_mma_kernel
+// (src/emitter/cuda/gemm.rs:92-207) and kernel_main / conv2d_implicit_gemm
+// (src/emitter/cuda/conv.rs:153-331); epilogue functors
+// src/kernels/gpu/epilogue.cuh:12-63.
+//
+// Structure
+//   * block tile BM x BN x BK, WM x WN wavefronts of 64 lanes, each wave owns
+//     (BM/WM) x (BN/WN) of C as 32x32 MFMA blocks (v_mfma_f32_32x32x16);
+//   * both operands are staged K-contiguous in LDS ([row][BK] halves) with an
+//     XOR swizzle of the 16-byte column index so that the ds_read_b128 operand
+//     fetches of 16 consecutive rows fall in 16 different bank groups;
+//   * global memory is read in 16-byte pieces, 8 lanes per 128-byte row
+//     segment; the next K tile is fetched into registers while the current one
+//     is multiplied, then written to the other LDS stage (one barrier per K
+//     tile);
+//   * the MFMA is issued with the operands swapped (D = B_frag x A_frag) so a
+//     lane ends up with 4 consecutive output channels of one row; the epilogue
+//     regroups the accumulators through LDS into 8 consecutive channels per
+//     lane, applies the fused operator chain on fp32 and stores 16 bytes.
+#pragma once
+#include "common.hpp"
+
+namespace tracea_amd {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+struct Mfma32;
+template <>
+struct Mfma32<DT_F16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma32<DT_BF16> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
+// q = n / d, r = n % d through a precomputed reciprocal: m = ceil(2^(32+s)/d),
+// or m == 0 for a power-of-two d with s = log2(d).  Same arithmetic as the
+// reference's device fast_divmod (src/emitter/cuda/conv.rs:144-151).
+__device__ __forceinline__ void fast_divmod(int n, unsigned m, unsigned s, int d, int &q, int &r) {
+  if (d == 1) {
+    q = n;
+    r = 0;
+  } else if (m == 0) {
+    q = n >> s;
+    r = n & (d - 1);
+  } else {
+    q = (int)(__umulhi((unsigned)n, m) >> s);
+    r = n - q * d;
+  }
+}
+
+// ---- epilogue helpers -------------------------------------------------------
+
+// Loads V (1, 4 or 8) consecutive elements starting at index idx as floats;
+// elements at or beyond nvalid read as zero.  One vector load when the run is
+// complete and naturally aligned, scalar loads otherwise.
+template <int V>
+__device__ __forceinline__ void load_as_float(const void *base, int dtype, long long idx,
+                                              int nvalid, float (&out)[V]) {
+  if (dtype == DT_F32) {
+    const float *p = (const float *)base + idx;
+    if (V > 1 && nvalid >= V && (((uintptr_t)p) & 15) == 0) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        f32x4 v = ((const f32x4 *)p)[q];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[q * 4 + e] = v[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = e < nvalid ? p[e] : 0.0f;
+    }
+  } else if (dtype == DT_F16) {
+    const _Float16 *p = (const _Float16 *)base + idx;
+    if (V > 1 && nvalid >= V && (((uintptr_t)p) & (V * 2 - 1)) == 0) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        f16x4 v = ((const f16x4 *)p)[q];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[q * 4 + e] = (float)v[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = e < nvalid ? (float)p[e] : 0.0f;
+    }
+  } else {
+    const __bf16 *p = (const __bf16 *)base + idx;
+    if (V > 1 && nvalid >= V && (((uintptr_t)p) & (V * 2 - 1)) == 0) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        bf16x4 v = ((const bf16x4 *)p)[q];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[q * 4 + e] = (float)v[e];
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e) out[e] = e < nvalid ? (float)p[e] : 0.0f;
+    }
+  }
+}
+
+// Applies the operator chain, in order, to V consecutive channels n..n+V-1 of
+// output row m (fp32 in, fp32 out).
+template <int V>
+__device__ __forceinline__ void apply_epilogue(float (&v)[V], long long m, int n, int nvalid,
+                                               const EpilogueChain &chain) {
+  for (int o = 0; o < chain.n_ops; ++o) {
+    const EpilogueOpDev &op = chain.ops[o];
+    float t[V];
+    switch (op.kind) {
+      case TRACEA_EPI_OP_BIAS_ADD:
+        load_as_float<V>(op.p0, op.dtype, n, nvalid, t);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = v[e] + t[e];
+        break;
+      case TRACEA_EPI_OP_RELU:
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = fmaxf(0.0f, v[e]);
+        break;
+      case TRACEA_EPI_OP_GELU:
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+          v[e] = 0.5f * v[e] * (1.0f + tanhf(0.79788456f * (v[e] + 0.044715f * v[e] * v[e] * v[e])));
+        break;
+      case TRACEA_EPI_OP_SILU:
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = v[e] / (1.0f + expf(-v[e]));
+        break;
+      case TRACEA_EPI_OP_RESIDUAL_ADD:
+        load_as_float<V>(op.p0, op.dtype, m * op.ld + n, nvalid, t);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = v[e] + t[e];
+        break;
+      case TRACEA_EPI_OP_BIAS_ADD_SILU:
+        load_as_float<V>(op.p0, op.dtype, n, nvalid, t);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          float x = v[e] + t[e];
+          v[e] = x / (1.0f + expf(-x));
+        }
+        break;
+      case TRACEA_EPI_OP_BATCHNORM: {
+        float b[V], mu[V], var[V];
+        load_as_float<V>(op.p0, DT_F32, n, nvalid, t);
+        load_as_float<V>(op.p1, DT_F32, n, nvalid, b);
+        load_as_float<V>(op.p2, DT_F32, n, nvalid, mu);
+        load_as_float<V>(op.p3, DT_F32, n, nvalid, var);
+#pragma unroll
+        for (int e = 0; e < V; ++e)
+          v[e] = (v[e] - mu[e]) * (1.0f / sqrtf(var[e] + op.epsilon)) * t[e] + b[e];
+      } break;
+      case TRACEA_EPI_OP_SCALE_SHIFT: {
+        float sh[V];
+        load_as_float<V>(op.p0, DT_F32, n, nvalid, t);
+        load_as_float<V>(op.p1, DT_F32, n, nvalid, sh);
+#pragma unroll
+        for (int e = 0; e < V; ++e) v[e] = v[e] * t[e] + sh[e];
+      } break;
+      default:
+        break;
+    }
+  }
+}
+
+// Converts V floats to the output type (round to nearest even) and stores
+// them at element index idx; only the first nvalid are written.
+template <int V>
+__device__ __forceinline__ void store_from_float(void *base, int dtype, long long idx, int nvalid,
+                                                 const float (&v)[V]) {
+  if (dtype == DT_F32) {
+    float *p = (float *)base + idx;
+    if (V > 1 && nvalid >= V && (((uintptr_t)p) & 15) == 0) {
+#pragma unroll
+      for (int q = 0; q < V / 4; ++q) {
+        f32x4 o = {v[q * 4], v[q * 4 + 1], v[q * 4 + 2], v[q * 4 + 3]};
+        ((f32x4 *)p)[q] = o;
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        if (e < nvalid) p[e] = v[e];
+    }
+  } else if (dtype == DT_F16) {
+    _Float16 *p = (_Float16 *)base + idx;
+    _Float16 h[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) h[e] = (_Float16)v[e];
+    if (V == 8 && nvalid >= 8 && (((uintptr_t)p) & 15) == 0) {
+      f16x8 o = {h[0], h[1], h[2], h[3], h[V > 4 ? 4 : 0], h[V > 5 ? 5 : 0], h[V > 6 ? 6 : 0], h[V > 7 ? 7 : 0]};
+      *(f16x8 *)p = o;
+    } else if (V == 4 && nvalid >= 4 && (((uintptr_t)p) & 7) == 0) {
+      f16x4 o = {h[0], h[1], h[2], h[3]};
+      *(f16x4 *)p = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        if (e < nvalid) p[e] = h[e];
+    }
+  } else {
+    __bf16 *p = (__bf16 *)base + idx;
+    __bf16 h[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) h[e] = (__bf16)v[e];
+    if (V == 8 && nvalid >= 8 && (((uintptr_t)p) & 15) == 0) {
+      bf16x8 o = {h[0], h[1], h[2], h[3], h[V > 4 ? 4 : 0], h[V > 5 ? 5 : 0], h[V > 6 ? 6 : 0], h[V > 7 ? 7 : 0]};
+      *(bf16x8 *)p = o;
+    } else if (V == 4 && nvalid >= 4 && (((uintptr_t)p) & 7) == 0) {
+      bf16x4 o = {h[0], h[1], h[2], h[3]};
+      *(bf16x4 *)p = o;
+    } else {
+#pragma unroll
+      for (int e = 0; e < V; ++e)
+        if (e < nvalid) p[e] = h[e];
+    }
+  }
+}
+
+// ---- tile order ---------------------------------------------------------------
+// Consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its
+// own L2.  The id is first regrouped so that one XCD receives a contiguous run
+// of tile indices, then the run is laid out in column-major groups of
+// `group_m` tile rows, which gives every XCD a compact rectangle of C and
+// therefore a small set of A and B panels to keep in its L2.
+__device__ __forceinline__ void tile_coordinates(const ContractionArgs &a, int &tile_m,
+                                                 int &tile_n) {
+  int bid = blockIdx.x;
+  const int total = a.grid_m * a.grid_n;
+  if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);
+  const int gsz = a.group_m * a.grid_n;
+  const int group = bid / gsz;
+  const int first = group * a.group_m;
+  const int rows = min(a.grid_m - first, a.group_m);
+  const int in_group = bid - group * gsz;
+  tile_m = first + in_group % rows;
+  tile_n = in_group / rows;
+}
+
+// ---- the kernel -----------------------------------------------------------------
+template <int DT, int BM, int BN, int BK, int WM, int WN, bool CONV, bool B_NCONTIG>
+__global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const ContractionArgs args) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int CH = BK / 8;       // 16-byte pieces per tile row
+  constexpr int ROW_BYTES = BK * 2;
+  constexpr int RP = (256 / ROW_BYTES) > 0 ? (256 / ROW_BYTES) : 1;  // rows per 256 B
+  constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
+  constexpr int A_STAGE = BM * ROW_BYTES, B_STAGE = BN * ROW_BYTES;
+  constexpr int STAGE = A_STAGE + B_STAGE;
+  constexpr int NA = BM * CH / NT;  // A pieces per thread per K tile
+  constexpr int NB = BN * CH / NT;  // B pieces per thread per K tile
+  static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tile must be 32-aligned");
+  static_assert((BM * CH) % NT == 0 && (BN * CH) % NT == 0, "pieces must divide over threads");
+  static_assert(NT % CH == 0 && BK % 16 == 0, "bad BK");
+  static_assert(!B_NCONTIG || (NT % (BN / 8) == 0), "bad BN for N-contiguous B");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave % WM, wn = wave / WM;
+
+  int tile_m, tile_n;
+  tile_coordinates(args, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int M = args.M, N = args.N, K = args.K;
+
+  // ---- per-thread source coordinates of the pieces this thread moves ----
+  const int pc = tid % CH;      // 16-byte column of every A piece of this thread
+  const int prow = tid / CH;    // first tile row; piece i is prow + i*(NT/CH)
+  constexpr int PR_STEP = NT / CH;
+
+  const unsigned short *Ag = (const unsigned short *)args.A;
+  const unsigned short *Bg = (const unsigned short *)args.B;
+
+  long long a_off[NA];              // GEMM: element offset of the row start (+ piece column)
+  int a_hb[CONV ? NA : 1], a_wb[CONV ? NA : 1];  // conv: ho*stride-pad, wo*stride-pad
+#pragma unroll
+  for (int i = 0; i < NA; ++i) {
+    int m = m0 + prow + i * PR_STEP;
+    m = m < M ? m : M - 1;
+    if constexpr (CONV) {
+      int bn, rem, ho, wo;
+      fast_divmod(m, args.hw_m, args.hw_s, args.h_out * args.w_out, bn, rem);
+      fast_divmod(rem, args.w_m, args.w_s, args.w_out, ho, wo);
+      a_off[i] = (long long)bn * args.h_in * args.w_in * args.c_in;
+      a_hb[i] = ho * args.stride_h - args.pad_h;
+      a_wb[i] = wo * args.stride_w - args.pad_w;
+    } else {
+      a_off[i] = (long long)m * args.lda;
+    }
+  }
+
+  long long b_off[NB];
+  if constexpr (!B_NCONTIG) {
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      int n = n0 + prow + i * PR_STEP;
+      n = n < N ? n : N - 1;
+      b_off[i] = (long long)n * args.ldb;
+    }
+  }
+  // N-contiguous B: piece q covers k row q / (BN/8), channels (q % (BN/8))*8..+7
+  constexpr int NCH = BN / 8;
+
+  u32x4 ra[NA], rb[NB];
+
+  // Every load is issued unconditionally from an address that is always
+  // inside the tensor (the real one, or the tensor base when the piece lies in
+  // padding or beyond K); pieces that must read as zero are recorded in a bit
+  // mask and cleared only when the registers are written to LDS, after the
+  // MFMAs of the current K tile.  No branch and no use of the loaded value
+  // separates the loads from those MFMAs, so their latency is hidden.
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  unsigned a_ok = 0, b_ok = 0;  // bit i: piece i holds real data
+  auto fetch = [&](int k0) {
+    const int kg = k0 + pc * 8;
+    const bool kvalid = kg < K;
+    const int k0c = kvalid ? kg : 0;  // column of this thread's piece, or a safe one
+    a_ok = 0;
+    b_ok = 0;
+    if constexpr (CONV) {
+      int rf, rem, sf, ci;
+      fast_divmod(kg, args.sc_m, args.sc_s, args.s_sz * args.c_in, rf, rem);
+      fast_divmod(rem, args.c_m, args.c_s, args.c_in, sf, ci);
+      const int dh = rf * args.dil_h, dw = sf * args.dil_w;
+#pragma unroll
+      for (int i = 0; i < NA; ++i) {
+        const int hi = a_hb[i] + dh, wi = a_wb[i] + dw;
+        const bool ok = kvalid && hi >= 0 && hi < args.h_in && wi >= 0 && wi < args.w_in;
+        const long long off = a_off[i] + ((long long)hi * args.w_in + wi) * args.c_in + ci;
+        ra[i] = *(const u32x4 *)(Ag + (ok ? off : 0ll));
+        a_ok |= ok ? (1u << i) : 0u;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NA; ++i) ra[i] = *(const u32x4 *)(Ag + a_off[i] + k0c);
+      a_ok = kvalid ? 0xffffffffu : 0u;
+    }
+    if constexpr (!B_NCONTIG) {
+#pragma unroll
+      for (int i = 0; i < NB; ++i) rb[i] = *(const u32x4 *)(Bg + b_off[i] + k0c);
+      b_ok = kvalid ? 0xffffffffu : 0u;
+    } else {
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        const int q = tid + i * NT;
+        const int kk = q / NCH, nch = q % NCH;
+        const int n = n0 + nch * 8;
+        const bool ok = k0 + kk < K && n < N;
+        rb[i] = *(const u32x4 *)(Bg + (ok ? (long long)(k0 + kk) * args.ldb + n : 0ll));
+        b_ok |= ok ? (1u << i) : 0u;
+      }
+    }
+  };
+
+  auto lds_piece = [&](int row, int c) -> int {
+    return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
+  };
+
+  // Zero-masking of pieces is needed for a convolution (padding) and whenever
+  // the last K tile is partial; a GEMM whose K is a multiple of BK skips it.
+  const bool mask_a = CONV || (K % BK) != 0;
+  const bool mask_b = B_NCONTIG || (K % BK) != 0;
+  auto stash = [&](unsigned char *sA, unsigned char *sB) {
+    if (mask_a) {
+#pragma unroll
+      for (int i = 0; i < NA; ++i)
+        *(u32x4 *)(sA + lds_piece(prow + i * PR_STEP, pc)) = ((a_ok >> i) & 1u) ? ra[i] : zero4;
+    } else {
+#pragma unroll
+      for (int i = 0; i < NA; ++i) *(u32x4 *)(sA + lds_piece(prow + i * PR_STEP, pc)) = ra[i];
+    }
+    if constexpr (!B_NCONTIG) {
+      if (mask_b) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i)
+          *(u32x4 *)(sB + lds_piece(prow + i * PR_STEP, pc)) = ((b_ok >> i) & 1u) ? rb[i] : zero4;
+      } else {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) *(u32x4 *)(sB + lds_piece(prow + i * PR_STEP, pc)) = rb[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        const int q = tid + i * NT;
+        const int kk = q / NCH, nch = q % NCH;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int row = nch * 8 + e;
+          const unsigned w = ((b_ok >> i) & 1u) ? rb[i][e >> 1] : 0u;
+          const unsigned short h = (e & 1) ? (unsigned short)(w >> 16) : (unsigned short)(w & 0xffffu);
+          *(unsigned short *)(sB + lds_piece(row, kk >> 3) + (kk & 7) * 2) = h;
+        }
+      }
+    }
+  };
+
+  f32x16 acc[FM][FN];
+#pragma unroll
+  for (int i = 0; i < FM; ++i)
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int lrow = lane & 31;
+  const int lhalf = lane >> 5;
+  const int lswz = (lrow / RP) & (CH - 1);  // wave tiles start on multiples of 32 rows
+
+  auto multiply = [&](const unsigned char *sA, const unsigned char *sB) {
+    const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
+    const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+      u32x4 af[FM], bf[FN];
+#pragma unroll
+      for (int i = 0; i < FM; ++i) af[i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) bf[j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(bf[j], af[i], acc[i][j]);
+    }
+  };
+
+  // ---- main loop: two LDS stages, register-staged prefetch ----
+  static_assert(NA <= 32 && NB <= 32, "piece masks are 32 bits");
+  const int nk = (K + BK - 1) / BK;
+  fetch(0);
+  stash(smem, smem + A_STAGE);
+  __syncthreads();
+  for (int kt = 0; kt + 1 < nk; ++kt) {
+    unsigned char *cur = smem + (kt & 1) * STAGE;
+    unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
+    // The scheduling fences keep the compiler from sinking the global loads
+    // below the MFMAs (towards their first use in stash), which would expose
+    // the whole memory latency once per K tile.
+    fetch((kt + 1) * BK);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(cur, cur + A_STAGE);
+    __builtin_amdgcn_sched_barrier(0);
+    stash(nxt, nxt + A_STAGE);
+    __syncthreads();
+  }
+  {
+    const unsigned char *cur = smem + ((nk - 1) & 1) * STAGE;
+    multiply(cur, cur + A_STAGE);
+  }
+  __syncthreads();
+
+  // ---- epilogue ----
+  // The MFMA leaves lane l with row (l&31) and channels 8g + 4*(l>>5) + 0..3 of
+  // each 32x32 block.  32 rows of the wave tile at a time are written to a
+  // wave-private fp32 staging area in LDS (free after the last barrier of the
+  // main loop) and read back 8 consecutive channels per lane, so that the
+  // operator chain runs on 8-vectors and a row leaves as whole 16-byte stores.
+  constexpr int EP_PITCH = TN + 4;                 // floats
+  constexpr int LPR = TN / 8;                      // lanes per output row
+  constexpr int RPI = 64 / LPR;                    // rows per pass
+  static_assert((size_t)WM * WN * 32 * EP_PITCH * 4 <= (size_t)2 * STAGE, "staging must fit");
+  float *stage = (float *)smem + wave * (32 * EP_PITCH);
+  const int er = lane / LPR, ec = (lane % LPR) * 8;
+#pragma unroll
+  for (int i = 0; i < FM; ++i) {
+#pragma unroll
+    for (int j = 0; j < FN; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
+                   acc[i][j][g * 4 + 3]};
+        *(f32x4 *)(stage + lrow * EP_PITCH + j * 32 + g * 8 + lhalf * 4) = v;
+      }
+    __syncthreads();
+    for (int r = er; r < 32; r += RPI) {
+      const int m = m0 + wm * TM + i * 32 + r;
+      const int n = n0 + wn * TN + ec;
+      if (m < M && n < N) {
+        float v[8];
+        const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
+        const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] = lo[e];
+          v[4 + e] = hi[e];
+        }
+        const int nvalid = N - n;
+        apply_epilogue<8>(v, m, n, nvalid, args.epi);
+        store_from_float<8>(args.C, args.out_dtype, (long long)m * args.ldc + n, nvalid, v);
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <int BM, int BN, int BK, int WM, int WN>
+int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
+                       hipStream_t stream) {
+  constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * 2;
+  const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(WM * WN * 64);
+#define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
+  do {                                                                                       \
+    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, CONVV, NCV>;                      \
+    static bool attr_done = false;                                                           \
+    if (!attr_done) {                                                                        \
+      hipError_t e = hipFuncSetAttribute((const void *)kfn,                                  \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return (int)e;                                                    \
+      attr_done = true;                                                                      \
+    }                                                                                        \
+    hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                    \
+    return (int)hipGetLastError();                                                           \
+  } while (0)
+  if (dtype == DT_F16) {
+    if (conv) { if (b_ncontig) TRACEA_LAUNCH(DT_F16, true, true); else TRACEA_LAUNCH(DT_F16, true, false); }
+    else      { if (b_ncontig) TRACEA_LAUNCH(DT_F16, false, true); else TRACEA_LAUNCH(DT_F16, false, false); }
+  } else {
+    if (conv) { if (b_ncontig) TRACEA_LAUNCH(DT_BF16, true, true); else TRACEA_LAUNCH(DT_BF16, true, false); }
+    else      { if (b_ncontig) TRACEA_LAUNCH(DT_BF16, false, true); else TRACEA_LAUNCH(DT_BF16, false, false); }
+  }
+#undef TRACEA_LAUNCH
+  return (int)hipErrorInvalidValue;
+}
+
+}  // namespace tracea_amd

@@ -1,0 +1,20 @@
+// One member of the contraction kernel family per translation unit; the build
+// compiles this file once per line of contraction_variants.def with
+// -DV_NAME=... -DV_BM=... -DV_BN=... -DV_BK=... -DV_WM=... -DV_WN=... -DV_STAGES=... -DV_DIRECT=...
+#include "contraction_kernel.hpp"
+
+#define TRACEA_CAT2(a, b) a##b
+#define TRACEA_CAT(a, b) TRACEA_CAT2(a, b)
+#define TRACEA_STR2(a) #a
+#define TRACEA_STR(a) TRACEA_STR2(a)
+
+namespace tracea_amd {
+// Host-side accessor (a function, so that nothing here is emitted for the device).
+const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
+  static const ContractionVariant v = {
+      TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT != 0,
+      (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
+      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN>};
+  return v;
+}
+}  // namespace tracea_amd

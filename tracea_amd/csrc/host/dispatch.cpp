@@ -1,0 +1,675 @@
+// Argument checking and kernel dispatch for tracea_gemm / tracea_conv2d /
+// tracea_attention.  Validation order and status codes follow the reference's
+// FFI layer (tracea-ffi/src/lib.rs:151-181; src/interface/c_bindings.rs:206-495):
+// runtime not initialised -> UNKNOWN_ERROR; NULL pointers and wrong ranks ->
+// INVALID_PARAMS; groups/dtype/layout the kernels do not cover ->
+// UNSUPPORTED_CONFIG; host pointers -> CPU_ERROR; HIP failures -> CUDA_ERROR.
+#include "dispatch.hpp"
+
+#include <atomic>
+#include <cmath>
+#include <cstring>
+#include <mutex>
+
+#include "tuning_cache.hpp"
+
+namespace tracea_amd {
+
+namespace {
+
+struct View {
+  void *ptr = nullptr;
+  int rank = 0;
+  long long shape[4] = {0, 0, 0, 0};
+  long long stride[4] = {0, 0, 0, 0};
+  int dtype = 0;
+  int device = -1;
+};
+
+// Copies a TraceaTensorView; a NULL stride array means contiguous row-major.
+TraceaStatus read_view(const char *what, const TraceaTensorView &t, int want_rank, View *v) {
+  if (t.ptr == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: data pointer is NULL", what);
+  if (t.shape == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: shape pointer is NULL", what);
+  if ((int)t.rank != want_rank)
+    return fail(TRACEA_INVALID_PARAMS, "%s: expected rank %d, got %u", what, want_rank, t.rank);
+  v->ptr = t.ptr;
+  v->rank = (int)t.rank;
+  for (int i = 0; i < want_rank; ++i) v->shape[i] = (long long)t.shape[i];
+  if (t.stride != nullptr) {
+    for (int i = 0; i < want_rank; ++i) v->stride[i] = (long long)t.stride[i];
+  } else {
+    long long s = 1;
+    for (int i = want_rank - 1; i >= 0; --i) {
+      v->stride[i] = s;
+      s *= v->shape[i];
+    }
+  }
+  v->dtype = (int)t.dtype;
+  v->device = t.device_id;
+  return TRACEA_SUCCESS;
+}
+
+bool is_half(int dt) { return dt == TRACEA_DTYPE_FLOAT16 || dt == TRACEA_DTYPE_BFLOAT16; }
+bool is_float_type(int dt) { return dt == TRACEA_DTYPE_FLOAT32 || is_half(dt); }
+int elem_size(int dt) { return dt == TRACEA_DTYPE_FLOAT32 ? 4 : 2; }
+bool aligned(const void *p, size_t a) { return (((uintptr_t)p) & (a - 1)) == 0; }
+
+const char *dtype_name(int dt) {
+  switch (dt) {
+    case TRACEA_DTYPE_FLOAT32: return "f32";
+    case TRACEA_DTYPE_FLOAT16: return "f16";
+    case TRACEA_DTYPE_BFLOAT16: return "bf16";
+    case TRACEA_DTYPE_INT32: return "i32";
+    case TRACEA_DTYPE_INT8: return "i8";
+    default: return "?";
+  }
+}
+
+TraceaStatus check_device(const char *what, int device) {
+  if (device < 0)
+    return fail(TRACEA_CPU_ERROR,
+                "%s: host memory (device_id -1) is not supported; this library has no CPU arm",
+                what);
+  if (device >= runtime_device_count())
+    return fail(TRACEA_INVALID_PARAMS, "%s: device_id %d out of range (%d devices)", what, device,
+                runtime_device_count());
+  return TRACEA_SUCCESS;
+}
+
+// Makes `device` current for the lifetime of the object.
+struct DeviceScope {
+  int prev = -1;
+  bool switched = false;
+  hipError_t err = hipSuccess;
+  explicit DeviceScope(int device) {
+    err = hipGetDevice(&prev);
+    if (err == hipSuccess && prev != device) {
+      err = hipSetDevice(device);
+      switched = err == hipSuccess;
+    }
+  }
+  ~DeviceScope() {
+    if (switched) (void)hipSetDevice(prev);
+  }
+};
+
+// ---- epilogue chains ---------------------------------------------------------
+
+// TraceaEpilogueKind -> operator list, as src/interface/c_bindings.rs:144-197:
+// an operator whose tensor is absent is dropped, not an error.
+int kind_to_ops(int kind, const TraceaTensorView *bias, const TraceaTensorView *residual,
+                TraceaEpilogueOp *ops) {
+  int n = 0;
+  auto bias_op = [&](TraceaEpilogueOpKind k) {
+    if (bias == nullptr) return;
+    ops[n] = TraceaEpilogueOp{k, bias->dtype, bias->ptr, nullptr, nullptr, nullptr, 0.0f, 0};
+    ++n;
+  };
+  auto res_op = [&]() {
+    if (residual == nullptr) return;
+    ops[n] = TraceaEpilogueOp{TRACEA_EPI_OP_RESIDUAL_ADD, residual->dtype, residual->ptr, nullptr,
+                              nullptr, nullptr, 0.0f, -1 /* resolved from the view */};
+    ++n;
+  };
+  auto plain = [&](TraceaEpilogueOpKind k) {
+    ops[n] = TraceaEpilogueOp{k, TRACEA_DTYPE_FLOAT32, nullptr, nullptr, nullptr, nullptr, 0.0f, 0};
+    ++n;
+  };
+  switch (kind) {
+    case TRACEA_EPILOGUE_IDENTITY: break;
+    case TRACEA_EPILOGUE_BIAS_ADD: bias_op(TRACEA_EPI_OP_BIAS_ADD); break;
+    case TRACEA_EPILOGUE_RELU: plain(TRACEA_EPI_OP_RELU); break;
+    case TRACEA_EPILOGUE_GELU: plain(TRACEA_EPI_OP_GELU); break;
+    case TRACEA_EPILOGUE_SILU: plain(TRACEA_EPI_OP_SILU); break;
+    case TRACEA_EPILOGUE_BIAS_RELU: bias_op(TRACEA_EPI_OP_BIAS_ADD); plain(TRACEA_EPI_OP_RELU); break;
+    case TRACEA_EPILOGUE_BIAS_SILU: bias_op(TRACEA_EPI_OP_BIAS_ADD_SILU); break;
+    case TRACEA_EPILOGUE_RESIDUAL: res_op(); break;
+    case TRACEA_EPILOGUE_RESIDUAL_RELU: res_op(); plain(TRACEA_EPI_OP_RELU); break;
+    default: return -1;
+  }
+  return n;
+}
+
+// Validates a caller-supplied chain and lowers it to device form.  `rows` and
+// `channels` are the GEMM view of the output; res_ld_default is the row stride
+// assumed for a residual whose ld is 0.
+TraceaStatus lower_chain(const char *what, const TraceaEpilogueOp *ops, uint32_t n_ops,
+                         long long channels, long long res_ld_default, EpilogueChain *chain) {
+  if (n_ops > TRACEA_MAX_EPILOGUE_OPS)
+    return fail(TRACEA_INVALID_PARAMS, "%s: %u epilogue operators, at most %d are supported", what,
+                n_ops, TRACEA_MAX_EPILOGUE_OPS);
+  if (n_ops > 0 && ops == nullptr)
+    return fail(TRACEA_INVALID_PARAMS, "%s: epilogue operator list is NULL", what);
+  chain->n_ops = 0;
+  for (uint32_t i = 0; i < n_ops; ++i) {
+    const TraceaEpilogueOp &op = ops[i];
+    EpilogueOpDev d{};
+    d.kind = (int)op.kind;
+    d.dtype = DT_F32;
+    d.epsilon = op.epsilon;
+    d.ld = 0;
+    switch (op.kind) {
+      case TRACEA_EPI_OP_NONE: continue;
+      case TRACEA_EPI_OP_RELU:
+      case TRACEA_EPI_OP_GELU:
+      case TRACEA_EPI_OP_SILU: break;
+      case TRACEA_EPI_OP_BIAS_ADD:
+      case TRACEA_EPI_OP_BIAS_ADD_SILU:
+      case TRACEA_EPI_OP_RESIDUAL_ADD:
+        if (op.p0 == nullptr)
+          return fail(TRACEA_INVALID_PARAMS, "%s: epilogue operator %u has a NULL tensor", what, i);
+        if (!is_float_type(op.dtype))
+          return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: epilogue operator %u: dtype %s unsupported",
+                      what, i, dtype_name(op.dtype));
+        d.dtype = op.dtype;
+        d.p0 = op.p0;
+        if (op.kind == TRACEA_EPI_OP_RESIDUAL_ADD) d.ld = op.ld > 0 ? op.ld : res_ld_default;
+        break;
+      case TRACEA_EPI_OP_BATCHNORM:
+        if (!op.p0 || !op.p1 || !op.p2 || !op.p3)
+          return fail(TRACEA_INVALID_PARAMS, "%s: BatchNorm needs gamma, beta, mean and var", what);
+        d.p0 = op.p0; d.p1 = op.p1; d.p2 = op.p2; d.p3 = op.p3;
+        break;
+      case TRACEA_EPI_OP_SCALE_SHIFT:
+        if (!op.p0 || !op.p1)
+          return fail(TRACEA_INVALID_PARAMS, "%s: ScaleShift needs scale and shift", what);
+        d.p0 = op.p0; d.p1 = op.p1;
+        break;
+      default:
+        return fail(TRACEA_INVALID_PARAMS, "%s: unknown epilogue operator kind %d", what,
+                    (int)op.kind);
+    }
+    chain->ops[chain->n_ops++] = d;
+  }
+  (void)channels;
+  return TRACEA_SUCCESS;
+}
+
+// Checks the optional bias / residual views of the TraceaEpilogueKind calls
+// against the output geometry and fills the residual row stride.
+TraceaStatus check_bias_residual(const char *what, const TraceaTensorView *bias,
+                                 const TraceaTensorView *residual, long long channels,
+                                 const View &out_view, int device, TraceaEpilogueOp *ops, int n) {
+  if (bias != nullptr) {
+    if (bias->ptr == nullptr || bias->shape == nullptr)
+      return fail(TRACEA_INVALID_PARAMS, "%s: bias view has a NULL pointer", what);
+    if (bias->rank != 1 || (long long)bias->shape[0] != channels)
+      return fail(TRACEA_INVALID_PARAMS, "%s: bias must have shape [%lld]", what, channels);
+    if (bias->stride != nullptr && bias->stride[0] != 1)
+      return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: bias must be contiguous", what);
+    if (!is_float_type(bias->dtype))
+      return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: bias dtype %s unsupported", what,
+                  dtype_name(bias->dtype));
+    if (bias->device_id != device)
+      return fail(TRACEA_INVALID_PARAMS, "%s: bias lives on device %d, output on %d", what,
+                  bias->device_id, device);
+  }
+  if (residual != nullptr) {
+    View r;
+    TraceaStatus st = read_view("residual", *residual, out_view.rank, &r);
+    if (st != TRACEA_SUCCESS) return st;
+    for (int i = 0; i < r.rank; ++i)
+      if (r.shape[i] != out_view.shape[i])
+        return fail(TRACEA_INVALID_PARAMS, "%s: residual shape differs from the output shape", what);
+    if (!is_float_type(r.dtype))
+      return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: residual dtype %s unsupported", what,
+                  dtype_name(r.dtype));
+    if (r.device != device)
+      return fail(TRACEA_INVALID_PARAMS, "%s: residual lives on device %d, output on %d", what,
+                  r.device, device);
+    // channel-contiguous rows with one row stride across all leading dims
+    const int last = r.rank - 1;
+    if (r.stride[last] != 1)
+      return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: residual channels must be contiguous", what);
+    const long long ld = r.rank >= 2 ? r.stride[last - 1] : channels;
+    long long expect = ld;
+    for (int i = last - 1; i >= 0; --i) {
+      if (r.stride[i] != expect)
+        return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: residual must be densely strided over rows", what);
+      expect *= r.shape[i];
+    }
+    for (int i = 0; i < n; ++i)
+      if (ops[i].kind == TRACEA_EPI_OP_RESIDUAL_ADD && ops[i].ld < 0) ops[i].ld = ld;
+  }
+  return TRACEA_SUCCESS;
+}
+
+std::atomic<int> g_forced_contraction{-1};
+std::atomic<int> g_forced_conv{-1};
+std::atomic<int> g_forced_attention{-1};
+
+TraceaStatus hip_status(const char *what, int e) {
+  if (e == 0) return TRACEA_SUCCESS;
+  return fail(TRACEA_CUDA_ERROR, "%s: %s", what, hipGetErrorString((hipError_t)e));
+}
+
+}  // namespace
+
+void set_forced_variant(const char *op, int index) {
+  if (!strcmp(op, "gemm")) g_forced_contraction.store(index);
+  else if (!strcmp(op, "conv2d")) g_forced_conv.store(index);
+  else if (!strcmp(op, "attention")) g_forced_attention.store(index);
+}
+int forced_variant(const char *op) {
+  if (!strcmp(op, "gemm")) return g_forced_contraction.load();
+  if (!strcmp(op, "conv2d")) return g_forced_conv.load();
+  if (!strcmp(op, "attention")) return g_forced_attention.load();
+  return -1;
+}
+
+// ---- reciprocals ---------------------------------------------------------------
+// The reference's magic_u32 (src/emitter/cuda/conv.rs:6-16) always ends at
+// p = 32, i.e. magic = ceil(2^32/d) with no extra shift, which is exact only
+// while n*d < 2^32.  That pair is kept whenever it is exact for the largest
+// dividend (so the packed block equals the reference's bit for bit); beyond
+// it the shift floor(log2 d) is used, which is exact for every n < 2^31.
+void magic_for_divisor(uint32_t d, uint64_t n_max, uint32_t *magic, uint32_t *shift) {
+  *magic = 0;
+  *shift = 0;
+  if (d <= 1) return;
+  if ((d & (d - 1)) == 0) {
+    *shift = (uint32_t)__builtin_ctz(d);
+    return;
+  }
+  if (n_max * (uint64_t)d < (1ull << 32)) {
+    *magic = (uint32_t)(((1ull << 32) + d - 1) / d);
+    return;
+  }
+  const uint32_t s = 31u - (uint32_t)__builtin_clz(d);
+  *magic = (uint32_t)((((unsigned __int128)1 << (32 + s)) + d - 1) / d);
+  *shift = s;
+}
+
+TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s, int stride_h,
+                                int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                                ConvGeometry *out) {
+  if (n <= 0 || h <= 0 || w <= 0 || c <= 0 || k <= 0 || r <= 0 || s <= 0)
+    return fail(TRACEA_INVALID_PARAMS, "conv2d: every dimension must be positive");
+  if (stride_h <= 0 || stride_w <= 0 || dil_h <= 0 || dil_w <= 0 || pad_h < 0 || pad_w < 0)
+    return fail(TRACEA_INVALID_PARAMS, "conv2d: stride and dilation must be >= 1, padding >= 0");
+  const long long ho = ((long long)h + 2 * pad_h - (long long)dil_h * (r - 1) - 1) / stride_h + 1;
+  const long long wo = ((long long)w + 2 * pad_w - (long long)dil_w * (s - 1) - 1) / stride_w + 1;
+  if ((long long)h + 2 * pad_h < (long long)dil_h * (r - 1) + 1 ||
+      (long long)w + 2 * pad_w < (long long)dil_w * (s - 1) + 1 || ho <= 0 || wo <= 0)
+    return fail(TRACEA_INVALID_PARAMS, "conv2d: filter larger than the padded input");
+  const long long m_gemm = (long long)n * ho * wo, k_gemm = (long long)r * s * c;
+  if (m_gemm >= (1ll << 31) || k_gemm >= (1ll << 31) || (long long)n * h * w * c >= (1ll << 40))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "conv2d: problem too large for 32-bit row indices");
+  TraceaConvParamsBlock &b = out->block;
+  b.batch = n; b.h_in = h; b.w_in = w; b.c_in = c; b.k_out = k;
+  b.h_out = (int)ho; b.w_out = (int)wo; b.r_sz = r; b.s_sz = s;
+  b.stride = stride_h; b.pad = pad_h; b.dilation = dil_h;
+  magic_for_divisor((uint32_t)(ho * wo), (uint64_t)m_gemm, &b.hw_m, &b.hw_s);
+  magic_for_divisor((uint32_t)wo, (uint64_t)(ho * wo), &b.w_m, &b.w_s);
+  magic_for_divisor((uint32_t)(s * c), (uint64_t)k_gemm + 1024, &b.sic_m, &b.sic_s);
+  magic_for_divisor((uint32_t)c, (uint64_t)s * c, &b.c_m, &b.c_s);
+  out->stride_h = stride_h; out->stride_w = stride_w;
+  out->pad_h = pad_h; out->pad_w = pad_w;
+  out->dil_h = dil_h; out->dil_w = dil_w;
+  out->m_gemm = (int)m_gemm; out->n_gemm = k; out->k_gemm = (int)k_gemm;
+  return TRACEA_SUCCESS;
+}
+
+// ---- variant choice --------------------------------------------------------------
+// Score = useful fraction of the padded tile grid x fraction of the last wave
+// of workgroups that is occupied x a per-shape efficiency prior (larger tiles
+// re-use more of each LDS fetch).  A tuning-cache entry, when present, wins.
+int select_contraction_variant(int m, int n, int k, bool conv) {
+  (void)k;
+  (void)conv;
+  const int cus = 256;
+  int best = -1;
+  double best_score = -1.0;
+  for (int i = 0; i < contraction_variant_count(); ++i) {
+    const ContractionVariant &v = contraction_variant(i);
+    const long long gm = (m + v.bm - 1) / v.bm, gn = (n + v.bn - 1) / v.bn;
+    const double useful = ((double)m * n) / ((double)gm * v.bm * gn * v.bn);
+    const long long tiles = gm * gn;
+    // workgroups resident per CU: bounded by LDS (160 KB) and by 8 waves per CU here
+    const int per_cu_lds = (int)(160 * 1024 / v.lds_bytes);
+    const int per_cu_waves = 8 / (v.waves_m * v.waves_n) > 0 ? 8 / (v.waves_m * v.waves_n) : 1;
+    const int per_cu = per_cu_lds < per_cu_waves ? (per_cu_lds > 0 ? per_cu_lds : 1) : per_cu_waves;
+    const long long slots = (long long)cus * per_cu;
+    const long long rounds = (tiles + slots - 1) / slots;
+    const double quant = (double)tiles / (double)(rounds * slots);
+    const double reuse = (double)(v.bm * v.bn) / (double)(v.bm + v.bn) / 128.0;
+    const double prior = reuse > 1.0 ? 1.0 : reuse;
+    const double score = useful * (0.35 + 0.65 * quant) * (0.3 + 0.7 * prior);
+    if (score > best_score) {
+      best_score = score;
+      best = i;
+    }
+  }
+  return best;
+}
+
+namespace {
+
+int pick_contraction(const char *op, const std::string &cache_key, int m, int n, int k, bool conv) {
+  const int forced = forced_variant(op);
+  if (forced >= 0) return forced;
+  int cached = tuning_cache_lookup_variant(cache_key);
+  if (cached >= 0) return cached;
+  return select_contraction_variant(m, n, k, conv);
+}
+
+void fill_grid(ContractionArgs *a, const ContractionVariant &v) {
+  a->grid_m = (a->M + v.bm - 1) / v.bm;
+  a->grid_n = (a->N + v.bn - 1) / v.bn;
+  // 8 XCDs each take total/8 consecutive tiles; a group height of 4 (256-row
+  // tiles) or 8 (smaller) keeps an XCD's run inside a near-square patch.
+  a->group_m = v.bm >= 256 ? 4 : 8;
+  if (a->group_m > a->grid_m) a->group_m = a->grid_m;
+}
+
+// ---- GEMM ----------------------------------------------------------------------
+TraceaStatus run_gemm(const View &a, const View &b, const View &c, const EpilogueChain &chain,
+                      hipStream_t stream) {
+  const long long M = a.shape[0], K = a.shape[1], N = b.shape[1];
+  if (M == 0 || N == 0) return TRACEA_SUCCESS;
+  DeviceScope scope(c.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+
+  if (is_half(a.dtype) && K > 0) {
+    const bool a_ok = a.stride[1] == 1 && a.stride[0] % 8 == 0 && K % 8 == 0 && aligned(a.ptr, 16);
+    const bool b_kcontig = b.stride[0] == 1 && b.stride[1] % 8 == 0 && aligned(b.ptr, 16);
+    const bool b_ncontig = b.stride[1] == 1 && b.stride[0] % 8 == 0 && N % 8 == 0 && aligned(b.ptr, 16);
+    const bool c_ok = c.stride[1] == 1;
+    if (a_ok && (b_kcontig || b_ncontig) && c_ok) {
+      ContractionArgs args{};
+      args.A = a.ptr; args.B = b.ptr; args.C = c.ptr;
+      args.M = (int)M; args.N = (int)N; args.K = (int)K;
+      args.lda = a.stride[0];
+      args.ldb = b_kcontig ? b.stride[1] : b.stride[0];
+      args.ldc = c.stride[0];
+      args.out_dtype = c.dtype;
+      args.epi = chain;
+      char key[160];
+      snprintf(key, sizeof(key), "gemm_%lld_%lld_%lld_%s", M, N, K, tuning_device_name());
+      const int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false);
+      if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "gemm: no kernel variant available");
+      const ContractionVariant &v = contraction_variant(vi);
+      fill_grid(&args, v);
+      return hip_status("gemm launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
+    }
+  }
+  if (a.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32 && K > 0 &&
+      a.stride[1] == 1 && b.stride[1] == 1 && c.stride[1] == 1 && K % 4 == 0 && N % 4 == 0 &&
+      a.stride[0] % 4 == 0 && b.stride[0] % 4 == 0 && aligned(a.ptr, 16) && aligned(b.ptr, 16)) {
+    ContractionArgs args{};
+    args.A = a.ptr; args.B = b.ptr; args.C = c.ptr;
+    args.M = (int)M; args.N = (int)N; args.K = (int)K;
+    args.lda = a.stride[0]; args.ldb = b.stride[0]; args.ldc = c.stride[0];
+    args.out_dtype = DT_F32;
+    args.epi = chain;
+    return hip_status("gemm_f32 launch", launch_gemm_f32(args, stream));
+  }
+  GenericGemmArgs g{};
+  g.A = a.ptr; g.B = b.ptr; g.C = c.ptr;
+  g.M = (int)M; g.N = (int)N; g.K = (int)K;
+  g.sam = a.stride[0]; g.sak = a.stride[1];
+  g.sbk = b.stride[0]; g.sbn = b.stride[1];
+  g.scm = c.stride[0]; g.scn = c.stride[1];
+  g.a_dtype = a.dtype; g.b_dtype = b.dtype; g.c_dtype = c.dtype;
+  g.epi = chain;
+  return hip_status("gemm_generic launch", launch_gemm_generic(g, stream));
+}
+
+TraceaStatus gemm_common(const TraceaTensorView &ta, const TraceaTensorView &tb,
+                         TraceaTensorView *tc, View *a, View *b, View *c) {
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "tracea_gemm: tracea_init has not been called");
+  if (tc == nullptr) return fail(TRACEA_INVALID_PARAMS, "tracea_gemm: output view is NULL");
+  TraceaStatus st;
+  if ((st = read_view("tracea_gemm: a", ta, 2, a)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_gemm: b", tb, 2, b)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_gemm: c", *tc, 2, c)) != TRACEA_SUCCESS) return st;
+  if (!is_float_type(a->dtype) || !is_float_type(b->dtype) || !is_float_type(c->dtype))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_gemm: dtypes %s x %s -> %s unsupported",
+                dtype_name(a->dtype), dtype_name(b->dtype), dtype_name(c->dtype));
+  if (a->shape[1] != b->shape[0] || c->shape[0] != a->shape[0] || c->shape[1] != b->shape[1])
+    return fail(TRACEA_INVALID_PARAMS,
+                "tracea_gemm: shapes a[%lld,%lld] b[%lld,%lld] c[%lld,%lld] do not agree",
+                a->shape[0], a->shape[1], b->shape[0], b->shape[1], c->shape[0], c->shape[1]);
+  if ((st = check_device("tracea_gemm", c->device)) != TRACEA_SUCCESS) return st;
+  if (a->device != c->device || b->device != c->device)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_gemm: operands live on different devices");
+  if (a->shape[0] >= (1ll << 31) || a->shape[1] >= (1ll << 31) || b->shape[1] >= (1ll << 31))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_gemm: dimension exceeds 2^31-1");
+  return TRACEA_SUCCESS;
+}
+
+}  // namespace
+
+TraceaStatus dispatch_gemm_kind(const TraceaTensorView &ta, const TraceaTensorView &tb,
+                                const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                TraceaTensorView *tc, const TraceaGemmParams &params) {
+  View a, b, c;
+  TraceaStatus st = gemm_common(ta, tb, tc, &a, &b, &c);
+  if (st != TRACEA_SUCCESS) return st;
+  TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
+  const int n = kind_to_ops((int)params.epilogue, bias, residual, ops);
+  if (n < 0) return fail(TRACEA_INVALID_PARAMS, "tracea_gemm: unknown epilogue kind %d", (int)params.epilogue);
+  st = check_bias_residual("tracea_gemm", bias, residual, c.shape[1], c, c.device, ops, n);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain("tracea_gemm", ops, (uint32_t)n, c.shape[1], c.shape[1], &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  return run_gemm(a, b, c, chain, (hipStream_t)params.stream);
+}
+
+TraceaStatus dispatch_gemm_ops(const TraceaTensorView &ta, const TraceaTensorView &tb,
+                               TraceaTensorView *tc, const TraceaGemmParams &params,
+                               const TraceaEpilogueOp *ops, uint32_t n_ops) {
+  View a, b, c;
+  TraceaStatus st = gemm_common(ta, tb, tc, &a, &b, &c);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain("tracea_gemm_ex", ops, n_ops, c.shape[1], c.shape[1], &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  return run_gemm(a, b, c, chain, (hipStream_t)params.stream);
+}
+
+// ---- Conv2d ----------------------------------------------------------------------
+namespace {
+
+struct ConvPlan {
+  View x, w, out;
+  ConvGeometry geo;
+  bool w_ncontig;  // filters stored [R,S,C,K]
+  long long ldb, ldc;
+};
+
+TraceaStatus conv_common(const TraceaTensorView &tx, const TraceaTensorView &tw,
+                         TraceaTensorView *tout, const TraceaConv2dParams &p, ConvPlan *plan) {
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "tracea_conv2d: tracea_init has not been called");
+  if (tout == nullptr) return fail(TRACEA_INVALID_PARAMS, "tracea_conv2d: output view is NULL");
+  if (tx.ptr == nullptr || tw.ptr == nullptr || tout->ptr == nullptr)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_conv2d: NULL data pointer");
+  if (p.groups != 1)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: groups=%u (only groups=1)", p.groups);
+  TraceaStatus st;
+  View &x = plan->x, &w = plan->w, &out = plan->out;
+  if ((st = read_view("tracea_conv2d: x", tx, 4, &x)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_conv2d: w", tw, 4, &w)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_conv2d: out", *tout, 4, &out)) != TRACEA_SUCCESS) return st;
+  if (!is_half(x.dtype) || w.dtype != x.dtype)
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_conv2d: activations %s / filters %s; f16 or bf16 (both alike) required",
+                dtype_name(x.dtype), dtype_name(w.dtype));
+  if (out.dtype != x.dtype && out.dtype != TRACEA_DTYPE_FLOAT32)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: output dtype %s unsupported",
+                dtype_name(out.dtype));
+  if ((st = check_device("tracea_conv2d", out.device)) != TRACEA_SUCCESS) return st;
+  if (x.device != out.device || w.device != out.device)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_conv2d: operands live on different devices");
+  const long long N = x.shape[0], H = x.shape[1], W = x.shape[2], C = x.shape[3];
+  const long long K = w.shape[0], R = w.shape[1], S = w.shape[2];
+  if (w.shape[3] != C)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_conv2d: x has %lld channels, w expects %lld", C, w.shape[3]);
+  if (N >= (1ll << 31) || H >= (1ll << 31) || W >= (1ll << 31) || C >= (1ll << 31) || K >= (1ll << 31))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: dimension exceeds 2^31-1");
+  st = make_conv_geometry((int)N, (int)H, (int)W, (int)C, (int)K, (int)R, (int)S, (int)p.stride_h,
+                          (int)p.stride_w, (int)p.padding_h, (int)p.padding_w, (int)p.dilation_h,
+                          (int)p.dilation_w, &plan->geo);
+  if (st != TRACEA_SUCCESS) return st;
+  const ConvGeometry &g = plan->geo;
+  if (out.shape[0] != N || out.shape[1] != g.block.h_out || out.shape[2] != g.block.w_out || out.shape[3] != K)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_conv2d: output shape must be [%lld,%d,%d,%lld]", N,
+                g.block.h_out, g.block.w_out, K);
+  // layouts
+  if (!(x.stride[3] == 1 && x.stride[2] == C && x.stride[1] == W * C && x.stride[0] == H * W * C))
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_conv2d: activations must be contiguous NHWC (shape [N,H,W,C])");
+  if (w.stride[3] == 1 && w.stride[2] == C && w.stride[1] == S * C && w.stride[0] == R * S * C) {
+    plan->w_ncontig = false;
+    plan->ldb = R * S * C;
+  } else if (w.stride[0] == 1 && w.stride[3] == K && w.stride[2] == C * K && w.stride[1] == S * C * K) {
+    plan->w_ncontig = true;
+    plan->ldb = K;
+  } else {
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_conv2d: filters must be stored [K,R,S,C] or [R,S,C,K] (dims always [K,R,S,C])");
+  }
+  const long long ldc = out.stride[2];
+  if (!(out.stride[3] == 1 && ldc >= K && out.stride[1] == g.block.w_out * ldc &&
+        out.stride[0] == (long long)g.block.h_out * g.block.w_out * ldc))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: output must be channel-contiguous NHWK");
+  plan->ldc = ldc;
+  if (C % 8 != 0)
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_conv2d: input channels (%lld) must be a multiple of 8 for 16-byte loads", C);
+  if (plan->w_ncontig && K % 8 != 0)
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_conv2d: [R,S,C,K] filters need output channels (%lld) to be a multiple of 8", K);
+  if (!aligned(x.ptr, 16) || !aligned(w.ptr, 16))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: x and w must be 16-byte aligned");
+  return TRACEA_SUCCESS;
+}
+
+TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStream_t stream) {
+  const ConvGeometry &g = plan.geo;
+  DeviceScope scope(plan.out.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  ContractionArgs a{};
+  a.A = plan.x.ptr; a.B = plan.w.ptr; a.C = plan.out.ptr;
+  a.M = g.m_gemm; a.N = g.n_gemm; a.K = g.k_gemm;
+  a.lda = 0; a.ldb = plan.ldb; a.ldc = plan.ldc;
+  a.out_dtype = plan.out.dtype;
+  a.h_in = g.block.h_in; a.w_in = g.block.w_in; a.c_in = g.block.c_in;
+  a.h_out = g.block.h_out; a.w_out = g.block.w_out; a.s_sz = g.block.s_sz;
+  a.stride_h = g.stride_h; a.stride_w = g.stride_w;
+  a.pad_h = g.pad_h; a.pad_w = g.pad_w; a.dil_h = g.dil_h; a.dil_w = g.dil_w;
+  a.hw_m = g.block.hw_m; a.hw_s = g.block.hw_s; a.w_m = g.block.w_m; a.w_s = g.block.w_s;
+  a.sc_m = g.block.sic_m; a.sc_s = g.block.sic_s; a.c_m = g.block.c_m; a.c_s = g.block.c_s;
+  a.epi = chain;
+  char key[200];
+  snprintf(key, sizeof(key), "conv_%d_%d_%d_%d_%d_%d_%d_%d_%d_%s", g.block.batch, g.block.h_in,
+           g.block.w_in, g.block.c_in, g.block.k_out, g.block.r_sz, g.block.s_sz, g.stride_h,
+           g.pad_h, tuning_device_name());
+  const int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
+  if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
+  const ContractionVariant &v = contraction_variant(vi);
+  fill_grid(&a, v);
+  return hip_status("conv2d launch", v.launch(a, true, plan.x.dtype, plan.w_ncontig, stream));
+}
+
+}  // namespace
+
+TraceaStatus dispatch_conv2d_kind(const TraceaTensorView &tx, const TraceaTensorView &tw,
+                                  const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                  TraceaTensorView *tout, const TraceaConv2dParams &params) {
+  ConvPlan plan;
+  TraceaStatus st = conv_common(tx, tw, tout, params, &plan);
+  if (st != TRACEA_SUCCESS) return st;
+  TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
+  const int n = kind_to_ops((int)params.epilogue, bias, residual, ops);
+  if (n < 0) return fail(TRACEA_INVALID_PARAMS, "tracea_conv2d: unknown epilogue kind %d", (int)params.epilogue);
+  st = check_bias_residual("tracea_conv2d", bias, residual, plan.out.shape[3], plan.out,
+                           plan.out.device, ops, n);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain("tracea_conv2d", ops, (uint32_t)n, plan.out.shape[3], plan.out.shape[3], &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  return run_conv(plan, chain, (hipStream_t)params.stream);
+}
+
+TraceaStatus dispatch_conv2d_ops(const TraceaTensorView &tx, const TraceaTensorView &tw,
+                                 TraceaTensorView *tout, const TraceaConv2dParams &params,
+                                 const TraceaEpilogueOp *ops, uint32_t n_ops) {
+  ConvPlan plan;
+  TraceaStatus st = conv_common(tx, tw, tout, params, &plan);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain("tracea_conv2d_ex", ops, n_ops, plan.out.shape[3], plan.out.shape[3], &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  return run_conv(plan, chain, (hipStream_t)params.stream);
+}
+
+// ---- attention ---------------------------------------------------------------------
+TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorView &tk,
+                                const TraceaTensorView &tv, TraceaTensorView *to,
+                                const TraceaAttentionParams &params) {
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "tracea_attention: tracea_init has not been called");
+  if (to == nullptr) return fail(TRACEA_INVALID_PARAMS, "tracea_attention: output view is NULL");
+  View q, k, v, o;
+  TraceaStatus st;
+  if ((st = read_view("tracea_attention: q", tq, 4, &q)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_attention: k", tk, 4, &k)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_attention: v", tv, 4, &v)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_attention: o", *to, 4, &o)) != TRACEA_SUCCESS) return st;
+  if (!is_half(q.dtype) || k.dtype != q.dtype || v.dtype != q.dtype || o.dtype != q.dtype)
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_attention: q/k/v/o must all be f16 or all bf16 (got %s,%s,%s,%s)",
+                dtype_name(q.dtype), dtype_name(k.dtype), dtype_name(v.dtype), dtype_name(o.dtype));
+  for (int i = 0; i < 4; ++i)
+    if (k.shape[i] != q.shape[i] || v.shape[i] != q.shape[i] || o.shape[i] != q.shape[i])
+      return fail(TRACEA_INVALID_PARAMS, "tracea_attention: q, k, v and o must share one [B,H,S,D] shape");
+  if ((st = check_device("tracea_attention", o.device)) != TRACEA_SUCCESS) return st;
+  if (q.device != o.device || k.device != o.device || v.device != o.device)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_attention: operands live on different devices");
+  const long long B = q.shape[0], H = q.shape[1], S = q.shape[2], D = q.shape[3];
+  if (B == 0 || H == 0 || S == 0) return TRACEA_SUCCESS;
+  if (D != 64 && D != 128)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: head dim %lld (64 or 128 supported)", D);
+  if (S >= (1ll << 31) || B * H * ((S + 127) / 128) >= (1ll << 31))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: problem too large");
+  const View *views[4] = {&q, &k, &v, &o};
+  for (const View *t : views) {
+    if (t->stride[3] != 1 || t->stride[2] % 8 != 0 || t->stride[1] % 8 != 0 || t->stride[0] % 8 != 0 ||
+        !aligned(t->ptr, 16))
+      return fail(TRACEA_UNSUPPORTED_CONFIG,
+                  "tracea_attention: head dim must be contiguous, other strides multiples of 8 "
+                  "elements, bases 16-byte aligned");
+  }
+  float scale = params.scale;
+  if (scale == 0.0f) scale = 1.0f / sqrtf((float)D);
+  if (!(scale == scale) || std::isinf(scale))
+    return fail(TRACEA_INVALID_PARAMS, "tracea_attention: scale is not finite");
+
+  AttentionArgs a{};
+  a.Q = q.ptr; a.K = k.ptr; a.V = v.ptr; a.O = o.ptr;
+  a.B = (int)B; a.H = (int)H; a.S = (int)S; a.D = (int)D;
+  a.q_sb = q.stride[0]; a.q_sh = q.stride[1]; a.q_ss = q.stride[2];
+  a.k_sb = k.stride[0]; a.k_sh = k.stride[1]; a.k_ss = k.stride[2];
+  a.v_sb = v.stride[0]; a.v_sh = v.stride[1]; a.v_ss = v.stride[2];
+  a.o_sb = o.stride[0]; a.o_sh = o.stride[1]; a.o_ss = o.stride[2];
+  a.scale_log2 = scale * 1.4426950408889634f;
+  a.causal = params.causal ? 1 : 0;
+
+  int vi = forced_variant("attention");
+  if (vi >= 0 && !attention_variant(vi).feasible(a)) vi = -1;
+  if (vi < 0) {
+    for (int i = 0; i < attention_variant_count(); ++i)
+      if (attention_variant(i).feasible(a)) {
+        vi = i;
+        break;
+      }
+  }
+  if (vi < 0) return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: no kernel variant fits");
+  DeviceScope scope(o.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  return hip_status("attention launch",
+                    attention_variant(vi).launch(a, q.dtype, (hipStream_t)params.stream));
+}
+
+}  // namespace tracea_amd

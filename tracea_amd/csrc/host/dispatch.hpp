@@ -1,0 +1,60 @@
+// Host side of the library above the kernels: argument checking, operator
+// chains, kernel-variant selection, tuning.  C++ counterpart of the reference's
+// Rust host layer for this path (src/interface/c_bindings.rs,
+// src/core/tuning.rs, src/optimizer/mod.rs).
+#pragma once
+#include <string>
+
+#include "../common.hpp"
+
+namespace tracea_amd {
+
+// error slot / lifecycle (defined in abi.cpp)
+TraceaStatus fail(TraceaStatus st, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+bool runtime_ready();
+int runtime_device_count();
+
+// Convolution geometry with the reciprocal ("magic") numbers of every divisor
+// the coordinate mapping uses.
+struct ConvGeometry {
+  TraceaConvParamsBlock block;  // reference-compatible 80-byte block (symmetric form)
+  int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
+  int m_gemm, n_gemm, k_gemm;
+};
+TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s, int stride_h,
+                                int stride_w, int pad_h, int pad_w, int dil_h, int dil_w,
+                                ConvGeometry *out);
+
+// magic = ceil(2^(32+shift)/d) (0 for powers of two, shift = log2 d), chosen so
+// that fast_divmod is exact for every 0 <= n <= n_max.
+void magic_for_divisor(uint32_t d, uint64_t n_max, uint32_t *magic, uint32_t *shift);
+
+void set_forced_variant(const char *op, int index);
+int forced_variant(const char *op);
+
+TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorView &b,
+                                const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                TraceaTensorView *c, const TraceaGemmParams &params);
+TraceaStatus dispatch_gemm_ops(const TraceaTensorView &a, const TraceaTensorView &b,
+                               TraceaTensorView *c, const TraceaGemmParams &params,
+                               const TraceaEpilogueOp *ops, uint32_t n_ops);
+TraceaStatus dispatch_conv2d_kind(const TraceaTensorView &x, const TraceaTensorView &w,
+                                  const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                  TraceaTensorView *out, const TraceaConv2dParams &params);
+TraceaStatus dispatch_conv2d_ops(const TraceaTensorView &x, const TraceaTensorView &w,
+                                 TraceaTensorView *out, const TraceaConv2dParams &params,
+                                 const TraceaEpilogueOp *ops, uint32_t n_ops);
+TraceaStatus dispatch_attention(const TraceaTensorView &q, const TraceaTensorView &k,
+                                const TraceaTensorView &v, TraceaTensorView *o,
+                                const TraceaAttentionParams &params);
+
+// Heuristic choice among the feasible contraction variants (used when neither a
+// forced variant nor a tuning-cache entry decides).  Returns -1 if none fits.
+int select_contraction_variant(int m, int n, int k, bool conv);
+
+TraceaResult tune_gemm(size_t m, size_t n, size_t k);
+TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal);
+TraceaResult tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s,
+                         size_t stride, size_t pad, size_t dilation);
+
+}  // namespace tracea_amd

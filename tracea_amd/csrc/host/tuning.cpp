@@ -1,0 +1,404 @@
+// Tuning cache and the exhaustive micro-benchmark tuner behind
+// tracea_tune_gemm / tracea_tune_conv2d / tracea_tune_fa2.
+//
+// Reference behaviour kept: TuningCache::get_or_tune is a grid search over
+// the candidate list with the best TFLOP/s winning and the entry persisted
+// at once (src/core/tuning.rs:92-139); the benchmark protocol is warm-up
+// launches followed by timed launches of the real kernel on device buffers
+// (src/optimizer/benchmark.rs:255-343, 814-868); GEMM flops = 2MNK
+// (benchmark.rs:188-190), conv flops = 2*M*N*K of the implicit GEMM
+// (benchmark.rs:466-469), attention flops = 4*B*H*S^2*D for causal and dense
+// alike (benchmark.rs:954-957).  Timing uses HIP events on one stream instead
+// of the reference's host clock.
+#include <sys/stat.h>
+
+#include <chrono>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <map>
+#include <mutex>
+#include <sstream>
+
+#include "dispatch.hpp"
+#include "tuning_cache.hpp"
+
+namespace tracea_amd {
+
+namespace {
+std::mutex g_mu;
+std::map<std::string, CacheEntry> g_cache;
+bool g_loaded = false;
+std::string g_device_name;
+
+void load_locked() {
+  if (g_loaded) return;
+  g_loaded = true;
+  std::ifstream f(tuning_cache_path());
+  if (!f) return;
+  std::stringstream ss;
+  ss << f.rdbuf();
+  Json root;
+  std::string err;
+  if (!Json::parse(ss.str(), &root, &err) || root.type != Json::Object) return;
+  for (const auto &kv : root.obj) {
+    const Json *cfg = kv.second.find("config");
+    CacheEntry e;
+    if (!cfg || !PipelineConfig::from_json_value(*cfg, &e.config, &err)) continue;
+    if (const Json *s = kv.second.find("score")) e.score = (float)s->num;
+    if (const Json *t = kv.second.find("timestamp")) e.timestamp = (uint64_t)t->num;
+    g_cache[kv.first] = e;
+  }
+}
+
+void save_locked() {
+  const std::string path = tuning_cache_path();
+  const size_t slash = path.find_last_of('/');
+  if (slash != std::string::npos) mkdir(path.substr(0, slash).c_str(), 0755);
+  Json root = Json::make_obj();
+  for (const auto &kv : g_cache) {
+    Json e = Json::make_obj();
+    e.set("config", kv.second.config.to_json_value());
+    e.set("score", Json::make_num(kv.second.score));
+    e.set("timestamp", Json::make_num((double)kv.second.timestamp));
+    root.set(kv.first, e);
+  }
+  std::ofstream f(path);
+  if (f) f << root.dump(2) << "\n";
+}
+}  // namespace
+
+const char *tuning_device_name() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (g_device_name.empty() && runtime_ready()) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) == hipSuccess) g_device_name = prop.name;
+  }
+  return g_device_name.c_str();
+}
+
+std::string tuning_cache_path() {
+  const char *env = getenv("TRACEA_TUNING_CACHE");
+  return env && *env ? std::string(env) : std::string(".tracea/tuning_cache_v2.json");
+}
+
+bool tuning_cache_get(const std::string &key, CacheEntry *out) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  load_locked();
+  auto it = g_cache.find(key);
+  if (it == g_cache.end()) return false;
+  if (out) *out = it->second;
+  return true;
+}
+
+void tuning_cache_put(const std::string &key, const CacheEntry &e, bool persist) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  load_locked();
+  g_cache[key] = e;
+  if (persist) save_locked();
+}
+
+void tuning_cache_reload() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  g_cache.clear();
+  g_loaded = false;
+}
+
+int tuning_cache_lookup_variant(const std::string &key) {
+  CacheEntry e;
+  if (!tuning_cache_get(key, &e)) return -1;
+  return contraction_variant_for_config(e.config);
+}
+
+// A contraction variant as a PipelineConfig: tiles, LDS stages, wave count
+// (force_num_warps) and the per-wave tile (micro_m x micro_n).  The reference's
+// IntrinsicShape enum has no 32x32x16 entry; M32N32K2 names the 32x32 MFMA
+// family, the only spelling a reference build would accept.
+PipelineConfig config_for_contraction_variant(int index) {
+  const ContractionVariant &v = contraction_variant(index);
+  PipelineConfig c((uint32_t)v.stages, (uint32_t)v.bm, (uint32_t)v.bn, (uint32_t)v.bk);
+  c.instruction = "RocmMFMA";
+  c.swizzle_mode = "Xor8";
+  c.layout_policy = "XorSwizzled";
+  c.has_force_num_warps = true;
+  c.force_num_warps = (uint32_t)(v.waves_m * v.waves_n);
+  c.micro_m = (uint32_t)(v.bm / v.waves_m);
+  c.micro_n = (uint32_t)(v.bn / v.waves_n);
+  c.intrinsic_shape = "M32N32K2";
+  c.gemm_variant = "Simd";
+  c.double_buffer = true;
+  c.cp_async_distance = v.direct_to_lds ? 1 : 0;
+  c.bank_conflict_padding = 0;
+  return c;
+}
+
+int contraction_variant_for_config(const PipelineConfig &c) {
+  for (int i = 0; i < contraction_variant_count(); ++i) {
+    const ContractionVariant &v = contraction_variant(i);
+    if ((uint32_t)v.bm != c.m_tile || (uint32_t)v.bn != c.n_tile || (uint32_t)v.bk != c.k_tile) continue;
+    if ((uint32_t)v.stages != c.num_stages) continue;
+    if (c.has_force_num_warps && (uint32_t)(v.waves_m * v.waves_n) != c.force_num_warps) continue;
+    if (c.micro_m > 1 && (uint32_t)(v.bm / v.waves_m) != c.micro_m) continue;
+    if ((c.cp_async_distance != 0) != v.direct_to_lds) continue;
+    return i;
+  }
+  return -1;
+}
+
+PipelineConfig config_for_attention_variant(int index) {
+  const AttentionVariant &v = attention_variant(index);
+  PipelineConfig c(2, (uint32_t)v.block_q, (uint32_t)v.block_kv, 32);
+  c.instruction = "RocmMFMA";
+  c.swizzle_mode = "Xor8";
+  c.has_force_num_warps = true;
+  c.force_num_warps = (uint32_t)v.waves;
+  c.intrinsic_shape = "M32N32K2";
+  c.attention_variant = "FlashV2";
+  c.softmax_granularity = "PerTile";
+  c.double_buffer = true;
+  c.bank_conflict_padding = 0;
+  return c;
+}
+
+// ---- micro-benchmarks ------------------------------------------------------------
+namespace {
+
+struct DeviceBuffer {
+  void *p = nullptr;
+  ~DeviceBuffer() {
+    if (p) (void)hipFree(p);
+  }
+  bool alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16) == hipSuccess; }
+};
+
+char *dup_cstr(const std::string &s) {
+  char *p = (char *)malloc(s.size() + 1);
+  if (p) memcpy(p, s.c_str(), s.size() + 1);
+  return p;
+}
+
+TraceaResult failure(const std::string &msg) {
+  TraceaResult r;
+  r.success = false;
+  r.error_msg = dup_cstr(msg);
+  r.score = 0.0f;
+  r.config_ptr = nullptr;
+  return r;
+}
+
+TraceaResult success(const PipelineConfig &cfg, float tflops) {
+  TraceaResult r;
+  r.success = true;
+  r.error_msg = nullptr;
+  r.score = tflops;
+  r.config_ptr = dup_cstr(cfg.to_json());
+  return r;
+}
+
+std::string last_error_text() {
+  uint8_t buf[512];
+  const int n = tracea_get_last_error(buf, sizeof(buf));
+  return n > 0 ? std::string((const char *)buf, (size_t)n) : std::string("unknown error");
+}
+
+// Times `launch` (which must enqueue exactly one kernel on the default stream):
+// warm-up launches, then `iters` launches between two events.  Returns seconds
+// per launch, or a negative value on error.
+template <typename F>
+double time_launches(F &&launch, int warmup, int iters) {
+  hipEvent_t e0, e1;
+  if (hipEventCreate(&e0) != hipSuccess) return -1.0;
+  if (hipEventCreate(&e1) != hipSuccess) {
+    (void)hipEventDestroy(e0);
+    return -1.0;
+  }
+  double result = -1.0;
+  bool ok = true;
+  for (int i = 0; i < warmup && ok; ++i) ok = launch();
+  if (ok && hipDeviceSynchronize() == hipSuccess) {
+    (void)hipEventRecord(e0, nullptr);
+    for (int i = 0; i < iters && ok; ++i) ok = launch();
+    (void)hipEventRecord(e1, nullptr);
+    if (ok && hipEventSynchronize(e1) == hipSuccess) {
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, e0, e1) == hipSuccess) result = (double)ms * 1e-3 / iters;
+    }
+  }
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  return result;
+}
+
+uint64_t now_seconds() {
+  return (uint64_t)std::chrono::duration_cast<std::chrono::seconds>(
+             std::chrono::system_clock::now().time_since_epoch())
+      .count();
+}
+
+}  // namespace
+
+TraceaResult tune_gemm(size_t m, size_t n, size_t k) {
+  if (!runtime_ready()) return failure("tracea_init has not been called");
+  if (m == 0 || n == 0 || k == 0 || k % 8 != 0 || m >= (1u << 31) || n >= (1u << 31) || k >= (1u << 31))
+    return failure("tune_gemm: dimensions must be positive, K a multiple of 8");
+  // fp16, A row-major [M,K], B column-major (stored [N,K]), C fp16 row-major
+  DeviceBuffer a, b, c;
+  if (!a.alloc(m * k * 2) || !b.alloc(n * k * 2) || !c.alloc(m * n * 2)) {
+    (void)hipGetLastError();
+    return failure("tune_gemm: device allocation failed");
+  }
+  const float amp = sqrtf(3.0f / (float)k);  // unit-variance dot products
+  launch_fill_uniform(a.p, m * k, DT_F16, 1u, amp, nullptr);
+  launch_fill_uniform(b.p, n * k, DT_F16, 2u, amp, nullptr);
+  const uint64_t sa[2] = {m, k}, sb[2] = {k, n}, sc[2] = {m, n};
+  const int64_t ta[2] = {(int64_t)k, 1}, tb[2] = {1, (int64_t)k}, tcs[2] = {(int64_t)n, 1};
+  TraceaTensorView va{a.p, 2, sa, ta, TRACEA_DTYPE_FLOAT16, 0};
+  TraceaTensorView vb{b.p, 2, sb, tb, TRACEA_DTYPE_FLOAT16, 0};
+  TraceaTensorView vc{c.p, 2, sc, tcs, TRACEA_DTYPE_FLOAT16, 0};
+  TraceaGemmParams gp{TRACEA_EPILOGUE_IDENTITY, nullptr};
+  const int saved = forced_variant("gemm");
+  const double flops = 2.0 * (double)m * (double)n * (double)k;
+  int best = -1;
+  double best_tflops = 0.0;
+  std::string err;
+  for (int i = 0; i < contraction_variant_count(); ++i) {
+    set_forced_variant("gemm", i);
+    const double t = time_launches(
+        [&]() { return dispatch_gemm_kind(va, vb, nullptr, nullptr, &vc, gp) == TRACEA_SUCCESS; }, 3, 10);
+    if (t <= 0.0) {
+      err = last_error_text();
+      continue;
+    }
+    const double tf = flops / t * 1e-12;
+    if (tf > best_tflops) {
+      best_tflops = tf;
+      best = i;
+    }
+  }
+  set_forced_variant("gemm", saved);
+  if (best < 0) return failure("tune_gemm: no variant ran: " + err);
+  CacheEntry e;
+  e.config = config_for_contraction_variant(best);
+  e.score = (float)best_tflops;
+  e.timestamp = now_seconds();
+  char key[160];
+  snprintf(key, sizeof(key), "gemm_%zu_%zu_%zu_%s", m, n, k, tuning_device_name());
+  tuning_cache_put(key, e, true);
+  return success(e.config, e.score);
+}
+
+TraceaResult tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s,
+                         size_t stride, size_t pad, size_t dilation) {
+  if (!runtime_ready()) return failure("tracea_init has not been called");
+  if (n == 0 || c == 0 || h == 0 || w == 0 || k == 0 || r == 0 || s == 0 || stride == 0 || dilation == 0)
+    return failure("tune_conv2d: dimensions, stride and dilation must be positive");
+  if (c % 8 != 0) return failure("tune_conv2d: input channels must be a multiple of 8");
+  ConvGeometry g;
+  if (make_conv_geometry((int)n, (int)h, (int)w, (int)c, (int)k, (int)r, (int)s, (int)stride,
+                         (int)stride, (int)pad, (int)pad, (int)dilation, (int)dilation,
+                         &g) != TRACEA_SUCCESS)
+    return failure("tune_conv2d: " + last_error_text());
+  const size_t ho = (size_t)g.block.h_out, wo = (size_t)g.block.w_out;
+  DeviceBuffer x, wt, y;
+  if (!x.alloc(n * h * w * c * 2) || !wt.alloc(k * r * s * c * 2) || !y.alloc(n * ho * wo * k * 2)) {
+    (void)hipGetLastError();
+    return failure("tune_conv2d: device allocation failed");
+  }
+  launch_fill_uniform(x.p, n * h * w * c, DT_F16, 3u, 1.0f, nullptr);
+  launch_fill_uniform(wt.p, k * r * s * c, DT_F16, 4u, sqrtf(3.0f / (float)(r * s * c)), nullptr);
+  const uint64_t sx[4] = {n, h, w, c}, sw[4] = {k, r, s, c}, sy[4] = {n, ho, wo, k};
+  TraceaTensorView vx{x.p, 4, sx, nullptr, TRACEA_DTYPE_FLOAT16, 0};
+  TraceaTensorView vw{wt.p, 4, sw, nullptr, TRACEA_DTYPE_FLOAT16, 0};
+  TraceaTensorView vy{y.p, 4, sy, nullptr, TRACEA_DTYPE_FLOAT16, 0};
+  TraceaConv2dParams cp{(uint32_t)stride, (uint32_t)stride, (uint32_t)pad, (uint32_t)pad,
+                        (uint32_t)dilation, (uint32_t)dilation, 1, TRACEA_EPILOGUE_RELU, nullptr};
+  const int saved = forced_variant("conv2d");
+  const double flops = 2.0 * (double)g.m_gemm * (double)g.n_gemm * (double)g.k_gemm;
+  int best = -1;
+  double best_tflops = 0.0;
+  std::string err;
+  for (int i = 0; i < contraction_variant_count(); ++i) {
+    set_forced_variant("conv2d", i);
+    const double t = time_launches(
+        [&]() { return dispatch_conv2d_kind(vx, vw, nullptr, nullptr, &vy, cp) == TRACEA_SUCCESS; }, 3, 10);
+    if (t <= 0.0) {
+      err = last_error_text();
+      continue;
+    }
+    const double tf = flops / t * 1e-12;
+    if (tf > best_tflops) {
+      best_tflops = tf;
+      best = i;
+    }
+  }
+  set_forced_variant("conv2d", saved);
+  if (best < 0) return failure("tune_conv2d: no variant ran: " + err);
+  CacheEntry e;
+  e.config = config_for_contraction_variant(best);
+  e.config.layout_policy = "NHWC";
+  e.score = (float)best_tflops;
+  e.timestamp = now_seconds();
+  char key[200];
+  snprintf(key, sizeof(key), "conv_%zu_%zu_%zu_%zu_%zu_%zu_%zu_%zu_%zu_%s", n, h, w, c, k, r, s,
+           stride, pad, tuning_device_name());
+  tuning_cache_put(key, e, true);
+  return success(e.config, e.score);
+}
+
+TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
+  if (!runtime_ready()) return failure("tracea_init has not been called");
+  if (b == 0 || h == 0 || s == 0 || (d != 64 && d != 128))
+    return failure("tune_fa2: B, H, S must be positive and D 64 or 128");
+  const size_t elems = b * h * s * d;
+  DeviceBuffer q, k, v, o;
+  if (!q.alloc(elems * 2) || !k.alloc(elems * 2) || !v.alloc(elems * 2) || !o.alloc(elems * 2)) {
+    (void)hipGetLastError();
+    return failure("tune_fa2: device allocation failed");
+  }
+  launch_fill_uniform(q.p, elems, DT_BF16, 5u, 1.7f, nullptr);
+  launch_fill_uniform(k.p, elems, DT_BF16, 6u, 1.7f, nullptr);
+  launch_fill_uniform(v.p, elems, DT_BF16, 7u, 1.7f, nullptr);
+  const uint64_t sh[4] = {b, h, s, d};
+  TraceaTensorView vq{q.p, 4, sh, nullptr, TRACEA_DTYPE_BFLOAT16, 0};
+  TraceaTensorView vk{k.p, 4, sh, nullptr, TRACEA_DTYPE_BFLOAT16, 0};
+  TraceaTensorView vv{v.p, 4, sh, nullptr, TRACEA_DTYPE_BFLOAT16, 0};
+  TraceaTensorView vo{o.p, 4, sh, nullptr, TRACEA_DTYPE_BFLOAT16, 0};
+  TraceaAttentionParams ap{(uint8_t)(causal ? 1 : 0), TRACEA_SOFTMAX_AUTO, 0.0f, nullptr};
+  const int saved = forced_variant("attention");
+  const double flops = 4.0 * (double)b * (double)h * (double)s * (double)s * (double)d;
+  int best = -1;
+  double best_tflops = 0.0;
+  std::string err;
+  for (int i = 0; i < attention_variant_count(); ++i) {
+    AttentionArgs probe{};
+    probe.D = (int)d;
+    if (!attention_variant(i).feasible(probe)) continue;
+    set_forced_variant("attention", i);
+    const double t = time_launches(
+        [&]() { return dispatch_attention(vq, vk, vv, &vo, ap) == TRACEA_SUCCESS; }, 2, 5);
+    if (t <= 0.0) {
+      err = last_error_text();
+      continue;
+    }
+    const double tf = flops / t * 1e-12;
+    if (tf > best_tflops) {
+      best_tflops = tf;
+      best = i;
+    }
+  }
+  set_forced_variant("attention", saved);
+  if (best < 0) return failure("tune_fa2: no variant ran: " + err);
+  CacheEntry e;
+  e.config = config_for_attention_variant(best);
+  e.score = (float)best_tflops;
+  e.timestamp = now_seconds();
+  // key of the reference's attention adapter (src/kernels/attention/cuda_adapter.rs)
+  char key[200];
+  snprintf(key, sizeof(key), "fa2_kernel:b%zu_s%zu_h%zu_d%zu_%s", b, s, h, d, causal ? "causal" : "dense");
+  tuning_cache_put(key, e, true);
+  return success(e.config, e.score);
+}
+
+}  // namespace tracea_amd

@@ -1,0 +1,224 @@
+// Kernels around the half-precision MFMA family: the fp32 GEMM, the
+// any-layout fallback GEMM and the coordinate-table dump of the convolution.
+#include "contraction_kernel.hpp"
+
+namespace tracea_amd {
+
+// ---------------------------------------------------------------------------
+// fp32 GEMM on the fp32 matrix cores (v_mfma_f32_32x32x2_f32).
+// C[M,N] = epilogue(A[M,K] . B[K,N]), all row-major.  This is the device
+// counterpart of the reference's only executable CPU path, gemm_cpu_packed
+// (src/kernels/cpu/gemm.rs:241-298), except that C is overwritten, as in the
+// reference's GPU GEMM (src/emitter/cuda/gemm.rs:179-205), not accumulated.
+// Tile 128x128x16, 4 waves (2x2), wave tile 64x64.  A is staged k-major in LDS
+// so that a wave's operand fetch reads 32 consecutive floats.
+// Requires K % 4 == 0, N % 4 == 0, lda % 4 == 0, ldb % 4 == 0 and 16-byte
+// aligned bases (checked by the dispatcher).
+// ---------------------------------------------------------------------------
+constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16, F32_PITCH = 132;
+
+__global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs args) {
+  __shared__ float As[F32_BK][F32_PITCH];
+  __shared__ float Bs[F32_BK][F32_PITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  int tile_m, tile_n;
+  tile_coordinates(args, tile_m, tile_n);
+  const int m0 = tile_m * F32_BM, n0 = tile_n * F32_BN;
+  const int M = args.M, N = args.N, K = args.K;
+  const float *A = (const float *)args.A;
+  const float *B = (const float *)args.B;
+
+  // A tile: 128 rows x 16 k = 512 float4 pieces, 2 per thread (row = q/4, kq = q%4)
+  // B tile: 16 k x 128 n   = 512 float4 pieces, 2 per thread (k = q/32, nq = q%32)
+  f32x4 ra[2], rb[2];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = tid + i * 256;
+      int m = m0 + q / 4;
+      m = m < M ? m : M - 1;
+      const int k = k0 + (q % 4) * 4;
+      const bool ok = k < K;
+      const f32x4 v = *(const f32x4 *)(A + (long long)m * args.lda + (ok ? k : 0));
+      const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+      ra[i] = ok ? v : z;
+      const int kb = k0 + q / 32;
+      const int n = n0 + (q % 32) * 4;
+      const bool okb = kb < K && n < N;
+      const f32x4 w = *(const f32x4 *)(B + (okb ? (long long)kb * args.ldb + n : 0ll));
+      rb[i] = okb ? w : z;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int q = tid + i * 256;
+      const int row = q / 4, kq = (q % 4) * 4;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) As[kq + e][row] = ra[i][e];
+      *(f32x4 *)&Bs[q / 32][(q % 32) * 4] = rb[i];
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int nk = (K + F32_BK - 1) / F32_BK;
+  fetch(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    stash();
+    __syncthreads();
+    if (kt + 1 < nk) fetch((kt + 1) * F32_BK);
+#pragma unroll
+    for (int ks = 0; ks < F32_BK / 2; ++ks) {
+      const int k = ks * 2 + lhalf;
+      float af[2], bf[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) af[i] = As[k][wm * 64 + i * 32 + lrow];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) bf[j] = Bs[k][wn * 64 + j * 32 + lrow];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j], af[i], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+  // operands were swapped: lane owns row (lane&31), channels 8g + 4*(lane>>5) + 0..3
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = m0 + wm * 64 + i * 32 + lrow;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * 64 + j * 32 + g * 8 + lhalf * 4;
+        if (m < M && n < N) {
+          float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
+                        acc[i][j][g * 4 + 3]};
+          apply_epilogue<4>(v, m, n, N - n, args.epi);
+          store_from_float<4>(args.C, args.out_dtype, (long long)m * args.ldc + n, N - n, v);
+        }
+      }
+  }
+}
+
+int launch_gemm_f32(const ContractionArgs &a, hipStream_t stream) {
+  ContractionArgs args = a;
+  args.grid_m = (a.M + F32_BM - 1) / F32_BM;
+  args.grid_n = (a.N + F32_BN - 1) / F32_BN;
+  args.group_m = 4;
+  hipLaunchKernelGGL(gemm_f32_kernel, dim3((unsigned)(args.grid_m * args.grid_n)), dim3(256), 0,
+                     stream, args);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Fallback GEMM: any element strides, any of f32/f16/bf16 per operand, no
+// alignment requirement.  One output element per thread, fp32 FMA on the
+// vector ALU.  Correct everywhere, fast nowhere; the dispatcher only uses it
+// when no matrix-core kernel applies.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float load_scalar(const void *p, int dtype, long long idx) {
+  if (dtype == DT_F32) return ((const float *)p)[idx];
+  if (dtype == DT_F16) return (float)((const _Float16 *)p)[idx];
+  return (float)((const __bf16 *)p)[idx];
+}
+
+__global__ void __launch_bounds__(256) gemm_generic_kernel(const GenericGemmArgs a) {
+  const int n = blockIdx.x * 16 + (threadIdx.x & 15);
+  const int m = blockIdx.y * 16 + (threadIdx.x >> 4);
+  if (m >= a.M || n >= a.N) return;
+  float acc = 0.0f;
+  for (int k = 0; k < a.K; ++k)
+    acc = fmaf(load_scalar(a.A, a.a_dtype, (long long)m * a.sam + (long long)k * a.sak),
+               load_scalar(a.B, a.b_dtype, (long long)k * a.sbk + (long long)n * a.sbn), acc);
+  float v[1] = {acc};
+  apply_epilogue<1>(v, m, n, 1, a.epi);
+  store_from_float<1>(a.C, a.c_dtype, (long long)m * a.scm + (long long)n * a.scn, 1, v);
+}
+
+int launch_gemm_generic(const GenericGemmArgs &a, hipStream_t stream) {
+  const dim3 grid((unsigned)((a.N + 15) / 16), (unsigned)((a.M + 15) / 16));
+  hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, stream, a);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Coordinate tables of the convolution, computed on the device with the same
+// fast_divmod the contraction kernel uses, for bit-exact comparison with the
+// CPU statement of src/emitter/cuda/conv.rs:176-191, 208-210.
+// ---------------------------------------------------------------------------
+__global__ void conv_coords_kernel(TraceaConvParamsBlock p, int32_t *rows, int64_t *base_off,
+                                   int32_t *cols) {
+  const int m_gemm = p.batch * p.h_out * p.w_out;
+  const int k_gemm = p.r_sz * p.s_sz * p.c_in;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < m_gemm) {
+    int bn, rem, ho, wo;
+    fast_divmod(i, p.hw_m, p.hw_s, p.h_out * p.w_out, bn, rem);
+    fast_divmod(rem, p.w_m, p.w_s, p.w_out, ho, wo);
+    rows[3 * i] = bn;
+    rows[3 * i + 1] = ho;
+    rows[3 * i + 2] = wo;
+    base_off[i] = (int64_t)bn * p.h_in * p.w_in * p.c_in;
+  }
+  if (i < k_gemm) {
+    int rf, rem, sf, ci;
+    fast_divmod(i, p.sic_m, p.sic_s, p.s_sz * p.c_in, rf, rem);
+    fast_divmod(rem, p.c_m, p.c_s, p.c_in, sf, ci);
+    cols[3 * i] = rf;
+    cols[3 * i + 1] = sf;
+    cols[3 * i + 2] = ci;
+  }
+}
+
+int launch_conv_coords(const TraceaConvParamsBlock &p, int32_t *rows, int64_t *base_off,
+                       int32_t *cols, hipStream_t stream) {
+  const int m_gemm = p.batch * p.h_out * p.w_out;
+  const int k_gemm = p.r_sz * p.s_sz * p.c_in;
+  const int n = m_gemm > k_gemm ? m_gemm : k_gemm;
+  hipLaunchKernelGGL(conv_coords_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, p,
+                     rows, base_off, cols);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Synthetic operand fill for the tuner: splitmix-style hash of the element
+// index, uniform in [-amplitude, amplitude].
+// ---------------------------------------------------------------------------
+__global__ void fill_uniform_kernel(void *ptr, size_t n, int dtype, unsigned seed, float amplitude) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    unsigned long long z = (i + 1) * 0x9E3779B97F4A7C15ull + ((unsigned long long)seed << 32);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    const float u = (float)(z >> 40) * (1.0f / 16777216.0f);  // [0,1)
+    const float v = (2.0f * u - 1.0f) * amplitude;
+    if (dtype == DT_F32) ((float *)ptr)[i] = v;
+    else if (dtype == DT_F16) ((_Float16 *)ptr)[i] = (_Float16)v;
+    else ((__bf16 *)ptr)[i] = (__bf16)v;
+  }
+}
+
+int launch_fill_uniform(void *ptr, size_t n, int dtype, unsigned seed, float amplitude,
+                        hipStream_t stream) {
+  if (n == 0) return 0;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(fill_uniform_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, ptr, n,
+                     dtype, seed, amplitude);
+  return (int)hipGetLastError();
+}
+
+}  // namespace tracea_amd

@@ -1,0 +1,172 @@
+"""Operator front end on torch tensors, over the C ABI.
+
+Mirrors the call surface of the reference's Python layer: ``gemm``,
+``conv2d`` and ``attention`` of ``PyContext`` (src/interface/python.rs:124-462)
+and ``tracea.ops.conv2d`` (tracea-python/python/tracea/ops.py:39-70), including
+its epilogue string grammar ("bias+relu", src/interface/python.rs:41-87).
+torch supplies device memory and the current stream; all arithmetic happens in
+``libtracea.so``.
+"""
+import ctypes as C
+
+import torch
+
+from . import capi
+
+_DTYPES = {torch.float32: capi.F32, torch.float16: capi.F16, torch.bfloat16: capi.BF16,
+           torch.int32: capi.I32, torch.int8: capi.I8}
+
+
+def _view(t, shape=None, stride=None):
+    if t.dtype not in _DTYPES:
+        raise TypeError("unsupported dtype %s" % t.dtype)
+    dev = t.device.index if t.is_cuda else -1
+    if t.is_cuda and dev is None:
+        dev = torch.cuda.current_device()
+    return capi.View(t.data_ptr(), list(shape if shape is not None else t.shape),
+                     list(stride if stride is not None else t.stride()), _DTYPES[t.dtype], dev)
+
+
+def _stream(t):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream) if t.is_cuda else None
+
+
+_EPILOGUE_STRINGS = {
+    "": capi.EPI_IDENTITY, "none": capi.EPI_IDENTITY, "identity": capi.EPI_IDENTITY,
+    "bias": capi.EPI_BIAS_ADD, "relu": capi.EPI_RELU, "gelu": capi.EPI_GELU, "silu": capi.EPI_SILU,
+    "bias+relu": capi.EPI_BIAS_RELU, "bias+silu": capi.EPI_BIAS_SILU,
+    "residual": capi.EPI_RESIDUAL, "residual+relu": capi.EPI_RESIDUAL_RELU,
+}
+
+
+def parse_epilogue(spec):
+    """"bias+relu" style string or a TraceaEpilogueKind integer -> kind."""
+    if isinstance(spec, int):
+        return spec
+    key = (spec or "").strip().lower().replace(" ", "")
+    if key not in _EPILOGUE_STRINGS:
+        raise ValueError("unknown epilogue %r" % spec)
+    return _EPILOGUE_STRINGS[key]
+
+
+def gemm(a, b, out=None, bias=None, residual=None, epilogue="none", out_dtype=None):
+    """out[M,N] = epilogue(a[M,K] @ b[K,N]).  b may be any strided 2-D view; a
+    column-major B is ``storage_nk.t()``."""
+    m, k = a.shape
+    k2, n = b.shape
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or a.dtype, device=a.device)
+    va, vb, vc = _view(a), _view(b), _view(out)
+    vbias = _view(bias) if bias is not None else None
+    vres = _view(residual) if residual is not None else None
+    params = capi.GemmParams(parse_epilogue(epilogue), _stream(a))
+    st = capi.lib().tracea_gemm(va.c, vb.c, C.byref(vbias.c) if vbias else None,
+                                C.byref(vres.c) if vres else None, C.byref(vc.c), params)
+    capi.check("tracea_gemm", st)
+    return out
+
+
+def _ops_array(ops):
+    """[(kind, tensors..., [eps])] -> (EpilogueOp array, keep-alive list)."""
+    arr = (capi.EpilogueOp * max(1, len(ops)))()
+    keep = []
+    for i, op in enumerate(ops):
+        kind = op[0]
+        tensors = [t for t in op[1:] if isinstance(t, torch.Tensor)]
+        scalars = [t for t in op[1:] if not isinstance(t, torch.Tensor)]
+        arr[i].kind = kind
+        arr[i].dtype = _DTYPES[tensors[0].dtype] if tensors else capi.F32
+        for slot, t in zip(("p0", "p1", "p2", "p3"), tensors):
+            setattr(arr[i], slot, t.data_ptr())
+            keep.append(t)
+        arr[i].epsilon = float(scalars[0]) if scalars else 0.0
+        arr[i].ld = 0
+        if kind == capi.OP_RESIDUAL_ADD and tensors:
+            arr[i].ld = tensors[0].stride(-2) if tensors[0].dim() >= 2 else 0
+    return arr, keep
+
+
+def gemm_ex(a, b, ops, out=None, out_dtype=None):
+    """GEMM with an explicit operator chain, e.g. [(OP_BIAS_ADD, bias), (OP_RELU,)]."""
+    m, _ = a.shape
+    _, n = b.shape
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or a.dtype, device=a.device)
+    va, vb, vc = _view(a), _view(b), _view(out)
+    arr, _keep = _ops_array(ops)
+    params = capi.GemmParams(capi.EPI_IDENTITY, _stream(a))
+    st = capi.lib().tracea_gemm_ex(va.c, vb.c, C.byref(vc.c), params, arr, len(ops))
+    capi.check("tracea_gemm_ex", st)
+    return out
+
+
+def conv_out_shape(x_shape, w_shape, stride, padding, dilation):
+    n, h, w, _ = x_shape
+    k, r, s, _ = w_shape
+    ho = (h + 2 * padding[0] - dilation[0] * (r - 1) - 1) // stride[0] + 1
+    wo = (w + 2 * padding[1] - dilation[1] * (s - 1) - 1) // stride[1] + 1
+    return (n, ho, wo, k)
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+def _weight_view(w, layout):
+    """Filter view with dims [K,R,S,C] whatever the storage order."""
+    if layout == "krsc":
+        return _view(w)
+    if layout == "rsck":
+        r, s, c, k = w.shape
+        sr, ss, sc, sk = w.stride()
+        return _view(w, shape=(k, r, s, c), stride=(sk, sr, ss, sc))
+    raise ValueError("weight layout must be 'krsc' or 'rsck'")
+
+
+def conv2d(x, w, bias=None, residual=None, stride=1, padding=0, dilation=1, epilogue="none",
+           out=None, weight_layout="krsc", out_dtype=None):
+    """x [N,H,W,C] (NHWC); w [K,R,S,C] ('krsc') or [R,S,C,K] ('rsck'); out [N,Ho,Wo,K]."""
+    stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+    vw = _weight_view(w, weight_layout)
+    wshape = tuple(vw.c.shape[i] for i in range(4))
+    if out is None:
+        out = torch.empty(conv_out_shape(x.shape, wshape, stride, padding, dilation),
+                          dtype=out_dtype or x.dtype, device=x.device)
+    vx, vo = _view(x), _view(out)
+    vbias = _view(bias) if bias is not None else None
+    vres = _view(residual) if residual is not None else None
+    params = capi.Conv2dParams(stride[0], stride[1], padding[0], padding[1], dilation[0],
+                               dilation[1], 1, parse_epilogue(epilogue), _stream(x))
+    st = capi.lib().tracea_conv2d(vx.c, vw.c, C.byref(vbias.c) if vbias else None,
+                                  C.byref(vres.c) if vres else None, C.byref(vo.c), params)
+    capi.check("tracea_conv2d", st)
+    return out
+
+
+def conv2d_ex(x, w, ops, stride=1, padding=0, dilation=1, out=None, weight_layout="krsc",
+              out_dtype=None):
+    """Convolution with an explicit operator chain (BatchNorm, scale/shift, ...)."""
+    stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
+    vw = _weight_view(w, weight_layout)
+    wshape = tuple(vw.c.shape[i] for i in range(4))
+    if out is None:
+        out = torch.empty(conv_out_shape(x.shape, wshape, stride, padding, dilation),
+                          dtype=out_dtype or x.dtype, device=x.device)
+    vx, vo = _view(x), _view(out)
+    arr, _keep = _ops_array(ops)
+    params = capi.Conv2dParams(stride[0], stride[1], padding[0], padding[1], dilation[0],
+                               dilation[1], 1, capi.EPI_IDENTITY, _stream(x))
+    st = capi.lib().tracea_conv2d_ex(vx.c, vw.c, C.byref(vo.c), params, arr, len(ops))
+    capi.check("tracea_conv2d_ex", st)
+    return out
+
+
+def attention(q, k, v, causal=False, scale=0.0, out=None):
+    """q,k,v [B,H,S,D] -> softmax(scale q k^T) v; scale 0 means 1/sqrt(D)."""
+    if out is None:
+        out = torch.empty_like(q)
+    vq, vk, vv, vo = _view(q), _view(k), _view(v), _view(out)
+    params = capi.AttentionParams(1 if causal else 0, 0, float(scale), _stream(q))
+    st = capi.lib().tracea_attention(vq.c, vk.c, vv.c, C.byref(vo.c), params)
+    capi.check("tracea_attention", st)
+    return out
