@@ -1,0 +1,145 @@
+"""Benchmark of the dense-contraction path on one MI355X.
+
+One "step" is one launch of the hot kernel on inputs already resident in HBM.
+The headline workload is the fp16 GEMM M=N=K=4096 (A row-major, B column-major,
+fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
+FlashAttention-2 forward named by the metric are timed in the same run and
+reported under "also".  Prints one JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|conv|attention|attention_causal]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
+METRIC = "TFLOPS + % fp16 MFMA peak: GEMM 4096^3, 3x3 implicit-GEMM conv, FA2 fwd"
+
+
+def make_workload(name, torch, ops):
+    """Returns (label, flops per step, algorithmic bytes per step, dtype, step function)."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0x7ACEA000)
+    if name == "gemm":
+        m = n = k = 4096
+        a = (torch.randn(m, k, device=dev, generator=g) / k ** 0.5).half()
+        bt = (torch.randn(n, k, device=dev, generator=g) / k ** 0.5).half()  # column-major B
+        c = torch.empty(m, n, device=dev, dtype=torch.float16)
+        b = bt.t()
+        return ("fp16 GEMM 4096x4096x4096, A row-major, B column-major, fp32 acc, fp16 out",
+                2.0 * m * n * k, 2.0 * (m * k + k * n + m * n), "f16", lambda: ops.gemm(a, b, out=c))
+    if name == "conv":
+        n, h, w, cin, cout = 32, 56, 56, 64, 64
+        x = torch.randn(n, h, w, cin, device=dev, generator=g).half()
+        wt = (torch.randn(cout, 3, 3, cin, device=dev, generator=g) * (2.0 / 576) ** 0.5).half()
+        bias = torch.randn(cout, device=dev, generator=g) * 0.1
+        y = torch.empty(n, h, w, cout, device=dev, dtype=torch.float16)
+        return ("fp16 NHWC conv N32 56x56x64->64 3x3 s1 p1, bias+ReLU",
+                2.0 * n * h * w * cout * 9 * cin, 2.0 * (x.numel() + wt.numel() + y.numel()), "f16",
+                lambda: ops.conv2d(x, wt, bias=bias, stride=1, padding=1, epilogue="bias+relu", out=y))
+    if name in ("attention", "attention_causal"):
+        causal = name.endswith("causal")
+        b, h, s, d = 4, 32, 4096, 128
+        q, k, v = [torch.randn(b, h, s, d, device=dev, generator=g).bfloat16() for _ in range(3)]
+        o = torch.empty_like(q)
+        flops = 4.0 * b * h * d * (s * (s + 1) / 2.0 if causal else float(s) * s)
+        return ("bf16 FA2 forward B4 H32 S4096 D128 %s" % ("causal" if causal else "dense"),
+                flops, 2.0 * 4 * q.numel(), "bf16", lambda: ops.attention(q, k, v, causal=causal, out=o))
+    raise SystemExit("unknown workload " + name)
+
+
+def time_steps(torch, step, steps, warmup):
+    """Wall clock around exactly `steps` launches, plus HIP-event time on the launch stream."""
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()  # the kernels are enqueued on torch's current stream, the one these events see
+    for _ in range(steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall / steps, e0.elapsed_time(e1) * 1e-3 / steps
+
+
+def cpu_baseline():
+    """The reference's CPU SIMD GEMM (restated gemm_cpu_packed, hero tiling) on the host cores,
+    protocol of examples/cpu_bench.rs:34-57: one warm-up call, three timed calls."""
+    import numpy as np
+
+    import oracle
+    threads = oracle.default_threads()
+    out = {}
+    for size in (1024, 4096):
+        rng = np.random.default_rng(0x7ACEA001)
+        a = rng.uniform(-1, 1, (size, size)).astype(np.float32)
+        b = rng.uniform(-1, 1, (size, size)).astype(np.float32)
+        c = np.zeros((size, size), np.float32)
+        oracle.gemm_cpu_packed(a, b, c, nthreads=threads)
+        t0 = time.perf_counter()
+        for _ in range(3):
+            oracle.gemm_cpu_packed(a, b, c, nthreads=threads)
+        out[size] = 2.0 * size ** 3 / ((time.perf_counter() - t0) / 3) / 1e12
+    return {"value": round(out[4096], 4), "unit": "TFLOPS", "cores": threads, "kind": "port",
+            "sample": "fp32 packed AVX2 SGEMM (Mc=Nc=128,Kc=256,Mr=6,Nr=16), 1 warm-up + 3 timed calls at "
+                      "4096^3 (value) and at the reference's 1024^3 (%.4f TFLOPS)" % out[1024]}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="gemm")
+    ap.add_argument("--no-extras", action="store_true", help="skip the conv/attention/CPU legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)")
+
+    import torch
+
+    from tracea_amd import capi, ops
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a HIP device")
+    capi.init()
+
+    label, flops, bytes_, dtype, step = make_workload(args.workload, torch, ops)
+    wall, dev_s = time_steps(torch, step, args.steps, args.warmup)
+    tflops = flops / wall / 1e12
+    achieved = flops / dev_s / 1e12
+    line = {
+        "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOPS", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+        "data": "synthetic", "config": {"workload": label},
+        "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None,
+                     "hbm_GBps_algorithmic": round(bytes_ / dev_s / 1e9, 1)},
+    }
+    if not args.no_extras:
+        also = {}
+        for name in ("gemm", "conv", "attention", "attention_causal"):
+            if name == args.workload:
+                continue
+            lab, fl, by, dt, st = make_workload(name, torch, ops)
+            _, d = time_steps(torch, st, max(5, args.steps // 2), max(2, args.warmup // 2))
+            also[name] = {"workload": lab, "tflops": round(fl / d / 1e12, 2),
+                          "pct_of_peak": round(100.0 * fl / d / 1e12 / PEAK_TFLOPS, 2),
+                          "us_per_launch": round(d * 1e6, 2), "dtype": dt}
+        line["also"] = also
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

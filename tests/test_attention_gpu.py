@@ -1,0 +1,116 @@
+"""FlashAttention-2 forward parity on the GPU, through the C ABI, against the CPU
+oracle (naive softmax(QK^T)V in float64 on the bf16/f16-rounded inputs)."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_close_scaled, round_bf16, round_f16, tol_for_k
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, dtype):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda().to(dtype)
+
+
+def _inputs(b, h, s, d, seed, rnd):
+    rng = np.random.default_rng(seed)
+    return [rnd(rng.standard_normal((b, h, s, d))) for _ in range(3)]
+
+
+# output is a convex combination of V rows (|o| <= max|v| ~ 4): bf16 rounding of o alone is up
+# to 2^-8 * |o|.  Gate: tolerance with K = D for the half-precision products plus that rounding.
+def _tol(d, dtype):
+    return tol_for_k(d) + (2.0 ** -8 if dtype == "bf16" else 2.0 ** -11) * 2
+
+
+@pytest.mark.parametrize("variant", ["tr", "u16"])
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_small_and_edge_lengths(tracea_gpu, variant, d, dtype):
+    from tracea_amd import capi
+    tdt, rnd = (torch.bfloat16, round_bf16) if dtype == "bf16" else (torch.float16, round_f16)
+    name = "fa2_q128_kv64_d%d_%s" % (d, variant)
+    capi.force_variant("attention", name)
+    try:
+        # S in {16,77,123,1025}: tests/python/edge_case_fa2.py:56-71; 128/256: tile multiples
+        for (b, h, s) in [(1, 2, 16), (1, 2, 77), (2, 1, 123), (1, 2, 128), (2, 3, 256), (1, 1, 1025)]:
+            q, k, v = _inputs(b, h, s, d, 31 * s + d, rnd)
+            for causal in (False, True):
+                want = oracle.attention_bhsd(q, k, v, 1.0 / np.sqrt(d), causal)
+                got = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal)
+                assert_close_scaled(got.float().cpu().numpy(), want, _tol(d, dtype),
+                                    "%s S=%d causal=%s %s" % (name, s, causal, dtype))
+    finally:
+        capi.force_variant("attention", -1)
+
+
+def test_reference_gpu_check_shape(tracea_gpu):
+    # examples/verify_fa2_gpu.rs:67-162: B1 H4 S512 D64 causal, inputs U[0,0.2), tolerance 2e-3
+    rng = np.random.default_rng(42)
+    q, k, v = [round_f16(rng.uniform(0, 0.2, (1, 4, 512, 64))) for _ in range(3)]
+    want = oracle.attention_bhsd(q, k, v, 1.0 / 8.0, True)
+    got = tracea_gpu.attention(_dev(q, torch.float16), _dev(k, torch.float16), _dev(v, torch.float16), causal=True)
+    assert np.abs(got.float().cpu().numpy() - want).max() < 2e-3
+
+
+def test_invariants_on_device(tracea_gpu):
+    b, h, s, d = 1, 2, 320, 128
+    q, k, _ = _inputs(b, h, s, d, 5, round_bf16)
+    v = round_bf16(np.tile(np.linspace(-1, 1, d, dtype=np.float32), (b, h, s, 1)))
+    dq, dk, dv = [_dev(t, torch.bfloat16) for t in (q, k, v)]
+    for causal in (False, True):
+        o = tracea_gpu.attention(dq, dk, dv, causal=causal).float().cpu().numpy()
+        assert np.abs(o - v).max() <= 2.0 ** -8  # rows of P sum to one
+    q, k, v = _inputs(b, h, s, d, 6, round_bf16)
+    o = tracea_gpu.attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16), causal=True)
+    assert np.abs(o[0, :, 0].float().cpu().numpy() - v[0, :, 0]).max() <= 2.0 ** -7  # causal row 0 = V[0]
+    # explicit scale equals the default 1/sqrt(D)
+    o2 = tracea_gpu.attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16), causal=True,
+                              scale=1.0 / np.sqrt(d))
+    assert torch.equal(o, o2)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_config5_full_size_sampled(tracea_gpu, causal):
+    # B=4, H=32, S=4096, D=128 bf16, N(0,1).  The oracle evaluates 3 (batch, head) slices at 40
+    # sampled query rows each (first/last rows of tiles, random interior); every output element
+    # is also checked to be finite and within the range of V.
+    b, h, s, d = 4, 32, 4096, 128
+    g = torch.Generator(device="cuda").manual_seed(0x7ACEA006)
+    q = torch.randn(b, h, s, d, device="cuda", generator=g).bfloat16()
+    k = torch.randn(b, h, s, d, device="cuda", generator=g).bfloat16()
+    v = torch.randn(b, h, s, d, device="cuda", generator=g).bfloat16()
+    o = tracea_gpu.attention(q, k, v, causal=causal)
+    assert torch.isfinite(o.float()).all().item()
+    assert o.float().abs().max().item() <= v.float().abs().max().item() + 1e-3
+    rng = np.random.default_rng(3)
+    rows = np.unique(np.concatenate([[0, 1, 63, 64, 127, 128, 4032, 4095], rng.choice(s, 32, replace=False)])).astype(np.int32)
+    for (bi, hi) in [(0, 0), (1, 17), (3, 31)]:
+        want = oracle.attention(q[bi, hi].float().cpu().numpy(), k[bi, hi].float().cpu().numpy(),
+                                v[bi, hi].float().cpu().numpy(), 1.0 / np.sqrt(d), causal, rows=rows)
+        got = o[bi, hi].float().cpu().numpy()[rows]
+        assert_close_scaled(got, want, _tol(d, "bf16"), "configuration 5 slice (%d,%d) causal=%s" % (bi, hi, causal))
+
+
+def test_strided_views_and_error_paths(tracea_gpu):
+    from tracea_amd import capi
+    b, h, s, d = 2, 3, 96, 64
+    qkv = torch.randn(b, s, 3, h, d, device="cuda").half()   # packed projection layout
+    q, k, v = [qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)]  # [B,H,S,D] views, D contiguous
+    o = tracea_gpu.attention(q, k, v, causal=True)
+    want = oracle.attention_bhsd(*[t.float().cpu().numpy() for t in (q, k, v)], 1.0 / 8.0, True)
+    assert_close_scaled(o.float().cpu().numpy(), want, _tol(d, "f16"), "strided q/k/v")
+    bad = torch.zeros(1, 1, 8, 48, device="cuda", dtype=torch.float16)
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.attention(bad, bad, bad)
+    assert e.value.status == capi.UNSUPPORTED_CONFIG
+    f = torch.zeros(1, 1, 8, 64, device="cuda")
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.attention(f, f, f)
+    assert e.value.status == capi.UNSUPPORTED_CONFIG
+    a = torch.zeros(1, 1, 8, 64, device="cuda", dtype=torch.float16)
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.attention(a, a[:, :, :4], a)
+    assert e.value.status == capi.INVALID_PARAMS

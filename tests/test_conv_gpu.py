@@ -1,0 +1,205 @@
+"""Implicit-GEMM convolution parity on the GPU, through the C ABI, against the
+CPU oracle: coordinate tables bit for bit, values within 2e-2*sqrt(K)/sqrt(1024)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_close_scaled, round_f16, round_bf16, tol_for_k
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t.to(dtype) if dtype is not None else t
+
+
+COORD_SHAPES = [
+    (32, 56, 56, 64, 64, 3, 3, 1, 1, 1),
+    (32, 28, 28, 128, 128, 3, 3, 1, 1, 1),
+    (32, 56, 56, 64, 128, 3, 3, 2, 1, 1),
+    (32, 56, 56, 64, 128, 1, 1, 2, 0, 1),
+    (3, 9, 7, 24, 8, 5, 3, 2, 2, 1),
+]
+
+
+@pytest.mark.parametrize("shape", COORD_SHAPES)
+def test_coordinate_tables_bit_exact(tracea_gpu, shape):
+    from tracea_amd import capi
+    blk = capi.ConvParamsBlock()
+    assert capi.lib().tracea_conv_params_pack(*shape, C.byref(blk)) == capi.SUCCESS
+    ref = oracle.conv_params(*shape)
+    assert bytes(blk) == bytes(ref)
+    rows_ref, base_ref, cols_ref = oracle.conv_coords(ref)
+    m, k = rows_ref.shape[0], cols_ref.shape[0]
+    rows = torch.empty(m, 3, dtype=torch.int32, device="cuda")
+    base = torch.empty(m, dtype=torch.int64, device="cuda")
+    cols = torch.empty(k, 3, dtype=torch.int32, device="cuda")
+    st = capi.lib().tracea_conv_coords_device(C.byref(blk), rows.data_ptr(), base.data_ptr(), cols.data_ptr(), None)
+    assert st == capi.SUCCESS, capi.last_error()
+    torch.cuda.synchronize()
+    assert np.array_equal(rows.cpu().numpy(), rows_ref)
+    assert np.array_equal(base.cpu().numpy(), base_ref)
+    assert np.array_equal(cols.cpu().numpy(), cols_ref)
+
+
+SMALL = [  # n, h, w, c, k, r, s, stride, pad, dilation
+    (1, 8, 8, 32, 32, 3, 3, 1, 1, 1),   # examples/verify_conv2d.rs:52-60
+    (3, 14, 14, 64, 128, 3, 3, 2, 1, 1),
+    (2, 9, 7, 16, 24, 1, 1, 2, 0, 1),
+    (1, 12, 12, 8, 40, 5, 3, 1, 2, 1),
+    (2, 10, 10, 16, 16, 3, 3, 1, 2, 2),
+    (5, 7, 7, 72, 8, 3, 3, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("variant", range(7))
+def test_small_shapes_every_variant_both_filter_layouts(tracea_gpu, variant):
+    from tracea_amd import capi
+    names = capi.variants("conv2d")
+    if variant >= len(names):
+        pytest.skip("no such variant")
+    capi.force_variant("conv2d", variant)
+    try:
+        for shape in SMALL:
+            n, h, w, c, k, r, s, stride, pad, dil = shape
+            rng = np.random.default_rng(variant * 100 + h + c)
+            x = round_f16(rng.standard_normal((n, h, w, c)))
+            w_rsck = round_f16(rng.standard_normal((r, s, c, k)) * np.sqrt(2.0 / (r * s * c)))
+            bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+            acc = oracle.conv2d_nhwc(x, w_rsck, stride, pad, dil)
+            want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+            dx = _dev(x, torch.float16)
+            dw_rsck = _dev(w_rsck, torch.float16)
+            dw_krsc = dw_rsck.permute(3, 0, 1, 2).contiguous()
+            tol = tol_for_k(r * s * c)
+            y = tracea_gpu.conv2d(dx, dw_krsc, bias=_dev(bias), stride=stride, padding=pad, dilation=dil,
+                                  epilogue="bias+relu")
+            assert_close_scaled(y.float().cpu().numpy(), want, tol, "%s krsc %s" % (names[variant], shape))
+            y = tracea_gpu.conv2d(dx, dw_rsck, bias=_dev(bias), stride=stride, padding=pad, dilation=dil,
+                                  epilogue="bias+relu", weight_layout="rsck")
+            assert_close_scaled(y.float().cpu().numpy(), want, tol, "%s rsck %s" % (names[variant], shape))
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
+def test_asymmetric_stride_and_padding_bf16(tracea_gpu):
+    torch_f = torch.nn.functional
+    rng = np.random.default_rng(9)
+    x = round_bf16(rng.standard_normal((2, 11, 13, 16)))
+    wk = round_bf16(rng.standard_normal((24, 3, 5, 16)) * 0.1)
+    y = tracea_gpu.conv2d(_dev(x, torch.bfloat16), _dev(wk, torch.bfloat16), stride=(2, 1), padding=(1, 2))
+    ref = torch_f.conv2d(torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
+                         stride=(2, 1), padding=(1, 2)).permute(0, 2, 3, 1).numpy()
+    assert_close_scaled(y.float().cpu().numpy(), ref, tol_for_k(3 * 5 * 16), "asymmetric conv")
+
+
+def test_config3_full_size_bias_relu(tracea_gpu):
+    # N=32, 56x56x64 -> 64, 3x3 s1 p1, bias+ReLU; activations N(0,1), Kaiming weights, bias N(0,0.1)
+    rng = np.random.default_rng(0x7ACEA003)
+    x = round_f16(rng.standard_normal((32, 56, 56, 64)))
+    w_rsck = round_f16(rng.standard_normal((3, 3, 64, 64)) * np.sqrt(2.0 / 576))
+    bias = (rng.standard_normal(64) * 0.1).astype(np.float32)
+    acc = oracle.conv2d_nhwc(x, w_rsck, 1, 1)
+    want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+    dw = _dev(w_rsck, torch.float16).permute(3, 0, 1, 2).contiguous()
+    y = tracea_gpu.conv2d(_dev(x, torch.float16), dw, bias=_dev(bias), stride=1, padding=1, epilogue="bias+relu")
+    assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "configuration 3")
+
+
+def _bn_params(rng, ch):
+    gamma = rng.uniform(0.5, 1.5, ch).astype(np.float32)
+    beta = (rng.standard_normal(ch) * 0.1).astype(np.float32)
+    mean = (rng.standard_normal(ch) * 0.1).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, ch).astype(np.float32)
+    scale = (gamma / np.sqrt(var + 1e-5)).astype(np.float32)
+    shift = (beta - mean * scale).astype(np.float32)
+    return (gamma, beta, mean, var), (scale, shift)
+
+
+def test_config4_fused_basic_block(tracea_gpu):
+    # conv3x3+BN+ReLU -> conv3x3+BN+residual+ReLU, N=32, 128 channels, 28x28; fusion order of
+    # src/core/optimizer.rs:122-150 (BN producers gamma,beta,mean,var; then Add; then Relu).
+    from tracea_amd import capi
+    rng = np.random.default_rng(0x7ACEA004)
+    ch = 128
+    x = round_f16(rng.standard_normal((32, 28, 28, ch)))
+    w1 = round_f16(rng.standard_normal((3, 3, ch, ch)) * np.sqrt(2.0 / (9 * ch)))
+    w2 = round_f16(rng.standard_normal((3, 3, ch, ch)) * np.sqrt(2.0 / (9 * ch)))
+    bn1, fold1 = _bn_params(rng, ch)
+    bn2, fold2 = _bn_params(rng, ch)
+    # oracle: y1 stored in f16, as on the device
+    y1 = oracle.epilogue_apply(oracle.conv2d_nhwc(x, w1, 1, 1), [(oracle.EPI_SCALE_SHIFT,) + fold1, (oracle.EPI_RELU,)])
+    y1 = round_f16(y1)
+    y2 = oracle.epilogue_apply(oracle.conv2d_nhwc(y1, w2, 1, 1),
+                               [(oracle.EPI_SCALE_SHIFT,) + fold2, (oracle.EPI_RESIDUAL_ADD, x.reshape(-1, ch)), (oracle.EPI_RELU,)])
+    dx = _dev(x, torch.float16)
+    dw1 = _dev(w1, torch.float16).permute(3, 0, 1, 2).contiguous()
+    dw2 = _dev(w2, torch.float16).permute(3, 0, 1, 2).contiguous()
+    d1 = tracea_gpu.conv2d_ex(dx, dw1, [(capi.OP_SCALE_SHIFT, _dev(fold1[0]), _dev(fold1[1])), (capi.OP_RELU,)],
+                              stride=1, padding=1)
+    assert_close_scaled(d1.float().cpu().numpy(), y1, tol_for_k(9 * ch), "block conv1")
+    d2 = tracea_gpu.conv2d_ex(d1, dw2, [(capi.OP_SCALE_SHIFT, _dev(fold2[0]), _dev(fold2[1])),
+                                        (capi.OP_RESIDUAL_ADD, dx), (capi.OP_RELU,)], stride=1, padding=1)
+    assert_close_scaled(d2.float().cpu().numpy(), y2, 2 * tol_for_k(9 * ch), "block output")
+    # unfolded BatchNorm gives the same block output up to fp32 rounding of the fold
+    u1 = tracea_gpu.conv2d_ex(dx, dw1, [(capi.OP_BATCHNORM,) + tuple(_dev(t) for t in bn1) + (1e-5,), (capi.OP_RELU,)],
+                              stride=1, padding=1)
+    assert (u1.float() - d1.float()).abs().max().item() <= 2e-2
+
+
+def test_config4_downsample_block(tracea_gpu):
+    # 64ch 56x56 -> 128ch 28x28: conv3x3 s2 + BN + ReLU -> conv3x3 s1 + BN, shortcut conv1x1 s2 + BN, add, ReLU
+    from tracea_amd import capi
+    rng = np.random.default_rng(0x7ACEA005)
+    x = round_f16(rng.standard_normal((32, 56, 56, 64)))
+    w1 = round_f16(rng.standard_normal((3, 3, 64, 128)) * np.sqrt(2.0 / 576))
+    w2 = round_f16(rng.standard_normal((3, 3, 128, 128)) * np.sqrt(2.0 / 1152))
+    ws = round_f16(rng.standard_normal((1, 1, 64, 128)) * np.sqrt(2.0 / 64))
+    _, f1 = _bn_params(rng, 128)
+    _, f2 = _bn_params(rng, 128)
+    _, fs = _bn_params(rng, 128)
+    y1 = round_f16(oracle.epilogue_apply(oracle.conv2d_nhwc(x, w1, 2, 1), [(oracle.EPI_SCALE_SHIFT,) + f1, (oracle.EPI_RELU,)]))
+    sc = round_f16(oracle.epilogue_apply(oracle.conv2d_nhwc(x, ws, 2, 0), [(oracle.EPI_SCALE_SHIFT,) + fs]))
+    y2 = oracle.epilogue_apply(oracle.conv2d_nhwc(y1, w2, 1, 1),
+                               [(oracle.EPI_SCALE_SHIFT,) + f2, (oracle.EPI_RESIDUAL_ADD, sc.reshape(-1, 128)), (oracle.EPI_RELU,)])
+    dx = _dev(x, torch.float16)
+    k = lambda w: _dev(w, torch.float16).permute(3, 0, 1, 2).contiguous()
+    d1 = tracea_gpu.conv2d_ex(dx, k(w1), [(capi.OP_SCALE_SHIFT, _dev(f1[0]), _dev(f1[1])), (capi.OP_RELU,)], stride=2, padding=1)
+    ds = tracea_gpu.conv2d_ex(dx, k(ws), [(capi.OP_SCALE_SHIFT, _dev(fs[0]), _dev(fs[1]))], stride=2, padding=0)
+    d2 = tracea_gpu.conv2d_ex(d1, k(w2), [(capi.OP_SCALE_SHIFT, _dev(f2[0]), _dev(f2[1])), (capi.OP_RESIDUAL_ADD, ds), (capi.OP_RELU,)],
+                              stride=1, padding=1)
+    assert_close_scaled(d1.float().cpu().numpy(), y1, tol_for_k(576), "downsample conv1")
+    assert_close_scaled(ds.float().cpu().numpy(), sc, tol_for_k(64), "shortcut 1x1")
+    assert_close_scaled(d2.float().cpu().numpy(), y2, 2 * tol_for_k(1152), "downsample block output")
+
+
+def test_error_paths(tracea_gpu):
+    from tracea_amd import capi
+    x = torch.zeros(1, 8, 8, 16, device="cuda", dtype=torch.float16)
+    w = torch.zeros(8, 3, 3, 16, device="cuda", dtype=torch.float16)
+    out = torch.zeros(1, 8, 8, 8, device="cuda", dtype=torch.float16)
+
+    def call(xv, wv, ov, **kw):
+        p = dict(stride_h=1, stride_w=1, padding_h=1, padding_w=1, dilation_h=1, dilation_w=1, groups=1)
+        p.update(kw)
+        params = capi.Conv2dParams(p["stride_h"], p["stride_w"], p["padding_h"], p["padding_w"], p["dilation_h"],
+                                   p["dilation_w"], p["groups"], 0, None)
+        from tracea_amd.ops import _view
+        vx, vw, vo = _view(xv), _view(wv), _view(ov)
+        return capi.lib().tracea_conv2d(vx.c, vw.c, None, None, C.byref(vo.c), params)
+
+    assert call(x, w, out) == capi.SUCCESS
+    assert call(x, w, out, groups=2) == capi.UNSUPPORTED_CONFIG       # tracea-ffi/src/lib.rs:158-163
+    assert call(x, w, out, stride_h=0) == capi.INVALID_PARAMS
+    assert call(x[0], w, out) == capi.INVALID_PARAMS                  # rank 3
+    assert call(x.float(), w.float(), out) == capi.UNSUPPORTED_CONFIG  # fp32 conv
+    assert call(x, w, torch.zeros(1, 7, 8, 8, device="cuda", dtype=torch.float16)) == capi.INVALID_PARAMS
+    assert call(x.permute(0, 3, 1, 2).contiguous().permute(0, 2, 3, 1), w, out) == capi.UNSUPPORTED_CONFIG  # NCHW storage
+    x12 = torch.zeros(1, 8, 8, 12, device="cuda", dtype=torch.float16)
+    w12 = torch.zeros(8, 3, 3, 12, device="cuda", dtype=torch.float16)
+    assert call(x12, w12, out) == capi.UNSUPPORTED_CONFIG             # C % 8 != 0
+    assert "multiple of 8" in capi.last_error()

@@ -1,0 +1,178 @@
+"""GEMM parity on the GPU, through the C ABI, against the CPU oracle on the same
+seeded inputs.  Tolerance for half precision: 2e-2*sqrt(K)/sqrt(1024), scaled by
+max(1,|ref|); fp32: 1e-4 relative to the float64 product."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_close_scaled, round_bf16, round_f16, tol_for_k
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t.to(dtype) if dtype is not None else t
+
+
+def test_fp32_1024_matches_cpu_packed_path(tracea_gpu):
+    # configuration 1: M=N=K=1024, U[-1,1) from seed; the device result is compared with the
+    # restated gemm_cpu_packed (hero tiling) and with the float64 product
+    rng = np.random.default_rng(0x7ACEA001)
+    a = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    b = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    c = tracea_gpu.gemm(_dev(a), _dev(b)).cpu().numpy()
+    ref64 = oracle.gemm_f64(a, b)
+    assert np.abs(c - ref64).max() <= 1e-4 * np.abs(ref64).max()
+    packed = np.zeros((1024, 1024), np.float32)
+    oracle.gemm_cpu_packed(a, b, packed)
+    assert np.abs(c - packed).max() <= 2e-4 * np.abs(ref64).max()
+    # all-ones variant of examples/cpu_bench.rs: exactly K everywhere
+    ones = torch.ones(1024, 1024, device="cuda")
+    assert (tracea_gpu.gemm(ones, ones) == 1024).all().item()
+
+
+@pytest.mark.parametrize("shape", [(64, 64, 64), (100, 36, 52), (129, 257, 200), (5, 4, 8)])
+def test_fp32_edges_and_fallback(tracea_gpu, shape):
+    m, n, k = shape
+    rng = np.random.default_rng(m * 7 + n)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    c = tracea_gpu.gemm(_dev(a), _dev(b)).cpu().numpy()
+    ref = oracle.gemm_f64(a, b)
+    assert np.abs(c - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+
+
+def test_reference_known_answer_16cubed_f16(tracea_gpu):
+    # tests/numerical_parity.rs:62-151: the reference's only numeric GPU test, tolerance 5e-2
+    a = (np.arange(256, dtype=np.float32) * np.float32(0.05) - np.float32(0.4)).reshape(16, 16)
+    b = (np.arange(256, dtype=np.float32) * np.float32(0.02) - np.float32(0.1)).reshape(16, 16)
+    ref = oracle.gemm_f64(round_f16(a), round_f16(b))
+    c = tracea_gpu.gemm(_dev(a, torch.float16), _dev(b, torch.float16)).float().cpu().numpy()
+    assert np.abs(c - ref).max() < 5e-2
+
+
+HALF_SHAPES = [(256, 256, 128), (300, 200, 136), (512, 384, 1024), (64, 72, 8), (1000, 24, 72)]
+
+
+@pytest.mark.parametrize("variant", range(7))
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_half_every_variant_both_b_layouts(tracea_gpu, variant, dtype):
+    from tracea_amd import capi
+    names = capi.variants("gemm")
+    if variant >= len(names):
+        pytest.skip("no such variant")
+    tdt, rnd = (torch.float16, round_f16) if dtype == "f16" else (torch.bfloat16, round_bf16)
+    capi.force_variant("gemm", variant)
+    try:
+        for (m, n, k) in HALF_SHAPES:
+            rng = np.random.default_rng(1000 * variant + m + n + k)
+            a = rnd(rng.standard_normal((m, k)) / np.sqrt(k))
+            bt = rnd(rng.standard_normal((n, k)))          # column-major B: stored [N,K]
+            ref = oracle.gemm_f64(a, bt.T)
+            da, dbt = _dev(a, tdt), _dev(bt, tdt)
+            c = tracea_gpu.gemm(da, dbt.t()).float().cpu().numpy()
+            assert_close_scaled(c, ref, tol_for_k(k), "%s %s NT %s" % (names[variant], dtype, (m, n, k)))
+            c2 = tracea_gpu.gemm(da, dbt.t().contiguous()).float().cpu().numpy()  # row-major B [K,N]
+            assert_close_scaled(c2, ref, tol_for_k(k), "%s %s NN %s" % (names[variant], dtype, (m, n, k)))
+    finally:
+        capi.force_variant("gemm", -1)
+
+
+def test_epilogue_kinds_match_oracle_chain(tracea_gpu):
+    # operator order of src/interface/c_bindings.rs:144-197, functors of epilogue.cuh
+    m, n, k = 256, 320, 256
+    rng = np.random.default_rng(77)
+    a = round_f16(rng.standard_normal((m, k)) / np.sqrt(k))
+    bt = round_f16(rng.standard_normal((n, k)))
+    bias = rng.standard_normal(n).astype(np.float32)
+    res = round_f16(rng.standard_normal((m, n)))
+    acc = oracle.gemm_f64(a, bt.T).astype(np.float32)
+    da, dbt = _dev(a, torch.float16), _dev(bt, torch.float16)
+    dbias, dres = _dev(bias), _dev(res, torch.float16)
+    E = oracle
+    cases = {
+        "none": [],
+        "bias": [(E.EPI_BIAS_ADD, bias)],
+        "relu": [(E.EPI_RELU,)],
+        "gelu": [(E.EPI_GELU,)],
+        "silu": [(E.EPI_SILU,)],
+        "bias+relu": [(E.EPI_BIAS_ADD, bias), (E.EPI_RELU,)],
+        "bias+silu": [(E.EPI_BIAS_ADD_SILU, bias)],
+        "residual": [(E.EPI_RESIDUAL_ADD, res)],
+        "residual+relu": [(E.EPI_RESIDUAL_ADD, res), (E.EPI_RELU,)],
+    }
+    for name, chain in cases.items():
+        want = oracle.epilogue_apply(acc, chain)
+        got = tracea_gpu.gemm(da, dbt.t(), bias=dbias if "bias" in name else None,
+                              residual=dres if "residual" in name else None,
+                              epilogue=name).float().cpu().numpy()
+        assert_close_scaled(got, want, tol_for_k(k), "epilogue " + name)
+    # f16 bias and fp32 output
+    got = tracea_gpu.gemm(da, dbt.t(), bias=_dev(bias, torch.float16), epilogue="bias",
+                          out_dtype=torch.float32).cpu().numpy()
+    want = oracle.epilogue_apply(acc, [(E.EPI_BIAS_ADD, round_f16(bias))])
+    assert_close_scaled(got, want, 1e-3, "f16 bias, f32 out")
+
+
+def test_explicit_chain_with_batchnorm(tracea_gpu):
+    from tracea_amd import capi
+    m, n, k = 128, 64, 64
+    rng = np.random.default_rng(5)
+    a = round_f16(rng.standard_normal((m, k)) / np.sqrt(k))
+    bt = round_f16(rng.standard_normal((n, k)))
+    gamma = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    beta = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    mean = (rng.standard_normal(n) * 0.1).astype(np.float32)
+    var = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    acc = oracle.gemm_f64(a, bt.T).astype(np.float32)
+    want = oracle.epilogue_apply(acc, [(oracle.EPI_BATCHNORM, gamma, beta, mean, var, 1e-5), (oracle.EPI_RELU,)])
+    got = tracea_gpu.gemm_ex(_dev(a, torch.float16), _dev(bt, torch.float16).t(),
+                             [(capi.OP_BATCHNORM, _dev(gamma), _dev(beta), _dev(mean), _dev(var), 1e-5),
+                              (capi.OP_RELU,)]).float().cpu().numpy()
+    assert_close_scaled(got, want, tol_for_k(k), "BN+ReLU chain")
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096, 4096), (8192, 2048, 8192)])
+def test_full_size_fp16_sampled_rows_and_linearity(tracea_gpu, shape):
+    # configuration 2 at its real size: N(0,1)/sqrt(K) entries, A row-major, B column-major.
+    # 48 sampled rows are checked against the float64 oracle; the whole output is checked
+    # through linearity: gemm(A, B)[rows] == gemm(A[rows], B) bit for bit (same kernel, same
+    # per-row arithmetic) and gemm(2A, B) == 2 gemm(A, B) exactly (powers of two commute with rounding).
+    m, n, k = shape
+    g = torch.Generator(device="cuda").manual_seed(0x7ACEA002)
+    a = (torch.randn(m, k, device="cuda", generator=g) / k ** 0.5).half()
+    bt = (torch.randn(n, k, device="cuda", generator=g) / k ** 0.5).half()
+    c = tracea_gpu.gemm(a, bt.t())
+    rows = np.random.default_rng(1).choice(m, 48, replace=False)
+    ref = oracle.gemm_f64(a[rows].float().cpu().numpy(), bt.float().cpu().numpy().T)
+    assert_close_scaled(c[rows].float().cpu().numpy(), ref, tol_for_k(k), "sampled rows %s" % (shape,))
+    c2 = tracea_gpu.gemm(a * 2, bt.t())
+    assert torch.equal(c2, c * 2)
+    assert torch.isfinite(c.float()).all().item()
+
+
+def test_error_paths(tracea_gpu):
+    from tracea_amd import capi
+    a = torch.zeros(8, 8, device="cuda", dtype=torch.float16)
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.gemm(a, torch.zeros(16, 8, device="cuda", dtype=torch.float16))
+    assert e.value.status == capi.INVALID_PARAMS
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.gemm(a.int(), a.int(), out=a.int())
+    assert e.value.status == capi.UNSUPPORTED_CONFIG
+    host = torch.zeros(8, 8, dtype=torch.float16)
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.gemm(host, host, out=host.clone())
+    assert e.value.status == capi.CPU_ERROR
+    with pytest.raises(capi.TraceaError) as e:
+        tracea_gpu.gemm(a, a, bias=torch.zeros(7, device="cuda"), epilogue="bias")
+    assert e.value.status == capi.INVALID_PARAMS
+    # NULL data pointer
+    shape = (C.c_uint64 * 2)(8, 8)
+    tv = capi.TensorView(None, 2, shape, None, capi.F16, 0)
+    st = capi.lib().tracea_gemm(tv, tv, None, None, C.byref(tv), capi.GemmParams(0, None))
+    assert st == capi.INVALID_PARAMS

@@ -106,8 +106,14 @@ fa2_fwd_kernel(const AttentionArgs a) {
   //      K rows are swizzled for 32 lanes reading the same column of 32 rows;
   //      V rows are swizzled at 64-byte granularity for the transpose load,
   //      whose 32 lanes read a 64-byte window of 4 consecutive rows. ----
-  auto k_piece = [&](int row, int c) -> int { return row * ROW_BYTES + ((c ^ (row & (CH - 1))) << 4); };
-  auto v_piece = [&](int row, int c) -> int { return row * ROW_BYTES + ((c ^ ((row & 3) << 2)) << 4); };
+  constexpr int RP = 256 / ROW_BYTES > 0 ? 256 / ROW_BYTES : 1;  // rows per 256 bytes of LDS
+  constexpr int WIN = ROW_BYTES / 64;                            // 64-byte windows per row
+  auto k_piece = [&](int row, int c) -> int {
+    return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
+  };
+  auto v_piece = [&](int row, int c) -> int {
+    return row * ROW_BYTES + ((c ^ (((row / RP) % WIN) << 2)) << 4);
+  };
 
   const int ntiles_all = (S + FA_BKV - 1) / FA_BKV;
   int ntiles = ntiles_all;
