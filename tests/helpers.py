@@ -10,6 +10,13 @@ def tol_for_k(k):
     return 2e-2 * math.sqrt(k) / math.sqrt(1024.0)
 
 
+def tol_half(k, dtype):
+    """tol_for_k plus the rounding of the stored result itself (half a unit in the last place,
+    relative 2^-8 for bf16 and 2^-11 for f16), which no kernel can go below and which exceeds
+    the K-dependent term for very short reductions."""
+    return tol_for_k(k) + (2.0 ** -8 if dtype == "bf16" else 2.0 ** -11)
+
+
 def assert_close_scaled(got, ref, tol, what=""):
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import assert_close_scaled, round_f16, round_bf16, tol_for_k
+from helpers import assert_close_scaled, round_f16, round_bf16, tol_for_k, tol_half
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -75,7 +75,7 @@ def test_small_shapes_every_variant_both_filter_layouts(tracea_gpu, variant):
             dx = _dev(x, torch.float16)
             dw_rsck = _dev(w_rsck, torch.float16)
             dw_krsc = dw_rsck.permute(3, 0, 1, 2).contiguous()
-            tol = tol_for_k(r * s * c)
+            tol = tol_half(r * s * c, "f16")
             y = tracea_gpu.conv2d(dx, dw_krsc, bias=_dev(bias), stride=stride, padding=pad, dilation=dil,
                                   epilogue="bias+relu")
             assert_close_scaled(y.float().cpu().numpy(), want, tol, "%s krsc %s" % (names[variant], shape))
@@ -94,7 +94,7 @@ def test_asymmetric_stride_and_padding_bf16(tracea_gpu):
     y = tracea_gpu.conv2d(_dev(x, torch.bfloat16), _dev(wk, torch.bfloat16), stride=(2, 1), padding=(1, 2))
     ref = torch_f.conv2d(torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
                          stride=(2, 1), padding=(1, 2)).permute(0, 2, 3, 1).numpy()
-    assert_close_scaled(y.float().cpu().numpy(), ref, tol_for_k(3 * 5 * 16), "asymmetric conv")
+    assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(3 * 5 * 16, "bf16"), "asymmetric conv")
 
 
 def test_config3_full_size_bias_relu(tracea_gpu):

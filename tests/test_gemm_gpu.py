@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import oracle
-from helpers import assert_close_scaled, round_bf16, round_f16, tol_for_k
+from helpers import assert_close_scaled, round_bf16, round_f16, tol_for_k, tol_half
 
 torch = pytest.importorskip("torch")
 pytestmark = pytest.mark.gpu
@@ -52,7 +52,11 @@ def test_reference_known_answer_16cubed_f16(tracea_gpu):
     b = (np.arange(256, dtype=np.float32) * np.float32(0.02) - np.float32(0.1)).reshape(16, 16)
     ref = oracle.gemm_f64(round_f16(a), round_f16(b))
     c = tracea_gpu.gemm(_dev(a, torch.float16), _dev(b, torch.float16)).float().cpu().numpy()
-    assert np.abs(c - ref).max() < 5e-2
+    # entries reach ~500, where one f16 step is 0.25: the reference's absolute 5e-2 can only hold
+    # below 64; beyond that the f16 output rounding (relative 2^-11) is the floor
+    small = np.abs(ref) < 64
+    assert np.abs(c - ref)[small].max() < 5e-2
+    assert_close_scaled(c, ref, 2.0 ** -10, "16^3 known answer")
 
 
 HALF_SHAPES = [(256, 256, 128), (300, 200, 136), (512, 384, 1024), (64, 72, 8), (1000, 24, 72)]
@@ -75,9 +79,9 @@ def test_half_every_variant_both_b_layouts(tracea_gpu, variant, dtype):
             ref = oracle.gemm_f64(a, bt.T)
             da, dbt = _dev(a, tdt), _dev(bt, tdt)
             c = tracea_gpu.gemm(da, dbt.t()).float().cpu().numpy()
-            assert_close_scaled(c, ref, tol_for_k(k), "%s %s NT %s" % (names[variant], dtype, (m, n, k)))
+            assert_close_scaled(c, ref, tol_half(k, dtype), "%s %s NT %s" % (names[variant], dtype, (m, n, k)))
             c2 = tracea_gpu.gemm(da, dbt.t().contiguous()).float().cpu().numpy()  # row-major B [K,N]
-            assert_close_scaled(c2, ref, tol_for_k(k), "%s %s NN %s" % (names[variant], dtype, (m, n, k)))
+            assert_close_scaled(c2, ref, tol_half(k, dtype), "%s %s NN %s" % (names[variant], dtype, (m, n, k)))
     finally:
         capi.force_variant("gemm", -1)
 
@@ -151,7 +155,9 @@ def test_full_size_fp16_sampled_rows_and_linearity(tracea_gpu, shape):
     ref = oracle.gemm_f64(a[rows].float().cpu().numpy(), bt.float().cpu().numpy().T)
     assert_close_scaled(c[rows].float().cpu().numpy(), ref, tol_for_k(k), "sampled rows %s" % (shape,))
     c2 = tracea_gpu.gemm(a * 2, bt.t())
-    assert torch.equal(c2, c * 2)
+    normal = c.float().abs() >= 2.0 ** -13   # f16 rounding is scale-invariant only for normal numbers
+    assert torch.equal(c2[normal], (c * 2)[normal])
+    assert ((c2.float() - 2 * c.float()).abs() <= 2.0 ** -23).all().item()  # subnormal outputs: one step
     assert torch.isfinite(c.float()).all().item()
 
 
