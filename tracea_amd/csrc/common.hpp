@@ -61,7 +61,7 @@ struct AttentionArgs {
 struct ContractionVariant {
   const char *name;
   int bm, bn, bk, waves_m, waves_n, stages;
-  bool direct_to_lds;
+  int pipeline;  // 0: operands read just in time; 1: read one k-step ahead, across the barrier
   size_t lds_bytes;
   // launch: returns hipError_t as int
   int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);

@@ -254,8 +254,26 @@ __device__ __forceinline__ void tile_coordinates(const ContractionArgs &a, int &
   tile_n = in_group / rows;
 }
 
+// ---- instruction interleaving --------------------------------------------------
+// Emits a scheduling pipeline for the current region: kMfmas MFMAs, before each
+// of which the shares of kCountA instructions of class kClassA and kCountB of
+// class kClassB are placed (classes as __builtin_amdgcn_sched_group_barrier defines them:
+// 0x008 MFMA, 0x020 VMEM read, 0x100 LDS read, 0x200 LDS write).
+template <int kStep, int kMfmas, int kClassA, int kCountA, int kClassB, int kCountB>
+struct Interleave {
+  static __device__ __forceinline__ void run() {
+    constexpr int na = ((kStep + 1) * kCountA) / kMfmas - (kStep * kCountA) / kMfmas;
+    constexpr int nb = ((kStep + 1) * kCountB) / kMfmas - (kStep * kCountB) / kMfmas;
+    if constexpr (na > 0) __builtin_amdgcn_sched_group_barrier(kClassA, na, 0);
+    if constexpr (nb > 0) __builtin_amdgcn_sched_group_barrier(kClassB, nb, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (kStep + 1 < kMfmas)
+      Interleave<kStep + 1, kMfmas, kClassA, kCountA, kClassB, kCountB>::run();
+  }
+};
+
 // ---- the kernel -----------------------------------------------------------------
-template <int DT, int BM, int BN, int BK, int WM, int WN, bool CONV, bool B_NCONTIG>
+template <int DT, int BM, int BN, int BK, int WM, int WN, int PIPE, bool CONV, bool B_NCONTIG>
 __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const ContractionArgs args) {
   constexpr int NT = WM * WN * 64;
   constexpr int CH = BK / 8;       // 16-byte pieces per tile row
@@ -376,11 +394,16 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
   };
 
-  // Zero-masking of pieces is needed for a convolution (padding) and whenever
-  // the last K tile is partial; a GEMM whose K is a multiple of BK skips it.
-  const bool mask_a = CONV || (K % BK) != 0;
-  const bool mask_b = B_NCONTIG || (K % BK) != 0;
+  // Zero-masking of pieces is needed for a convolution (padding, K tail of
+  // R*S*C) and for a GEMM whose last K tile is partial.  The pipelined loop must
+  // stay free of branches (its instruction interleaving is per basic block), so
+  // there the decision is made at compile time: always for a convolution, never
+  // for a GEMM, and the dispatcher only picks a pipelined GEMM variant when K is
+  // a multiple of BK.
+  const bool mask_rt = (K % BK) != 0;
   auto stash = [&](unsigned char *sA, unsigned char *sB) {
+    const bool mask_a = PIPE != 0 ? CONV : (CONV || mask_rt);
+    const bool mask_b = PIPE != 0 ? CONV : (CONV || mask_rt);
     if (mask_a) {
 #pragma unroll
       for (int i = 0; i < NA; ++i)
@@ -450,22 +473,92 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   fetch(0);
   stash(smem, smem + A_STAGE);
   __syncthreads();
-  for (int kt = 0; kt + 1 < nk; ++kt) {
-    unsigned char *cur = smem + (kt & 1) * STAGE;
-    unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
-    // The scheduling fences keep the compiler from sinking the global loads
-    // below the MFMAs (towards their first use in stash), which would expose
-    // the whole memory latency once per K tile.
-    fetch((kt + 1) * BK);
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(cur, cur + A_STAGE);
-    __builtin_amdgcn_sched_barrier(0);
-    stash(nxt, nxt + A_STAGE);
-    __syncthreads();
-  }
-  {
-    const unsigned char *cur = smem + ((nk - 1) & 1) * STAGE;
-    multiply(cur, cur + A_STAGE);
+  if constexpr (PIPE == 0) {
+    // Plain form: operands are read from LDS just before the MFMAs that use them.
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+      unsigned char *cur = smem + (kt & 1) * STAGE;
+      unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
+      // The scheduling fences keep the compiler from sinking the global loads
+      // below the MFMAs (towards their first use in stash), which would expose
+      // the whole memory latency once per K tile.
+      fetch((kt + 1) * BK);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(cur, cur + A_STAGE);
+      __builtin_amdgcn_sched_barrier(0);
+      stash(nxt, nxt + A_STAGE);
+      __syncthreads();
+    }
+    {
+      const unsigned char *cur = smem + ((nk - 1) & 1) * STAGE;
+      multiply(cur, cur + A_STAGE);
+    }
+  } else {
+    // Software-pipelined form.  The operands of k-step s+1 are read from LDS
+    // while the MFMAs of k-step s run; the last k-step of a tile runs AFTER the
+    // barrier that publishes the next tile, overlapped with the reads of that
+    // tile's first operands, so the matrix pipe does not drain at the barrier.
+    // The global loads of the next tile are spread over the first k-step and
+    // the LDS writes that stage it over the one before the barrier.
+    constexpr int KS = BK / 16;
+    static_assert(KS >= 4 && KS % 2 == 0, "pipelined loop needs an even number (>= 4) of k-steps");
+    constexpr int R = FM * FN, D = FM + FN, L = NA + NB;
+    u32x4 fa[2][FM], fb[2][FN];
+    auto read_operands = [&](int set, const unsigned char *sA, const unsigned char *sB, int ks) {
+      const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
+      const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
+      const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+    };
+    auto mma = [&](int set) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(fb[set][j], fa[set][i], acc[i][j]);
+    };
+    read_operands(0, smem, smem + A_STAGE, 0);
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+      unsigned char *cur = smem + (kt & 1) * STAGE;
+      unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
+      // k-step 0: global loads of the next tile + operand reads of k-step 1
+      fetch((kt + 1) * BK);
+      read_operands(1, cur, cur + A_STAGE, 1);
+      mma(0);
+      Interleave<0, R, 0x020, L, 0x100, D>::run();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 1; ks + 2 < KS; ++ks) {
+        read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
+        mma(ks & 1);
+        Interleave<0, R, 0x100, D, 0x100, 0>::run();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // k-step KS-2: operand reads of the last k-step, then the LDS writes of the next tile
+      read_operands((KS - 1) & 1, cur, cur + A_STAGE, KS - 1);
+      stash(nxt, nxt + A_STAGE);
+      mma((KS - 2) & 1);
+      Interleave<0, R, 0x100, D, 0x200, (B_NCONTIG ? NA : L)>::run();
+      __builtin_amdgcn_sched_barrier(0);
+      __syncthreads();
+      // k-step KS-1 overlaps the first operand reads of the tile just published
+      read_operands(0, nxt, nxt + A_STAGE, 0);
+      mma((KS - 1) & 1);
+      Interleave<0, R, 0x100, D, 0x100, 0>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    {
+      const unsigned char *cur = smem + ((nk - 1) & 1) * STAGE;
+#pragma unroll
+      for (int ks = 0; ks + 1 < KS; ++ks) {
+        read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
+        mma(ks & 1);
+        Interleave<0, R, 0x100, D, 0x100, 0>::run();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma((KS - 1) & 1);
+    }
   }
   __syncthreads();
 
@@ -513,14 +606,14 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   }
 }
 
-template <int BM, int BN, int BK, int WM, int WN>
+template <int BM, int BN, int BK, int WM, int WN, int PIPE>
 int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
                        hipStream_t stream) {
   constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * 2;
   const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \
-    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, CONVV, NCV>;                      \
+    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, PIPE, CONVV, NCV>;                      \
     static bool attr_done = false;                                                           \
     if (!attr_done) {                                                                        \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                  \

@@ -1,6 +1,6 @@
 // One member of the contraction kernel family per translation unit; the build
 // compiles this file once per line of contraction_variants.def with
-// -DV_NAME=... -DV_BM=... -DV_BN=... -DV_BK=... -DV_WM=... -DV_WN=... -DV_STAGES=... -DV_DIRECT=...
+// -DV_NAME=... -DV_BM=... -DV_BN=... -DV_BK=... -DV_WM=... -DV_WN=... -DV_STAGES=... -DV_DIRECT=<pipeline mode>
 #include "contraction_kernel.hpp"
 
 #define TRACEA_CAT2(a, b) a##b
@@ -12,9 +12,9 @@ namespace tracea_amd {
 // Host-side accessor (a function, so that nothing here is emitted for the device).
 const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
   static const ContractionVariant v = {
-      TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT != 0,
+      TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT,
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
-      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN>};
+      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_DIRECT>};
   return v;
 }
 }  // namespace tracea_amd

@@ -353,6 +353,20 @@ int pick_contraction(const char *op, const std::string &cache_key, int m, int n,
   return select_contraction_variant(m, n, k, conv);
 }
 
+// The non-pipelined variant of the same tile shape (or the first plain variant).
+int plain_twin(int vi) {
+  const ContractionVariant &p = contraction_variant(vi);
+  int first_plain = -1;
+  for (int i = 0; i < contraction_variant_count(); ++i) {
+    const ContractionVariant &v = contraction_variant(i);
+    if (v.pipeline != 0) continue;
+    if (first_plain < 0) first_plain = i;
+    if (v.bm == p.bm && v.bn == p.bn && v.bk == p.bk && v.waves_m == p.waves_m && v.waves_n == p.waves_n)
+      return i;
+  }
+  return first_plain;
+}
+
 void fill_grid(ContractionArgs *a, const ContractionVariant &v) {
   a->grid_m = (a->M + v.bm - 1) / v.bm;
   a->grid_n = (a->N + v.bn - 1) / v.bn;
@@ -386,8 +400,11 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.epi = chain;
       char key[160];
       snprintf(key, sizeof(key), "gemm_%lld_%lld_%lld_%s", M, N, K, tuning_device_name());
-      const int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false);
+      int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false);
       if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "gemm: no kernel variant available");
+      // a pipelined GEMM variant has no K-tail masking: fall back to its plain twin
+      if (contraction_variant(vi).pipeline != 0 && K % contraction_variant(vi).bk != 0)
+        vi = plain_twin(vi);
       const ContractionVariant &v = contraction_variant(vi);
       fill_grid(&args, v);
       return hip_status("gemm launch", v.launch(args, false, a.dtype, !b_kcontig, stream));

@@ -129,7 +129,7 @@ PipelineConfig config_for_contraction_variant(int index) {
   c.intrinsic_shape = "M32N32K2";
   c.gemm_variant = "Simd";
   c.double_buffer = true;
-  c.cp_async_distance = v.direct_to_lds ? 1 : 0;
+  c.cp_async_distance = (uint32_t)v.pipeline;  // operand prefetch distance in k-steps
   c.bank_conflict_padding = 0;
   return c;
 }
@@ -141,7 +141,7 @@ int contraction_variant_for_config(const PipelineConfig &c) {
     if ((uint32_t)v.stages != c.num_stages) continue;
     if (c.has_force_num_warps && (uint32_t)(v.waves_m * v.waves_n) != c.force_num_warps) continue;
     if (c.micro_m > 1 && (uint32_t)(v.bm / v.waves_m) != c.micro_m) continue;
-    if ((c.cp_async_distance != 0) != v.direct_to_lds) continue;
+    if (c.cp_async_distance != (uint32_t)v.pipeline) continue;
     return i;
   }
   return -1;
