@@ -14,15 +14,19 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-CSRC = os.path.join(HERE, "csrc")
-OBJ = os.path.join(HERE, "_obj")
-LIB_DIR = os.path.join(HERE, "lib")
+# TRACEA_BUILD_CSRC / TRACEA_BUILD_OUT redirect the build to another source tree / output
+# directory (kernel experiments); by default everything stays inside the package.
+CSRC = os.environ.get("TRACEA_BUILD_CSRC") or os.path.join(HERE, "csrc")
+_OUT = os.environ.get("TRACEA_BUILD_OUT") or HERE
+OBJ = os.path.join(_OUT, "_obj")
+LIB_DIR = os.path.join(_OUT, "lib")
 LIB = os.path.join(LIB_DIR, "libtracea.so")
 
 ARCH = "gfx950"
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
+INCLUDE = os.path.normpath(os.path.join(HERE, "..", "include"))
+COMMON = ["-I" + INCLUDE, "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
           "-Wno-pass-failed"]
 
 HOST_SOURCES = ["abi.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
@@ -52,7 +56,7 @@ def _headers_digest():
         for fn in sorted(files):
             if fn.endswith((".hpp", ".h", ".def")):
                 h.update(open(os.path.join(root, fn), "rb").read())
-    h.update(open(os.path.join(HERE, "..", "include", "tracea.h"), "rb").read())
+    h.update(open(os.path.join(INCLUDE, "tracea.h"), "rb").read())
     return h.hexdigest()
 
 

@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libtracea.so")
+# TRACEA_LIB points at another build of the same library (kernel experiments).
+LIB_PATH = os.environ.get("TRACEA_LIB") or os.path.join(_HERE, "lib", "libtracea.so")
 
 # TraceaStatus
 SUCCESS, INVALID_PARAMS, UNSUPPORTED_CONFIG, CUDA_ERROR, CPU_ERROR, UNKNOWN_ERROR = 0, 1, 2, 3, 4, 99

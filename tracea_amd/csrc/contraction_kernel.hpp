@@ -305,6 +305,13 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   const int pc = tid % CH;      // 16-byte column of every A piece of this thread
   const int prow = tid / CH;    // first tile row; piece i is prow + i*(NT/CH)
   constexpr int PR_STEP = NT / CH;
+  // PIPE 2 moves tiles with loads that write LDS directly: a wave instruction
+  // fills 1024 contiguous bytes, lane l at byte 16*l, so the LDS position of a
+  // piece is fixed (row tid/CH + i*PR_STEP, 16-byte column tid%CH) and the
+  // swizzle is applied to the GLOBAL column instead.  PR_STEP is a multiple of
+  // RP*CH, hence the swizzle term is the same for all pieces of a thread.
+  static_assert(PIPE != 2 || (PR_STEP % (RP * CH) == 0 && !B_NCONTIG), "bad shape for direct-to-LDS loads");
+  const int gpc = PIPE == 2 ? (pc ^ ((prow / RP) & (CH - 1))) : pc;
 
   const unsigned short *Ag = (const unsigned short *)args.A;
   const unsigned short *Bg = (const unsigned short *)args.B;
@@ -350,7 +357,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   unsigned a_ok = 0, b_ok = 0;  // bit i: piece i holds real data
   auto fetch = [&](int k0) {
-    const int kg = k0 + pc * 8;
+    const int kg = k0 + gpc * 8;
     const bool kvalid = kg < K;
     const int k0c = kvalid ? kg : 0;  // column of this thread's piece, or a safe one
     a_ok = 0;
@@ -387,6 +394,54 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         rb[i] = *(const u32x4 *)(Bg + (ok ? (long long)(k0 + kk) * args.ldb + n : 0ll));
         b_ok |= ok ? (1u << i) : 0u;
       }
+    }
+  };
+
+  // Direct-to-LDS tile load (PIPE 2).  Pieces that must read as zero (padding,
+  // rows of K beyond the end) are fetched from a small all-zero device buffer.
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  // Only pieces lo <= index < hi of the thread's list (A pieces first, then B)
+  // are requested, so that the requests of one tile can be spread over several
+  // k-steps: the L1 data path takes 16 cycles per 1 KB instruction, and a burst
+  // of all waves' requests right after the barrier would stall instruction issue.
+  auto dma = [&](unsigned char *sA, unsigned char *sB, int k0, int lo, int hi) {
+    constexpr int RPI = 64 / CH;  // tile rows one wave instruction covers
+    const int kg = k0 + gpc * 8;
+    const bool kvalid = kg < K;
+    // masked pieces read the zero page, addressed relative to the operand's own
+    // base so that each piece stays a single load instruction
+    const long long a_zero = (const unsigned short *)args.zeros - Ag;
+    const long long b_zero = (const unsigned short *)args.zeros - Bg;
+    int dh = 0, dw = 0, ci = 0;
+    if constexpr (CONV) {
+      int rf, rem, sf;
+      fast_divmod(kg, args.sc_m, args.sc_s, args.s_sz * args.c_in, rf, rem);
+      fast_divmod(rem, args.c_m, args.c_s, args.c_in, sf, ci);
+      dh = rf * args.dil_h;
+      dw = sf * args.dil_w;
+    }
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+      if (i < lo || i >= hi) continue;
+      const unsigned short *src;
+      if constexpr (CONV) {
+        const int hi = a_hb[i] + dh, wi = a_wb[i] + dw;
+        const bool ok = kvalid && hi >= 0 && hi < args.h_in && wi >= 0 && wi < args.w_in;
+        src = Ag + (ok ? a_off[i] + ((long long)hi * args.w_in + wi) * args.c_in + ci : a_zero);
+      } else {
+        src = Ag + (kvalid ? a_off[i] + kg : a_zero);
+      }
+      unsigned char *dst = sA + (i * PR_STEP + wave_u * RPI) * ROW_BYTES;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                       (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < NB; ++i) {
+      if (NA + i < lo || NA + i >= hi) continue;
+      const unsigned short *src = Bg + (kvalid ? b_off[i] + kg : b_zero);
+      unsigned char *dst = sB + (i * PR_STEP + wave_u * RPI) * ROW_BYTES;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                       (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
     }
   };
 
@@ -467,12 +522,14 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     }
   };
 
-  // ---- main loop: two LDS stages, register-staged prefetch ----
+  // ---- main loop: two LDS stages ----
   static_assert(NA <= 32 && NB <= 32, "piece masks are 32 bits");
   const int nk = (K + BK - 1) / BK;
-  fetch(0);
-  stash(smem, smem + A_STAGE);
-  __syncthreads();
+  if constexpr (PIPE != 2) {
+    fetch(0);
+    stash(smem, smem + A_STAGE);
+    __syncthreads();
+  }
   if constexpr (PIPE == 0) {
     // Plain form: operands are read from LDS just before the MFMAs that use them.
     for (int kt = 0; kt + 1 < nk; ++kt) {
@@ -492,13 +549,15 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       const unsigned char *cur = smem + ((nk - 1) & 1) * STAGE;
       multiply(cur, cur + A_STAGE);
     }
-  } else {
+  } else if constexpr (PIPE == 1) {
     // Software-pipelined form.  The operands of k-step s+1 are read from LDS
     // while the MFMAs of k-step s run; the last k-step of a tile runs AFTER the
     // barrier that publishes the next tile, overlapped with the reads of that
     // tile's first operands, so the matrix pipe does not drain at the barrier.
-    // The global loads of the next tile are spread over the first k-step and
-    // the LDS writes that stage it over the one before the barrier.
+    // Global loads run a whole tile ahead: they are issued right after the
+    // barrier (when the staging registers have just been written to LDS) and
+    // consumed by the LDS writes spread over the last k-step before the next
+    // barrier.
     constexpr int KS = BK / 16;
     static_assert(KS >= 4 && KS % 2 == 0, "pipelined loop needs an even number (>= 4) of k-steps");
     constexpr int R = FM * FN, D = FM + FN, L = NA + NB;
@@ -519,33 +578,33 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(fb[set][j], fa[set][i], acc[i][j]);
     };
     read_operands(0, smem, smem + A_STAGE, 0);
+    if (nk > 1) fetch(BK);  // tile 1 travels while tile 0 is multiplied
     for (int kt = 0; kt + 1 < nk; ++kt) {
       unsigned char *cur = smem + (kt & 1) * STAGE;
       unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
-      // k-step 0: global loads of the next tile + operand reads of k-step 1
-      fetch((kt + 1) * BK);
-      read_operands(1, cur, cur + A_STAGE, 1);
-      mma(0);
-      Interleave<0, R, 0x020, L, 0x100, D>::run();
-      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int ks = 1; ks + 2 < KS; ++ks) {
+      for (int ks = 0; ks + 2 < KS; ++ks) {
         read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
         mma(ks & 1);
         Interleave<0, R, 0x100, D, 0x100, 0>::run();
         __builtin_amdgcn_sched_barrier(0);
       }
-      // k-step KS-2: operand reads of the last k-step, then the LDS writes of the next tile
+      // k-step KS-2: operand reads of the last k-step, and the LDS writes that
+      // stage the next tile (its global loads were issued a whole tile earlier)
       read_operands((KS - 1) & 1, cur, cur + A_STAGE, KS - 1);
       stash(nxt, nxt + A_STAGE);
       mma((KS - 2) & 1);
       Interleave<0, R, 0x100, D, 0x200, (B_NCONTIG ? NA : L)>::run();
       __builtin_amdgcn_sched_barrier(0);
       __syncthreads();
-      // k-step KS-1 overlaps the first operand reads of the tile just published
+      // k-step KS-1, after the barrier: first operand reads of the tile just
+      // published and the global loads of the tile after it (the staging
+      // registers are free again); clamped to the last tile, whose reload is
+      // never written to LDS
+      fetch((kt + 2 < nk ? kt + 2 : nk - 1) * BK);
       read_operands(0, nxt, nxt + A_STAGE, 0);
       mma((KS - 1) & 1);
-      Interleave<0, R, 0x100, D, 0x100, 0>::run();
+      Interleave<0, R, 0x020, L, 0x100, D>::run();
       __builtin_amdgcn_sched_barrier(0);
     }
     {
@@ -559,6 +618,83 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       }
       mma((KS - 1) & 1);
     }
+  } else {
+    // Software-pipelined form with direct-to-LDS loads: no staging registers and
+    // no LDS write instructions.  A tile is requested right after the barrier
+    // that frees its buffer, a whole tile of MFMAs before the barrier that
+    // publishes it; the only wait on global memory is the one in front of that
+    // barrier.
+    constexpr int KS = BK / 16;
+    static_assert(KS >= 2 && KS % 2 == 0, "pipelined loop needs an even number of k-steps");
+    constexpr int R = FM * FN, D = FM + FN, L = NA + NB;
+    u32x4 fa[2][FM], fb[2][FN];
+    auto read_operands = [&](int set, const unsigned char *sA, const unsigned char *sB, int ks) {
+      const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
+      const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
+      const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+    };
+    auto mma = [&](int set) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(fb[set][j], fa[set][i], acc[i][j]);
+    };
+    // The L requests of a tile are issued in SPREAD consecutive k-step regions,
+    // the first of which is the one right after the barrier that freed the
+    // destination buffer; the rest follow at the start of the next tile.
+    constexpr int SPREAD = 2;  // three shares measured no better than two
+    constexpr int CUT1 = L / SPREAD, CUT2 = SPREAD == 3 ? 2 * L / SPREAD : L;
+    dma(smem, smem + A_STAGE, 0, 0, L);
+    dma(smem + STAGE, smem + STAGE + A_STAGE, nk > 1 ? BK : 0, 0, CUT1);  // first share of tile 1
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile 0 is in LDS
+    __syncthreads();
+    read_operands(0, smem, smem + A_STAGE, 0);
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+      unsigned char *cur = smem + (kt & 1) * STAGE;
+      unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
+      // k-step 0 carries the second share of tile kt+1 (its first share was
+      // requested right after the previous barrier, or in the prologue)
+      dma(nxt, nxt + A_STAGE, (kt + 1) * BK, CUT1, CUT2);
+      read_operands(1, cur, cur + A_STAGE, 1);
+      mma(0);
+      Interleave<0, R, 0x020, CUT2 - CUT1, 0x100, D>::run();
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int ks = 1; ks + 1 < KS; ++ks) {
+        if (ks == 1) dma(nxt, nxt + A_STAGE, (kt + 1) * BK, CUT2, L);  // third share, if any
+        read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
+        mma(ks & 1);
+        if (ks == 1) Interleave<0, R, 0x020, L - CUT2, 0x100, D>::run();
+        else Interleave<0, R, 0x100, D, 0x100, 0>::run();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): tile kt+1 has landed
+      __syncthreads();
+      // every wave has finished reading `cur`: request the first share of tile
+      // kt+2 into it (clamped to the last tile, whose second copy is never read)
+      // while the last k-step of tile kt runs from registers
+      dma(cur, cur + A_STAGE, (kt + 2 < nk ? kt + 2 : nk - 1) * BK, 0, CUT1);
+      read_operands(0, nxt, nxt + A_STAGE, 0);
+      mma((KS - 1) & 1);
+      Interleave<0, R, 0x020, CUT1, 0x100, D>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    {
+      const unsigned char *cur = smem + ((nk - 1) & 1) * STAGE;
+#pragma unroll
+      for (int ks = 0; ks + 1 < KS; ++ks) {
+        read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
+        mma(ks & 1);
+        Interleave<0, R, 0x100, D, 0x100, 0>::run();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma((KS - 1) & 1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the clamped reload must not land on the epilogue staging
   }
   __syncthreads();
 
@@ -584,7 +720,12 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
                    acc[i][j][g * 4 + 3]};
         *(f32x4 *)(stage + lrow * EP_PITCH + j * 32 + g * 8 + lhalf * 4) = v;
       }
-    __syncthreads();
+    // The staging area is private to the wave and a wave's LDS operations
+    // complete in program order: a compiler-level fence is all that is needed
+    // between the writes above and the reads below (and before the next pass
+    // overwrites what this one reads).
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     for (int r = er; r < 32; r += RPI) {
       const int m = m0 + wm * TM + i * 32 + r;
       const int n = n0 + wn * TN + ec;
@@ -602,7 +743,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         store_from_float<8>(args.C, args.out_dtype, (long long)m * args.ldc + n, nvalid, v);
       }
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -624,7 +766,16 @@ int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_nc
     hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                    \
     return (int)hipGetLastError();                                                           \
   } while (0)
-  if (dtype == DT_F16) {
+  if constexpr (PIPE == 2) {
+    // direct-to-LDS loads cannot transpose: K-contiguous B only (the dispatcher
+    // routes an N-contiguous B to the register-staged twin)
+    if (b_ncontig) return (int)hipErrorInvalidValue;
+    if (dtype == DT_F16) {
+      if (conv) TRACEA_LAUNCH(DT_F16, true, false); else TRACEA_LAUNCH(DT_F16, false, false);
+    } else {
+      if (conv) TRACEA_LAUNCH(DT_BF16, true, false); else TRACEA_LAUNCH(DT_BF16, false, false);
+    }
+  } else if (dtype == DT_F16) {
     if (conv) { if (b_ncontig) TRACEA_LAUNCH(DT_F16, true, true); else TRACEA_LAUNCH(DT_F16, true, false); }
     else      { if (b_ncontig) TRACEA_LAUNCH(DT_F16, false, true); else TRACEA_LAUNCH(DT_F16, false, false); }
   } else {
