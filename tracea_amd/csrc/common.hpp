@@ -36,7 +36,7 @@ struct ContractionArgs {
   long long ldb;       // B: stride between consecutive n (K-contiguous B) or k (N-contiguous B)
   long long ldc;       // C row stride, elements
   int out_dtype;       // DataType of C
-  const void *zeros;   // >= 16 bytes of zeros in device memory (source of masked direct-to-LDS loads)
+  unsigned a_bytes, b_bytes;  // extent of A and B in bytes (bounds of the direct-to-LDS buffer loads)
   int grid_m, grid_n;  // tiles along M and N
   int group_m;         // tile-order group height
   // convolution geometry (ConvParams of the reference, h/w split)
@@ -63,7 +63,8 @@ struct ContractionVariant {
   const char *name;
   int bm, bn, bk, waves_m, waves_n, stages;
   int pipeline;  // 0: operands read just in time; 1: read one k-step ahead, across the barrier;
-                 // 2: as 1, with direct-to-LDS tile loads (K-contiguous B only)
+                 // 2: as 1, with direct-to-LDS tile loads (K-contiguous B only);
+                 // 3: ring of `stages` LDS buffers, direct-to-LDS loads stages-1 tiles ahead
   size_t lds_bytes;
   // launch: returns hipError_t as int
   int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);

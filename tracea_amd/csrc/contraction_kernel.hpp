@@ -273,7 +273,7 @@ struct Interleave {
 };
 
 // ---- the kernel -----------------------------------------------------------------
-template <int DT, int BM, int BN, int BK, int WM, int WN, int PIPE, bool CONV, bool B_NCONTIG>
+template <int DT, int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, bool CONV, bool B_NCONTIG>
 __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const ContractionArgs args) {
   constexpr int NT = WM * WN * 64;
   constexpr int CH = BK / 8;       // 16-byte pieces per tile row
@@ -310,8 +310,9 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // piece is fixed (row tid/CH + i*PR_STEP, 16-byte column tid%CH) and the
   // swizzle is applied to the GLOBAL column instead.  PR_STEP is a multiple of
   // RP*CH, hence the swizzle term is the same for all pieces of a thread.
-  static_assert(PIPE != 2 || (PR_STEP % (RP * CH) == 0 && !B_NCONTIG), "bad shape for direct-to-LDS loads");
-  const int gpc = PIPE == 2 ? (pc ^ ((prow / RP) & (CH - 1))) : pc;
+  static_assert(PIPE < 2 || (PR_STEP % (RP * CH) == 0 && !B_NCONTIG), "bad shape for direct-to-LDS loads");
+  static_assert(PIPE == 3 ? NS >= 3 : NS == 2, "stage count does not fit the pipeline mode");
+  const int gpc = PIPE >= 2 ? (pc ^ ((prow / RP) & (CH - 1))) : pc;
 
   const unsigned short *Ag = (const unsigned short *)args.A;
   const unsigned short *Bg = (const unsigned short *)args.B;
@@ -397,21 +398,35 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     }
   };
 
-  // Direct-to-LDS tile load (PIPE 2).  Pieces that must read as zero (padding,
-  // rows of K beyond the end) are fetched from a small all-zero device buffer.
+  // Direct-to-LDS tile load (PIPE >= 2) through buffer addressing: the address
+  // of a piece is (buffer base) + (per-lane 32-bit byte offset) + (scalar byte
+  // offset of the K tile).  For a GEMM the per-lane offsets never change, so a
+  // request costs one M0 update and one instruction, no vector ALU work.  A
+  // per-lane offset at or beyond the buffer size makes the hardware return
+  // zeros: pieces that must read as zero (padding, columns of K beyond the end)
+  // get the offset 0x80000000 (the dispatcher only selects these variants for
+  // operands smaller than 2 GiB).
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  constexpr unsigned OOB = 0x80000000u;
+  __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)args.A, 0, (int)args.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)args.B, 0, (int)args.b_bytes, 0x00020000);
+  unsigned a_voff[NA], b_voff[NB];
+  if constexpr (PIPE >= 2) {
+#pragma unroll
+    for (int i = 0; i < NA; ++i)
+      a_voff[i] = CONV ? (unsigned)(a_off[i] * 2) : (unsigned)((a_off[i] + gpc * 8) * 2);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) b_voff[i] = (unsigned)((b_off[i] + gpc * 8) * 2);
+  }
   // Only pieces lo <= index < hi of the thread's list (A pieces first, then B)
   // are requested, so that the requests of one tile can be spread over several
-  // k-steps: the L1 data path takes 16 cycles per 1 KB instruction, and a burst
-  // of all waves' requests right after the barrier would stall instruction issue.
+  // k-steps.
   auto dma = [&](unsigned char *sA, unsigned char *sB, int k0, int lo, int hi) {
     constexpr int RPI = 64 / CH;  // tile rows one wave instruction covers
     const int kg = k0 + gpc * 8;
     const bool kvalid = kg < K;
-    // masked pieces read the zero page, addressed relative to the operand's own
-    // base so that each piece stays a single load instruction
-    const long long a_zero = (const unsigned short *)args.zeros - Ag;
-    const long long b_zero = (const unsigned short *)args.zeros - Bg;
     int dh = 0, dw = 0, ci = 0;
     if constexpr (CONV) {
       int rf, rem, sf;
@@ -423,25 +438,28 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
       if (i < lo || i >= hi) continue;
-      const unsigned short *src;
+      unsigned voff;
+      int soff;
       if constexpr (CONV) {
-        const int hi = a_hb[i] + dh, wi = a_wb[i] + dw;
-        const bool ok = kvalid && hi >= 0 && hi < args.h_in && wi >= 0 && wi < args.w_in;
-        src = Ag + (ok ? a_off[i] + ((long long)hi * args.w_in + wi) * args.c_in + ci : a_zero);
+        const int hi_ = a_hb[i] + dh, wi = a_wb[i] + dw;
+        const bool ok = kvalid && hi_ >= 0 && hi_ < args.h_in && wi >= 0 && wi < args.w_in;
+        voff = ok ? a_voff[i] + (unsigned)(((hi_ * args.w_in + wi) * args.c_in + ci) * 2) : OOB;
+        soff = 0;
       } else {
-        src = Ag + (kvalid ? a_off[i] + kg : a_zero);
+        voff = kvalid ? a_voff[i] : OOB;
+        soff = k0 * 2;
       }
       unsigned char *dst = sA + (i * PR_STEP + wave_u * RPI) * ROW_BYTES;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                       (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void *)dst, 16,
+                                               (int)voff, soff, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       if (NA + i < lo || NA + i >= hi) continue;
-      const unsigned short *src = Bg + (kvalid ? b_off[i] + kg : b_zero);
+      const unsigned voff = kvalid ? b_voff[i] : OOB;
       unsigned char *dst = sB + (i * PR_STEP + wave_u * RPI) * ROW_BYTES;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
-                                       (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16,
+                                               (int)voff, k0 * 2, 0, 0);
     }
   };
 
@@ -525,7 +543,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // ---- main loop: two LDS stages ----
   static_assert(NA <= 32 && NB <= 32, "piece masks are 32 bits");
   const int nk = (K + BK - 1) / BK;
-  if constexpr (PIPE != 2) {
+  if constexpr (PIPE < 2) {
     fetch(0);
     stash(smem, smem + A_STAGE);
     __syncthreads();
@@ -618,7 +636,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       }
       mma((KS - 1) & 1);
     }
-  } else {
+  } else if constexpr (PIPE == 2) {
     // Software-pipelined form with direct-to-LDS loads: no staging registers and
     // no LDS write instructions.  A tile is requested right after the barrier
     // that frees its buffer, a whole tile of MFMAs before the barrier that
@@ -695,6 +713,86 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       mma((KS - 1) & 1);
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // the clamped reload must not land on the epilogue staging
+  } else {
+    // Ring of NS >= 3 LDS stages filled by direct-to-LDS loads.  Global-memory
+    // latency on this part is of the order of a whole K tile of a 256x256x64
+    // block and of several tiles of a smaller one, so one tile of look-ahead
+    // cannot hide it: here tile t+NS-1 is requested while tile t is multiplied
+    // (its buffer held tile t-1 and was released by the previous barrier), and
+    // waited for NS-2 barriers later.  The requests of a tile are spread evenly
+    // over the k-steps of the tile that overlaps them.
+    constexpr int KS = BK / 16;
+    static_assert(KS >= 2 && KS % 2 == 0, "pipelined loop needs an even number of k-steps");
+    constexpr int R = FM * FN, D = FM + FN, L = NA + NB;
+    constexpr int LAST_SHARE = L - ((KS - 1) * L) / KS;          // pieces issued after the barrier
+    constexpr int IN_FLIGHT = (NS - 3) * L + (L - LAST_SHARE);   // requests newer than tile t+1 at barrier t
+    static_assert(IN_FLIGHT <= 63, "vmcnt is a 6-bit counter");
+    constexpr int WAIT_TILE = (IN_FLIGHT & 15) | (7 << 4) | (15 << 8) | ((IN_FLIGHT >> 4) << 14);
+    constexpr int PRO_FLIGHT = (NS - 2) * L;                     // prologue: all but tile 0 may be in flight
+    static_assert(PRO_FLIGHT <= 63, "vmcnt is a 6-bit counter");
+    constexpr int WAIT_PRO = (PRO_FLIGHT & 15) | (7 << 4) | (15 << 8) | ((PRO_FLIGHT >> 4) << 14);
+    u32x4 fa[2][FM], fb[2][FN];
+    auto read_operands = [&](int set, const unsigned char *sA, const unsigned char *sB, int ks) {
+      const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
+      const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
+      const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+#pragma unroll
+      for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
+#pragma unroll
+      for (int j = 0; j < FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+    };
+    auto mma = [&](int set) {
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(fb[set][j], fa[set][i], acc[i][j]);
+    };
+#pragma unroll
+    for (int st = 0; st < NS - 1; ++st) {
+      const int tile = st < nk ? st : nk - 1;
+      dma(smem + st * STAGE, smem + st * STAGE + A_STAGE, tile * BK, 0, L);
+    }
+    __builtin_amdgcn_s_waitcnt(WAIT_PRO);  // this wave's share of tile 0 is in LDS
+    __syncthreads();
+    read_operands(0, smem, smem + A_STAGE, 0);
+    int cur_i = 0;          // stage of tile kt
+    int fill_i = NS - 1;    // stage released by the previous barrier, receives tile kt+NS-1
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+      unsigned char *cur = smem + cur_i * STAGE;
+      const int nxt_i = cur_i + 1 == NS ? 0 : cur_i + 1;
+      unsigned char *nxt = smem + nxt_i * STAGE;
+      unsigned char *fill = smem + fill_i * STAGE;
+      const int tile_f = kt + NS - 1 < nk ? kt + NS - 1 : nk - 1;  // clamped: a repeat of the last tile is never read
+#pragma unroll
+      for (int ks = 0; ks + 1 < KS; ++ks) {
+        dma(fill, fill + A_STAGE, tile_f * BK, (ks * L) / KS, ((ks + 1) * L) / KS);
+        read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
+        mma(ks & 1);
+        Interleave<0, R, 0x020, L / KS, 0x100, D>::run();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // tile kt+1 has landed; newer requests stay in flight
+      __syncthreads();
+      dma(fill, fill + A_STAGE, tile_f * BK, ((KS - 1) * L) / KS, L);
+      read_operands(0, nxt, nxt + A_STAGE, 0);
+      mma((KS - 1) & 1);
+      Interleave<0, R, 0x020, LAST_SHARE, 0x100, D>::run();
+      __builtin_amdgcn_sched_barrier(0);
+      fill_i = cur_i;
+      cur_i = nxt_i;
+    }
+    {
+      const unsigned char *cur = smem + cur_i * STAGE;
+#pragma unroll
+      for (int ks = 0; ks + 1 < KS; ++ks) {
+        read_operands((ks + 1) & 1, cur, cur + A_STAGE, ks + 1);
+        mma(ks & 1);
+        Interleave<0, R, 0x100, D, 0x100, 0>::run();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mma((KS - 1) & 1);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // clamped repeats must not land on the epilogue staging
   }
   __syncthreads();
 
@@ -707,7 +805,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int EP_PITCH = TN + 4;                 // floats
   constexpr int LPR = TN / 8;                      // lanes per output row
   constexpr int RPI = 64 / LPR;                    // rows per pass
-  static_assert((size_t)WM * WN * 32 * EP_PITCH * 4 <= (size_t)2 * STAGE, "staging must fit");
+  static_assert((size_t)WM * WN * 32 * EP_PITCH * 4 <= (size_t)NS * STAGE, "staging must fit");
   float *stage = (float *)smem + wave * (32 * EP_PITCH);
   const int er = lane / LPR, ec = (lane % LPR) * 8;
 #pragma unroll
@@ -748,14 +846,14 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   }
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int PIPE>
+template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE>
 int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
                        hipStream_t stream) {
-  constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * 2;
+  constexpr size_t lds = (size_t)NS * (BM + BN) * BK * 2;
   const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \
-    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, PIPE, CONVV, NCV>;                      \
+    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, NS, PIPE, CONVV, NCV>;                      \
     static bool attr_done = false;                                                           \
     if (!attr_done) {                                                                        \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                  \
@@ -766,7 +864,7 @@ int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_nc
     hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                    \
     return (int)hipGetLastError();                                                           \
   } while (0)
-  if constexpr (PIPE == 2) {
+  if constexpr (PIPE >= 2) {
     // direct-to-LDS loads cannot transpose: K-contiguous B only (the dispatcher
     // routes an N-contiguous B to the register-staged twin)
     if (b_ncontig) return (int)hipErrorInvalidValue;

@@ -14,7 +14,7 @@ const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
   static const ContractionVariant v = {
       TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT,
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
-      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_DIRECT>};
+      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT>};
   return v;
 }
 }  // namespace tracea_amd

@@ -374,7 +374,7 @@ int twin(int vi, int pipeline) {
 // pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
 int resolve_variant(int vi, bool conv, bool b_ncontig, bool k_exact) {
   int pipe = contraction_variant(vi).pipeline;
-  if (pipe == 2 && b_ncontig) pipe = 1;
+  if (pipe >= 2 && b_ncontig) pipe = 1;
   if (pipe == 1 && !conv && !k_exact) pipe = 0;
   if (pipe == contraction_variant(vi).pipeline) return vi;
   for (int want = pipe; want >= 0; --want) {
@@ -385,24 +385,6 @@ int resolve_variant(int vi, bool conv, bool b_ncontig, bool k_exact) {
   for (int i = 0; i < contraction_variant_count(); ++i)
     if (contraction_variant(i).pipeline == 0) return i;
   return vi;
-}
-
-// 256 bytes of zeros per device, the source of masked direct-to-LDS loads.
-const void *device_zeros(int device) {
-  static std::mutex mu;
-  static void *zeros[64] = {nullptr};
-  if (device < 0 || device >= 64) return nullptr;
-  std::lock_guard<std::mutex> lk(mu);
-  if (zeros[device] == nullptr) {
-    void *p = nullptr;
-    if (hipMalloc(&p, 256) != hipSuccess) return nullptr;
-    if (hipMemset(p, 0, 256) != hipSuccess) {
-      (void)hipFree(p);
-      return nullptr;
-    }
-    zeros[device] = p;
-  }
-  return zeros[device];
 }
 
 void fill_grid(ContractionArgs *a, const ContractionVariant &v) {
@@ -440,10 +422,14 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       snprintf(key, sizeof(key), "gemm_%lld_%lld_%lld_%s", M, N, K, tuning_device_name());
       int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false);
       if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "gemm: no kernel variant available");
-      vi = resolve_variant(vi, false, !b_kcontig, K % contraction_variant(vi).bk == 0);
+      // direct-to-LDS variants address operands with 32-bit byte offsets below 2 GiB
+      const long long a_extent = ((M - 1) * a.stride[0] + K) * 2;
+      const long long b_extent = b_kcontig ? ((N - 1) * b.stride[1] + K) * 2 : ((K - 1) * b.stride[0] + N) * 2;
+      const bool small = a_extent < (1ll << 31) && b_extent < (1ll << 31);
+      vi = resolve_variant(vi, false, !b_kcontig || !small, K % contraction_variant(vi).bk == 0);
       const ContractionVariant &v = contraction_variant(vi);
-      args.zeros = device_zeros(c.device);
-      if (args.zeros == nullptr) return fail(TRACEA_CUDA_ERROR, "gemm: cannot allocate the zero page");
+      args.a_bytes = (unsigned)(small ? a_extent : 0);
+      args.b_bytes = (unsigned)(small ? b_extent : 0);
       fill_grid(&args, v);
       return hip_status("gemm launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
     }
@@ -623,10 +609,13 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
            g.pad_h, tuning_device_name());
   int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
   if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
-  vi = resolve_variant(vi, true, plan.w_ncontig, true);
+  const long long x_extent = (long long)g.block.batch * g.block.h_in * g.block.w_in * g.block.c_in * 2;
+  const long long w_extent = (long long)g.n_gemm * g.k_gemm * 2;
+  const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
+  vi = resolve_variant(vi, true, plan.w_ncontig || !small, true);
   const ContractionVariant &v = contraction_variant(vi);
-  a.zeros = device_zeros(plan.out.device);
-  if (a.zeros == nullptr) return fail(TRACEA_CUDA_ERROR, "conv2d: cannot allocate the zero page");
+  a.a_bytes = (unsigned)(small ? x_extent : 0);
+  a.b_bytes = (unsigned)(small ? w_extent : 0);
   fill_grid(&a, v);
   return hip_status("conv2d launch", v.launch(a, true, plan.x.dtype, plan.w_ncontig, stream));
 }
