@@ -243,6 +243,10 @@ TraceaStatus tracea_gemm_ex(TraceaTensorView a, TraceaTensorView b, TraceaTensor
 int32_t tracea_variant_count(const char *op);
 const char *tracea_variant_name(const char *op, int32_t index); /* library-owned */
 int32_t tracea_force_variant(const char *op, int32_t index);    /* 0 ok, -1 bad argument */
+/* The variant automatic selection would run for a "gemm" or "conv2d" problem in
+ * its implicit-GEMM view (m rows, n channels, k reduction), K-contiguous B, before
+ * any forced variant is applied; -1 on a bad argument. */
+int32_t tracea_select_variant(const char *op, int64_t m, int64_t n, int64_t k);
 
 /* The 80-byte ConvParams block of the reference (src/emitter/cuda/conv.rs:134-142;
  * packing src/interface/python.rs:423-435) as this library computes it, for

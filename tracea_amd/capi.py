@@ -98,6 +98,7 @@ SIGNATURES = {
     "tracea_variant_count": (C.c_int32, [C.c_char_p]),
     "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),
     "tracea_force_variant": (C.c_int32, [C.c_char_p, C.c_int32]),
+    "tracea_select_variant": (C.c_int32, [C.c_char_p, C.c_int64, C.c_int64, C.c_int64]),
     "tracea_conv_params_pack": (C.c_int, [C.c_int32] * 10 + [C.POINTER(ConvParamsBlock)]),
     "tracea_conv_coords_device": (C.c_int, [C.POINTER(ConvParamsBlock), C.c_void_p, C.c_void_p,
                                             C.c_void_p, C.c_void_p]),

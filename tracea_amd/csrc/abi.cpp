@@ -142,6 +142,14 @@ int32_t tracea_force_variant(const char *op, int32_t index) {
   return 0;
 }
 
+int32_t tracea_select_variant(const char *op, int64_t m, int64_t n, int64_t k) {
+  if (op == nullptr || m <= 0 || n <= 0 || k <= 0 || m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31))
+    return -1;
+  const bool conv = !strcmp(op, "conv2d");
+  if (!conv && strcmp(op, "gemm") != 0) return -1;
+  return select_contraction_variant((int)m, (int)n, (int)k, conv);
+}
+
 TraceaStatus tracea_conv_params_pack(int32_t n, int32_t h, int32_t w, int32_t c, int32_t k,
                                      int32_t r, int32_t s, int32_t stride, int32_t pad,
                                      int32_t dilation, TraceaConvParamsBlock *out) {

@@ -28,9 +28,24 @@
 // ds_read_b64_tr_b16 delivers from a row-major [key][d] tile.
 // O^T accumulators of a lane all belong to the lane's query, so the online
 // rescale is a per-lane scalar multiply.
+#include <type_traits>
+
 #include "contraction_kernel.hpp"
 
 namespace tracea_amd {
+
+// Scheduling pipeline of the softmax region: per step one LDS read, one MFMA and
+// eight vector-ALU instructions (classes 0x100, 0x008, 0x002 of
+// __builtin_amdgcn_sched_group_barrier).
+template <int kStep, int kSteps>
+struct Interleave3 {
+  static __device__ __forceinline__ void run() {
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);
+    if constexpr (kStep + 1 < kSteps) Interleave3<kStep + 1, kSteps>::run();
+  }
+};
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -202,7 +217,7 @@ fa2_fwd_kernel(const AttentionArgs a) {
         }
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = exp2f(m_run - m_new);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
       m_run = m_new;
 
       // ---- P = exp2(S - m), row-sum share, B operands of the second product ----
@@ -300,6 +315,331 @@ fa2_fwd_kernel(const AttentionArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Pipelined form.  Same arithmetic and register layouts as fa2_fwd_kernel, but
+//   * K and V tiles travel with direct-to-LDS buffer loads (no staging
+//     registers, no LDS write instructions; rows at or beyond S are outside the
+//     buffer and read as zeros),
+//   * K runs one tile ahead of V: the score product of tile t+1 is issued
+//     before the softmax of tile t, so the matrix pipe works on S^T(t+1) while
+//     the vector ALU does the exponentials of tile t, and
+//   * the rescale of O is skipped while no running maximum of the wave moves.
+// LDS: two K stages and two V stages.  Iteration t starts with one barrier
+// that publishes K(t+1) and V(t) and retires K(t) and V(t-1); K(t+2) and
+// V(t+1) are then requested into the retired stages, a whole iteration before
+// they are needed.
+// ---------------------------------------------------------------------------
+template <int DT, int D>
+__global__ void __launch_bounds__(FA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+fa2_fwd_pipe_kernel(const AttentionArgs a) {
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int CH = D / 8;
+  constexpr int TILE_BYTES = FA_BKV * ROW_BYTES;
+  constexpr int KS = D / 16;
+  constexpr int DB = D / 32;
+  constexpr int RPI = 64 / CH;                 // tile rows per wave-wide load instruction
+  constexpr int NI = FA_BKV / (RPI * FA_WAVES); // load instructions per wave per tensor per tile
+  constexpr int RP = 256 / ROW_BYTES > 0 ? 256 / ROW_BYTES : 1;
+  constexpr int WIN = ROW_BYTES / 64;
+  static_assert(D % 32 == 0 && FA_BKV % (RPI * FA_WAVES) == 0, "unsupported head dim");
+
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char *const sKbase = smem;                   // 2 stages
+  unsigned char *const sVbase = smem + 2 * TILE_BYTES;  // 2 stages
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int lrow = lane & 31, g = lane >> 5;
+
+  const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
+  const int total = nqb * a.B * a.H;
+  int vid = blockIdx.x;
+  if ((total & 7) == 0) vid = (vid & 7) * (total >> 3) + (vid >> 3);
+  const int bh = vid / nqb;
+  const int qb = nqb - 1 - (vid - bh * nqb);
+  const int b = bh / a.H, h = bh - b * a.H;
+  const int q0 = qb * FA_BQ;
+  const int S = a.S;
+
+  const unsigned short *Qg = (const unsigned short *)a.Q + (long long)b * a.q_sb + (long long)h * a.q_sh;
+  const unsigned short *Kg = (const unsigned short *)a.K + (long long)b * a.k_sb + (long long)h * a.k_sh;
+  const unsigned short *Vg = (const unsigned short *)a.V + (long long)b * a.v_sb + (long long)h * a.v_sh;
+  unsigned short *Og = (unsigned short *)a.O + (long long)b * a.o_sb + (long long)h * a.o_sh;
+
+  const int q_wave0 = q0 + wave * 32;
+  const int q_mine = q_wave0 + lrow;
+  u32x4 qf[KS];
+  {
+    const int qr = q_mine < S ? q_mine : S - 1;
+    const unsigned short *qp = Qg + (long long)qr * a.q_ss + g * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4 *)(qp + ks * 16);
+  }
+
+  auto k_piece = [&](int row, int c) -> int {
+    return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
+  };
+  auto v_piece = [&](int row, int c) -> int {
+    return row * ROW_BYTES + ((c ^ (((row / RP) % WIN) << 2)) << 4);
+  };
+
+  // Buffer views of this (batch, head) slice: rows 0..S-1; anything beyond reads as zero.
+  __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)Kg, 0, (int)(((long long)(S - 1) * a.k_ss + D) * 2), 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)Vg, 0, (int)(((long long)(S - 1) * a.v_ss + D) * 2), 0x00020000);
+  // Load instruction i of this wave covers tile rows (i*FA_WAVES + wave)*RPI + lane/CH; the lane's
+  // LDS slot is 16-byte column lane%CH of that row, so it fetches the global column that the
+  // swizzle of the tensor maps there.
+  unsigned k_voff[NI], v_voff[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    const int row = (i * FA_WAVES + wave) * RPI + lane / CH;
+    const int p = lane % CH;
+    k_voff[i] = (unsigned)(row * (int)a.k_ss * 2 + ((p ^ ((row / RP) & (CH - 1))) << 4));
+    v_voff[i] = (unsigned)(row * (int)a.v_ss * 2 + ((p ^ (((row / RP) % WIN) << 2)) << 4));
+  }
+  auto load_k = [&](int t, unsigned char *dst) {
+    const unsigned adv = (unsigned)t * (unsigned)(FA_BKV * 2) * (unsigned)a.k_ss;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_k, (__attribute__((address_space(3))) void *)(dst + (i * FA_WAVES + wave_u) * RPI * ROW_BYTES),
+          16, (int)(k_voff[i] + adv), 0, 0, 0);
+  };
+  auto load_v = [&](int t, unsigned char *dst) {
+    const unsigned adv = (unsigned)t * (unsigned)(FA_BKV * 2) * (unsigned)a.v_ss;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_v, (__attribute__((address_space(3))) void *)(dst + (i * FA_WAVES + wave_u) * RPI * ROW_BYTES),
+          16, (int)(v_voff[i] + adv), 0, 0, 0);
+  };
+
+  int ntiles = (S + FA_BKV - 1) / FA_BKV;
+  if (a.causal) {
+    const int last_q = (q0 + FA_BQ - 1 < S ? q0 + FA_BQ - 1 : S - 1);
+    const int need = last_q / FA_BKV + 1;
+    ntiles = need < ntiles ? need : ntiles;
+  }
+
+  auto scores = [&](const unsigned char *sK, f32x16 (&s)[2]) {
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s[blk][e] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        const u32x4 kf = *(const u32x4 *)(sK + k_piece(blk * 32 + lrow, ks * 2 + g));
+        s[blk] = Mfma32<DT>::run(kf, qf[ks], s[blk]);
+      }
+  };
+
+  f32x16 o[DB];
+#pragma unroll
+  for (int d = 0; d < DB; ++d)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[d][e] = 0.0f;
+  float m_run = -1.0e30f, l_run = 0.0f;
+
+  // tiles at or beyond the end of the sequence lie outside the buffers and load as zeros
+  load_k(0, sKbase);
+  load_v(0, sVbase);
+  load_k(1, sKbase + TILE_BYTES);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+  f32x16 s_cur[2], s_nxt[2];
+  scores(sKbase, s_cur);
+
+  // One iteration, compiled twice: EDGE tiles (sequence end or causal diagonal)
+  // mask scores with selects, interior tiles do not test at all.  Either body is
+  // branch-free up to the optional rescale, so the MFMAs of the next tile's score
+  // product can be interleaved instruction by instruction with the vector-ALU
+  // work of this tile's softmax.
+  auto iteration = [&](int t, auto edge_tag) {
+    constexpr bool EDGE = decltype(edge_tag)::value;
+    const unsigned char *sV = sVbase + (t & 1) * TILE_BYTES;
+    const unsigned char *sKn = sKbase + ((t + 1) & 1) * TILE_BYTES;
+    const int kv0 = t * FA_BKV;
+
+    // phase 1: mask, running maximum.  The maximum is taken over the raw scores
+    // (the scale is positive) and the scale is folded into the exponent's
+    // multiply-add of phase 2.
+    float mx = -INFINITY;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        if constexpr (EDGE) {
+          const int kv = kv0 + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+          const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine));
+          s_cur[blk][e] = dead ? -INFINITY : s_cur[blk][e];
+        }
+        mx = fmaxf(mx, s_cur[blk][e]);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx * a.scale_log2);
+    const bool moved = m_new > m_run;
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    // alpha is exactly 1 for every lane whose maximum did not move: skip the
+    // 16*DB multiplies unless some lane of the wave needs them
+    if (__any(moved)) {
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    // phase 2, one scheduling region: the score product of the NEXT tile on the
+    // matrix pipe, the exponentials and row sums of THIS tile on the vector ALU
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s_nxt[blk][e] = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        const u32x4 kf = *(const u32x4 *)(sKn + k_piece(blk * 32 + lrow, ks * 2 + g));
+        s_nxt[blk] = Mfma32<DT>::run(kf, qf[ks], s_nxt[blk]);
+      }
+    float lsum = 0.0f;
+    u32x4 pf[4];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+      for (int hh = 0; hh < 2; ++hh) {
+        float p[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[blk][hh * 8 + j], a.scale_log2, -m_new));
+          lsum += p[j];
+        }
+        pf[blk * 2 + hh] = pack8<DT>(p);
+      }
+    l_run = l_run * alpha + lsum;
+    Interleave3<0, 2 * KS>::run();
+    __builtin_amdgcn_sched_barrier(0);
+
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+      for (int d = 0; d < DB; ++d) {
+        const int r = lane & 15;
+        const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
+        const int row_lo = kk * 16 + g * 4 + (r >> 2);
+        const int row_hi = row_lo + 8;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_lo, col >> 3) + (col & 7) * 2));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_hi, col >> 3) + (col & 7) * 2));
+        const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+        u32x4 vf;
+        vf[0] = lo2[0]; vf[1] = lo2[1]; vf[2] = hi2[0]; vf[3] = hi2[1];
+        o[d] = Mfma32<DT>::run(vf, pf[kk], o[d]);
+      }
+    }
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) s_cur[blk] = s_nxt[blk];
+  };
+
+  // Interior tiles first, then the edge tiles (they are the last ones: the tail of
+  // the sequence and, under a causal mask, the tiles that reach the diagonal of
+  // this wave's queries), each in a loop of its own with a single body.
+  int first_edge = ntiles;
+  if (ntiles * FA_BKV > S) first_edge = ntiles - 1;
+  if (a.causal) {
+    const int fe = (q_wave0 + 1) / FA_BKV;  // first tile with kv0 + 63 > q_wave0
+    first_edge = fe < first_edge ? fe : first_edge;
+  }
+  first_edge = __builtin_amdgcn_readfirstlane(first_edge);
+  int t = 0;
+  for (; t < first_edge; ++t) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1) and V(t), requested one iteration ago
+    __syncthreads();
+    load_k(t + 2, sKbase + (t & 1) * TILE_BYTES);
+    load_v(t + 1, sVbase + ((t + 1) & 1) * TILE_BYTES);
+    iteration(t, std::false_type{});
+  }
+  for (; t < ntiles; ++t) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    load_k(t + 2, sKbase + (t & 1) * TILE_BYTES);
+    load_v(t + 1, sVbase + ((t + 1) & 1) * TILE_BYTES);
+    iteration(t, std::true_type{});
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // look-ahead loads must not land on the output staging
+  __syncthreads();
+
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv_l = 1.0f / l_tot;
+  unsigned char *so = smem + wave * (32 * ROW_BYTES);
+#pragma unroll
+  for (int d = 0; d < DB; ++d)
+#pragma unroll
+    for (int v4 = 0; v4 < 4; ++v4) {
+      float x[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = o[d][v4 * 4 + e] * inv_l;
+      u32x2 w;
+      if constexpr (DT == DT_F16) {
+        f16x4 hq = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+        w = __builtin_bit_cast(u32x2, hq);
+      } else {
+        bf16x4 hq = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
+        w = __builtin_bit_cast(u32x2, hq);
+      }
+      *(u32x2 *)(so + lrow * ROW_BYTES + (d * 32 + v4 * 8 + g * 4) * 2) = w;
+    }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 32 * CH / 64; ++i) {
+    const int p = lane + i * 64;
+    const int row = p / CH, c = p % CH;
+    const int q = q_wave0 + row;
+    if (q < S)
+      *(u32x4 *)(Og + (long long)q * a.o_ss + c * 8) = *(const u32x4 *)(so + row * ROW_BYTES + c * 16);
+  }
+}
+
+template <int D>
+static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
+  constexpr size_t lds = 4 * (size_t)FA_BKV * D * 2;
+  const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
+  const dim3 grid((unsigned)(nqb * a.B * a.H)), block(FA_WAVES * 64);
+#define TRACEA_FA_LAUNCH(DTV)                                                                  \
+  do {                                                                                         \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D>;                                                    \
+    static bool attr_done = false;                                                             \
+    if (!attr_done) {                                                                          \
+      hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return (int)e;                                                      \
+      attr_done = true;                                                                        \
+    }                                                                                          \
+    hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                      \
+    return (int)hipGetLastError();                                                             \
+  } while (0)
+  if (dtype == DT_F16) TRACEA_FA_LAUNCH(DT_F16);
+  else TRACEA_FA_LAUNCH(DT_BF16);
+#undef TRACEA_FA_LAUNCH
+}
+
+// The buffer loads address a (batch, head) slice with 32-bit byte offsets.
+static bool slice_fits(const AttentionArgs &a) {
+  const long long k_ext = ((long long)(a.S - 1 + 3 * FA_BKV) * a.k_ss + a.D) * 2;
+  const long long v_ext = ((long long)(a.S - 1 + 3 * FA_BKV) * a.v_ss + a.D) * 2;
+  return k_ext < (1ll << 31) && v_ext < (1ll << 31);
+}
+// (the running maximum is taken over raw scores, which needs a positive scale)
+static bool feasible_pipe_d128(const AttentionArgs &a) { return a.D == 128 && a.scale_log2 > 0.0f && slice_fits(a); }
+static bool feasible_pipe_d64(const AttentionArgs &a) { return a.D == 64 && a.scale_log2 > 0.0f && slice_fits(a); }
+
 template <int D, bool V_TR>
 static int launch_fa2(const AttentionArgs &a, int dtype, hipStream_t stream) {
   constexpr size_t lds = 2 * 2 * (size_t)FA_BKV * D * 2;
@@ -327,6 +667,8 @@ static bool feasible_d128(const AttentionArgs &a) { return a.D == 128; }
 static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 
 static const AttentionVariant kAttentionVariants[] = {
+    {"fa2_q128_kv64_d128_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<128>, &feasible_pipe_d128},
+    {"fa2_q128_kv64_d64_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<64>, &feasible_pipe_d64},
     {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, true>, &feasible_d128},
     {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, false>, &feasible_d128},
     {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<64, true>, &feasible_d64},

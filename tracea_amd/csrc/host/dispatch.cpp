@@ -311,36 +311,32 @@ TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s,
 }
 
 // ---- variant choice --------------------------------------------------------------
-// Score = useful fraction of the padded tile grid x fraction of the last wave
-// of workgroups that is occupied x a per-shape efficiency prior (larger tiles
-// re-use more of each LDS fetch).  A tuning-cache entry, when present, wins.
+// Cost model: the tile grid is executed in rounds over the 256 compute units;
+// a round costs the tile area divided by the efficiency prior of the variant
+// (operand re-use of the tile shape x measured gain of its pipeline).  Partial
+// tiles at the edges are paid in full through the tile count.  A tuning-cache
+// entry, when present, wins over this.
 int select_contraction_variant(int m, int n, int k, bool conv) {
   (void)k;
   (void)conv;
-  const int cus = 256;
+  const double cus = 256.0;
   int best = -1;
-  double best_score = -1.0;
+  double best_cost = 0.0;
   for (int i = 0; i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
-    const long long gm = (m + v.bm - 1) / v.bm, gn = (n + v.bn - 1) / v.bn;
-    const double useful = ((double)m * n) / ((double)gm * v.bm * gn * v.bn);
-    const long long tiles = gm * gn;
-    // workgroups resident per CU: bounded by LDS (160 KB) and by 8 waves per CU here
-    const int per_cu_lds = (int)(160 * 1024 / v.lds_bytes);
-    const int per_cu_waves = 8 / (v.waves_m * v.waves_n) > 0 ? 8 / (v.waves_m * v.waves_n) : 1;
-    const int per_cu = per_cu_lds < per_cu_waves ? (per_cu_lds > 0 ? per_cu_lds : 1) : per_cu_waves;
-    const long long slots = (long long)cus * per_cu;
-    const long long rounds = (tiles + slots - 1) / slots;
-    const double quant = (double)tiles / (double)(rounds * slots);
+    const double gm = (double)((m + v.bm - 1) / v.bm), gn = (double)((n + v.bn - 1) / v.bn);
+    const double tiles = gm * gn;
+    const double exact = tiles / cus > 1.0 ? tiles / cus : 1.0;
+    const double rounds = 0.5 * std::ceil(tiles / cus) + 0.5 * exact;  // co-resident workgroups soften the step
     const double reuse = (double)(v.bm * v.bn) / (double)(v.bm + v.bn) / 128.0;
     double prior = reuse > 1.0 ? 1.0 : reuse;
     // measured on MI355X at 4096^3: the pipelined loops gain ~35 % over the plain
-    // one, direct-to-LDS loads a further ~5 %, eight waves ~4 % over four
-    prior *= v.pipeline == 2 ? 1.42 : (v.pipeline == 1 ? 1.35 : 1.0);
+    // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
+    prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
-    const double score = useful * (0.35 + 0.65 * quant) * (0.3 + 0.7 * prior);
-    if (score > best_score) {
-      best_score = score;
+    const double cost = rounds * (double)v.bm * (double)v.bn / prior;
+    if (best < 0 || cost < best_cost) {
+      best_cost = cost;
       best = i;
     }
   }

@@ -374,6 +374,9 @@ TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
   for (int i = 0; i < attention_variant_count(); ++i) {
     AttentionArgs probe{};
     probe.D = (int)d;
+    probe.S = (int)s;
+    probe.k_ss = probe.v_ss = (long long)d;
+    probe.scale_log2 = 1.0f;
     if (!attention_variant(i).feasible(probe)) continue;
     set_forced_variant("attention", i);
     const double t = time_launches(
