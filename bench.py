@@ -6,7 +6,7 @@ fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
 FlashAttention-2 forward named by the metric are timed in the same run and
 reported under "also".  Prints one JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|conv|attention|attention_causal]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|conv|attention|attention_causal|copy]
 """
 import argparse
 import json
@@ -19,6 +19,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
+# HBM-side bytes per launch of the dominant kernel of each workload, from the rocprofv3
+# FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
+# (profiles/bench_kernels_mi355x.md); None where no counter run exists.
+TRAFFIC_BYTES = {"gemm": 235.1e6, "conv": 26.6e6, "attention": 580.7e6, "attention_causal": None, "copy": None}
 METRIC = "TFLOPS + % fp16 MFMA peak: GEMM 4096^3, 3x3 implicit-GEMM conv, FA2 fwd"
 
 
@@ -51,6 +55,12 @@ def make_workload(name, torch, ops):
         flops = 4.0 * b * h * d * (s * (s + 1) / 2.0 if causal else float(s) * s)
         return ("bf16 FA2 forward B4 H32 S4096 D128 %s" % ("causal" if causal else "dense"),
                 flops, 2.0 * 4 * q.numel(), "bf16", lambda: ops.attention(q, k, v, causal=causal, out=o))
+    if name == "copy":
+        # calibration workload for the HBM traffic counters: a plain device copy of known size
+        n = 256 << 20
+        src = torch.empty(n, device=dev, dtype=torch.uint8).fill_(1)
+        dst = torch.empty(n, device=dev, dtype=torch.uint8)
+        return ("device copy of 256 MiB (counter calibration)", 0.0, 2.0 * n, "u8", lambda: dst.copy_(src))
     raise SystemExit("unknown workload " + name)
 
 
@@ -123,7 +133,8 @@ def main():
         "data": "synthetic", "config": {"workload": label},
         "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS, 4), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS, 4),
+                     "traffic": TRAFFIC_BYTES.get(args.workload),
                      "hbm_GBps_algorithmic": round(bytes_ / dev_s / 1e9, 1)},
     }
     if not args.no_extras:
