@@ -121,3 +121,19 @@ def test_tune_without_runtime_reports_failure():
     l.tracea_shutdown()
     ok, score, cfg, err = capi.take_result(l.tracea_tune_gemm(256, 256, 256))
     assert not ok and cfg is None and "tracea_init" in err
+
+
+def test_cpp_header_compiles_and_links(tmp_path):
+    """include/tracea.hpp is usable by a plain C++17 caller linked against libtracea.so."""
+    import shutil
+    import subprocess
+    cxx = shutil.which("g++")
+    if cxx is None:
+        pytest.skip("no g++")
+    exe = tmp_path / "hdr"
+    libdir = os.path.dirname(capi.LIB_PATH)
+    subprocess.check_call([cxx, "-std=c++17", "-I", os.path.join(ROOT, "include"),
+                           os.path.join(ROOT, "tests", "cpp_header_check.cpp"), "-o", str(exe),
+                           "-L", libdir, "-ltracea", "-Wl,-rpath," + libdir])
+    out = subprocess.check_output([str(exe)]).decode()
+    assert "tracea.hpp ok" in out
