@@ -1,5 +1,5 @@
 """The C ABI as far as it can be exercised without a GPU: the library loads,
-exports every symbol include/tracea.h declares, and its host-side logic
+exports every symbol include/tracea.h and include/tracea_tuner.h declare, and its host-side logic
 (errors, version, ConvParams packing, variant table) behaves as documented."""
 import ctypes as C
 import os
@@ -15,9 +15,12 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_functions():
-    text = open(os.path.join(ROOT, "include", "tracea.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(tracea_[a-z0-9_]+)\s*\(", text)))
+    names = set()
+    for header in ("tracea.h", "tracea_tuner.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names.update(re.findall(r"\b(tracea_[a-z0-9_]+)\s*\(", text))
+    return sorted(names)
 
 
 def test_every_declared_symbol_is_exported():

@@ -29,7 +29,7 @@ INCLUDE = os.path.normpath(os.path.join(HERE, "..", "include"))
 COMMON = ["-I" + INCLUDE, "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
           "-Wno-pass-failed"]
 
-HOST_SOURCES = ["abi.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
+HOST_SOURCES = ["abi.cpp", "tuner_abi.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
                 "host/pipeline_config.cpp", "host/gaussian_process.cpp", "host/autotuner.cpp"]
 DEVICE_SOURCES = ["support_kernels.hip", "attention_kernels.hip"]
 
@@ -71,8 +71,7 @@ def _jobs():
     for s in DEVICE_SOURCES:
         jobs.append((os.path.join(CSRC, s), os.path.join(OBJ, s.replace("/", "_") + ".o"), DEVICE_FLAGS))
     for s in HOST_SOURCES:
-        if os.path.exists(os.path.join(CSRC, s)):
-            jobs.append((os.path.join(CSRC, s), os.path.join(OBJ, s.replace("/", "_") + ".o"), []))
+        jobs.append((os.path.join(CSRC, s), os.path.join(OBJ, s.replace("/", "_") + ".o"), []))
     return jobs
 
 

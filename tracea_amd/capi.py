@@ -104,6 +104,53 @@ SIGNATURES = {
                                             C.c_void_p, C.c_void_p]),
 }
 
+MEASURE_FN = C.CFUNCTYPE(C.c_float, C.c_char_p, C.c_void_p)
+_STR = C.c_void_p  # char* the caller frees with tracea_free_string
+
+# every symbol include/tracea_tuner.h declares
+SIGNATURES.update({
+    "tracea_pipeline_config_new": (_STR, [C.c_uint32] * 4),
+    "tracea_pipeline_config_normalize": (_STR, [C.c_char_p]),
+    "tracea_pipeline_config_validate": (C.c_int32, [C.c_char_p, C.POINTER(C.c_void_p)]),
+    "tracea_pipeline_config_to_vector": (C.c_int32, [C.c_char_p, C.POINTER(C.c_float), C.c_int32]),
+    "tracea_hardware_profile_json": (_STR, [C.c_char_p]),
+    "tracea_check_feasibility": (C.c_int32, [C.c_char_p, C.c_char_p, C.c_uint64, C.POINTER(C.c_void_p)]),
+    "tracea_estimate_occupancy": (C.c_float, [C.c_char_p, C.c_char_p]),
+    "tracea_gp_create": (C.c_void_p, []),
+    "tracea_gp_destroy": (None, [C.c_void_p]),
+    "tracea_gp_set_noise_sigma": (None, [C.c_void_p, C.c_float]),
+    "tracea_gp_set_exploration_beta": (None, [C.c_void_p, C.c_float]),
+    "tracea_gp_observe": (C.c_int32, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_char_p, C.c_float,
+                                      C.c_char_p]),
+    "tracea_gp_predict": (C.c_int32, [C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_char_p, C.c_char_p,
+                                      C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "tracea_gp_acquisition": (C.c_float, [C.c_void_p, C.c_int32, C.c_uint32, C.c_uint32, C.c_uint32,
+                                          C.c_char_p, C.c_char_p, C.c_float, C.c_uint64]),
+    "tracea_gp_marginal_log_likelihood": (C.c_float, [C.c_void_p, C.c_char_p]),
+    "tracea_gp_optimize_hyperparams": (None, [C.c_void_p, C.c_char_p]),
+    "tracea_gp_length_scales": (C.c_int32, [C.c_void_p, C.POINTER(C.c_float), C.c_int32]),
+    "tracea_gp_features": (C.c_int32, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_char_p, C.POINTER(C.c_float),
+                                       C.c_int32]),
+    "tracea_gp_roofline_prior": (C.c_float, [C.c_uint32, C.c_uint32, C.c_uint32, C.c_char_p, C.c_char_p]),
+    "tracea_propose_gemm_configs": (_STR, [C.c_uint32] * 3),
+    "tracea_propose_conv_configs": (_STR, [C.c_uint32] * 3),
+    "tracea_propose_attention_configs": (_STR, [C.c_uint32]),
+    "tracea_search_space_enumerate": (_STR, [C.c_char_p]),
+    "tracea_variant_for_config": (C.c_int32, [C.c_char_p]),
+    "tracea_magic_number_strategy": (C.c_char_p, [C.c_uint64]),
+    "tracea_tuning_cache_path": (_STR, []),
+    "tracea_tuning_cache_get": (_STR, [C.c_char_p]),
+    "tracea_tuning_cache_put": (C.c_int32, [C.c_char_p, C.c_char_p, C.c_float, C.c_uint64]),
+    "tracea_tuning_cache_reload": (None, []),
+    "tracea_tuning_key_gemm": (_STR, [C.c_uint64] * 3 + [C.c_char_p]),
+    "tracea_tuning_key_conv2d": (_STR, [C.c_uint32] * 9 + [C.c_char_p]),
+    "tracea_autotune_candidates": (Result, [C.c_char_p, C.c_char_p, MEASURE_FN, C.c_void_p]),
+    "tracea_autotune_guided": (Result, [C.c_char_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_char_p,
+                                        MEASURE_FN, C.c_void_p, C.c_uint32, C.c_int, C.c_uint64]),
+    "tracea_autotune_gemm": (Result, [C.c_size_t] * 3 + [C.c_uint32]),
+    "tracea_autotune_conv2d": (Result, [C.c_size_t] * 10 + [C.c_uint32]),
+})
+
 _lib = None
 
 
@@ -165,6 +212,15 @@ def take_result(res):
     if res.error_msg:
         lib().tracea_free_string(res.error_msg)
     return bool(res.success), float(res.score), cfg, err
+
+
+def take_string(ptr):
+    """char* from the library -> str (None for NULL); frees it."""
+    if not ptr:
+        return None
+    text = C.string_at(ptr).decode()
+    lib().tracea_free_string(ptr)
+    return text
 
 
 def variants(op):

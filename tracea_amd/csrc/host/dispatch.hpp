@@ -52,7 +52,16 @@ TraceaStatus dispatch_attention(const TraceaTensorView &q, const TraceaTensorVie
 // forced variant nor a tuning-cache entry decides).  Returns -1 if none fits.
 int select_contraction_variant(int m, int n, int k, bool conv);
 
+// TraceaResult builders: strings are malloc'ed, released by tracea_free_string.
+struct PipelineConfig;
+char *dup_cstr(const std::string &s);
+TraceaResult failure(const std::string &msg);
+TraceaResult success(const PipelineConfig &cfg, float tflops);
+
 TraceaResult tune_gemm(size_t m, size_t n, size_t k);
+TraceaResult autotune_gemm(size_t m, size_t n, size_t k, uint32_t iterations);
+TraceaResult autotune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s,
+                             size_t stride, size_t pad, size_t dilation, uint32_t iterations);
 TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal);
 TraceaResult tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s,
                          size_t stride, size_t pad, size_t dilation);

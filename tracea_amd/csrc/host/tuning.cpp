@@ -23,6 +23,7 @@
 #include <sstream>
 
 #include "dispatch.hpp"
+#include "tuner.hpp"
 #include "tuning_cache.hpp"
 
 namespace tracea_amd {
@@ -162,17 +163,6 @@ PipelineConfig config_for_attention_variant(int index) {
   return c;
 }
 
-// ---- micro-benchmarks ------------------------------------------------------------
-namespace {
-
-struct DeviceBuffer {
-  void *p = nullptr;
-  ~DeviceBuffer() {
-    if (p) (void)hipFree(p);
-  }
-  bool alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16) == hipSuccess; }
-};
-
 char *dup_cstr(const std::string &s) {
   char *p = (char *)malloc(s.size() + 1);
   if (p) memcpy(p, s.c_str(), s.size() + 1);
@@ -196,6 +186,17 @@ TraceaResult success(const PipelineConfig &cfg, float tflops) {
   r.config_ptr = dup_cstr(cfg.to_json());
   return r;
 }
+
+// ---- micro-benchmarks ------------------------------------------------------------
+namespace {
+
+struct DeviceBuffer {
+  void *p = nullptr;
+  ~DeviceBuffer() {
+    if (p) (void)hipFree(p);
+  }
+  bool alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 16) == hipSuccess; }
+};
 
 std::string last_error_text() {
   uint8_t buf[512];
@@ -239,112 +240,252 @@ uint64_t now_seconds() {
 
 }  // namespace
 
-TraceaResult tune_gemm(size_t m, size_t n, size_t k) {
-  if (!runtime_ready()) return failure("tracea_init has not been called");
-  if (m == 0 || n == 0 || k == 0 || k % 8 != 0 || m >= (1u << 31) || n >= (1u << 31) || k >= (1u << 31))
-    return failure("tune_gemm: dimensions must be positive, K a multiple of 8");
-  // fp16, A row-major [M,K], B column-major (stored [N,K]), C fp16 row-major
+// ---- micro-benchmarks as objects (the reference's MicroBenchmark / Conv2dBenchmark
+// traits: src/optimizer/benchmark.rs:140-200, 420-470) ----------------------------
+namespace {
+
+// fp16 GEMM, A row-major [M,K], B column-major (stored [N,K]), C fp16 row-major.
+struct GemmBenchmark {
+  size_t m = 0, n = 0, k = 0;
   DeviceBuffer a, b, c;
-  if (!a.alloc(m * k * 2) || !b.alloc(n * k * 2) || !c.alloc(m * n * 2)) {
-    (void)hipGetLastError();
-    return failure("tune_gemm: device allocation failed");
+  std::string error;
+
+  bool init(size_t m_, size_t n_, size_t k_) {
+    m = m_; n = n_; k = k_;
+    if (!a.alloc(m * k * 2) || !b.alloc(n * k * 2) || !c.alloc(m * n * 2)) {
+      (void)hipGetLastError();
+      error = "device allocation failed";
+      return false;
+    }
+    const float amp = sqrtf(3.0f / (float)k);  // unit-variance dot products
+    launch_fill_uniform(a.p, m * k, DT_F16, 1u, amp, nullptr);
+    launch_fill_uniform(b.p, n * k, DT_F16, 2u, amp, nullptr);
+    return true;
   }
-  const float amp = sqrtf(3.0f / (float)k);  // unit-variance dot products
-  launch_fill_uniform(a.p, m * k, DT_F16, 1u, amp, nullptr);
-  launch_fill_uniform(b.p, n * k, DT_F16, 2u, amp, nullptr);
-  const uint64_t sa[2] = {m, k}, sb[2] = {k, n}, sc[2] = {m, n};
-  const int64_t ta[2] = {(int64_t)k, 1}, tb[2] = {1, (int64_t)k}, tcs[2] = {(int64_t)n, 1};
-  TraceaTensorView va{a.p, 2, sa, ta, TRACEA_DTYPE_FLOAT16, 0};
-  TraceaTensorView vb{b.p, 2, sb, tb, TRACEA_DTYPE_FLOAT16, 0};
-  TraceaTensorView vc{c.p, 2, sc, tcs, TRACEA_DTYPE_FLOAT16, 0};
-  TraceaGemmParams gp{TRACEA_EPILOGUE_IDENTITY, nullptr};
-  const int saved = forced_variant("gemm");
-  const double flops = 2.0 * (double)m * (double)n * (double)k;
-  int best = -1;
-  double best_tflops = 0.0;
-  std::string err;
-  for (int i = 0; i < contraction_variant_count(); ++i) {
-    set_forced_variant("gemm", i);
+  // TFLOP/s of one contraction variant, <= 0 when it did not run.
+  float measure(int variant) {
+    const uint64_t sa[2] = {m, k}, sb[2] = {k, n}, sc[2] = {m, n};
+    const int64_t ta[2] = {(int64_t)k, 1}, tb[2] = {1, (int64_t)k}, tcs[2] = {(int64_t)n, 1};
+    TraceaTensorView va{a.p, 2, sa, ta, TRACEA_DTYPE_FLOAT16, 0};
+    TraceaTensorView vb{b.p, 2, sb, tb, TRACEA_DTYPE_FLOAT16, 0};
+    TraceaTensorView vc{c.p, 2, sc, tcs, TRACEA_DTYPE_FLOAT16, 0};
+    TraceaGemmParams gp{TRACEA_EPILOGUE_IDENTITY, nullptr};
+    const int saved = forced_variant("gemm");
+    set_forced_variant("gemm", variant);
     const double t = time_launches(
         [&]() { return dispatch_gemm_kind(va, vb, nullptr, nullptr, &vc, gp) == TRACEA_SUCCESS; }, 3, 10);
+    set_forced_variant("gemm", saved);
     if (t <= 0.0) {
-      err = last_error_text();
-      continue;
+      error = last_error_text();
+      return 0.0f;
     }
-    const double tf = flops / t * 1e-12;
+    return (float)(2.0 * (double)m * (double)n * (double)k / t * 1e-12);
+  }
+};
+
+// fp16 NHWC convolution with a ReLU epilogue, square stride / padding / dilation.
+struct ConvBenchmark {
+  size_t n = 0, c = 0, h = 0, w = 0, k = 0, r = 0, s = 0, stride = 1, pad = 0, dilation = 1;
+  ConvGeometry g;
+  DeviceBuffer x, wt, y;
+  std::string error;
+
+  bool init(size_t n_, size_t c_, size_t h_, size_t w_, size_t k_, size_t r_, size_t s_, size_t stride_,
+            size_t pad_, size_t dilation_) {
+    n = n_; c = c_; h = h_; w = w_; k = k_; r = r_; s = s_;
+    stride = stride_; pad = pad_; dilation = dilation_;
+    if (make_conv_geometry((int)n, (int)h, (int)w, (int)c, (int)k, (int)r, (int)s, (int)stride,
+                           (int)stride, (int)pad, (int)pad, (int)dilation, (int)dilation,
+                           &g) != TRACEA_SUCCESS) {
+      error = last_error_text();
+      return false;
+    }
+    const size_t ho = (size_t)g.block.h_out, wo = (size_t)g.block.w_out;
+    if (!x.alloc(n * h * w * c * 2) || !wt.alloc(k * r * s * c * 2) || !y.alloc(n * ho * wo * k * 2)) {
+      (void)hipGetLastError();
+      error = "device allocation failed";
+      return false;
+    }
+    launch_fill_uniform(x.p, n * h * w * c, DT_F16, 3u, 1.0f, nullptr);
+    launch_fill_uniform(wt.p, k * r * s * c, DT_F16, 4u, sqrtf(3.0f / (float)(r * s * c)), nullptr);
+    return true;
+  }
+  float measure(int variant) {
+    const size_t ho = (size_t)g.block.h_out, wo = (size_t)g.block.w_out;
+    const uint64_t sx[4] = {n, h, w, c}, sw[4] = {k, r, s, c}, sy[4] = {n, ho, wo, k};
+    TraceaTensorView vx{x.p, 4, sx, nullptr, TRACEA_DTYPE_FLOAT16, 0};
+    TraceaTensorView vw{wt.p, 4, sw, nullptr, TRACEA_DTYPE_FLOAT16, 0};
+    TraceaTensorView vy{y.p, 4, sy, nullptr, TRACEA_DTYPE_FLOAT16, 0};
+    TraceaConv2dParams cp{(uint32_t)stride, (uint32_t)stride, (uint32_t)pad, (uint32_t)pad,
+                          (uint32_t)dilation, (uint32_t)dilation, 1, TRACEA_EPILOGUE_RELU, nullptr};
+    const int saved = forced_variant("conv2d");
+    set_forced_variant("conv2d", variant);
+    const double t = time_launches(
+        [&]() { return dispatch_conv2d_kind(vx, vw, nullptr, nullptr, &vy, cp) == TRACEA_SUCCESS; }, 3, 10);
+    set_forced_variant("conv2d", saved);
+    if (t <= 0.0) {
+      error = last_error_text();
+      return 0.0f;
+    }
+    return (float)(2.0 * (double)g.m_gemm * (double)g.n_gemm * (double)g.k_gemm / t * 1e-12);
+  }
+};
+
+bool gemm_dims_ok(size_t m, size_t n, size_t k) {
+  return m != 0 && n != 0 && k != 0 && k % 8 == 0 && m < (1u << 31) && n < (1u << 31) && k < (1u << 31);
+}
+
+bool conv_dims_ok(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s, size_t stride,
+                  size_t dilation, std::string *why) {
+  if (n == 0 || c == 0 || h == 0 || w == 0 || k == 0 || r == 0 || s == 0 || stride == 0 || dilation == 0) {
+    *why = "dimensions, stride and dilation must be positive";
+    return false;
+  }
+  if (c % 8 != 0) {
+    *why = "input channels must be a multiple of 8";
+    return false;
+  }
+  return true;
+}
+
+}  // namespace
+
+TraceaResult tune_gemm(size_t m, size_t n, size_t k) {
+  if (!runtime_ready()) return failure("tracea_init has not been called");
+  if (!gemm_dims_ok(m, n, k)) return failure("tune_gemm: dimensions must be positive, K a multiple of 8");
+  GemmBenchmark bench;
+  if (!bench.init(m, n, k)) return failure("tune_gemm: " + bench.error);
+  int best = -1;
+  float best_tflops = 0.0f;
+  for (int i = 0; i < contraction_variant_count(); ++i) {
+    const float tf = bench.measure(i);
     if (tf > best_tflops) {
       best_tflops = tf;
       best = i;
     }
   }
-  set_forced_variant("gemm", saved);
-  if (best < 0) return failure("tune_gemm: no variant ran: " + err);
+  if (best < 0) return failure("tune_gemm: no variant ran: " + bench.error);
   CacheEntry e;
   e.config = config_for_contraction_variant(best);
-  e.score = (float)best_tflops;
+  e.score = best_tflops;
   e.timestamp = now_seconds();
-  char key[160];
-  snprintf(key, sizeof(key), "gemm_%zu_%zu_%zu_%s", m, n, k, tuning_device_name());
-  tuning_cache_put(key, e, true);
+  tuning_cache_put(gemm_cache_key(m, n, k, tuning_device_name()), e, true);
   return success(e.config, e.score);
 }
 
 TraceaResult tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s,
                          size_t stride, size_t pad, size_t dilation) {
   if (!runtime_ready()) return failure("tracea_init has not been called");
-  if (n == 0 || c == 0 || h == 0 || w == 0 || k == 0 || r == 0 || s == 0 || stride == 0 || dilation == 0)
-    return failure("tune_conv2d: dimensions, stride and dilation must be positive");
-  if (c % 8 != 0) return failure("tune_conv2d: input channels must be a multiple of 8");
-  ConvGeometry g;
-  if (make_conv_geometry((int)n, (int)h, (int)w, (int)c, (int)k, (int)r, (int)s, (int)stride,
-                         (int)stride, (int)pad, (int)pad, (int)dilation, (int)dilation,
-                         &g) != TRACEA_SUCCESS)
-    return failure("tune_conv2d: " + last_error_text());
-  const size_t ho = (size_t)g.block.h_out, wo = (size_t)g.block.w_out;
-  DeviceBuffer x, wt, y;
-  if (!x.alloc(n * h * w * c * 2) || !wt.alloc(k * r * s * c * 2) || !y.alloc(n * ho * wo * k * 2)) {
-    (void)hipGetLastError();
-    return failure("tune_conv2d: device allocation failed");
-  }
-  launch_fill_uniform(x.p, n * h * w * c, DT_F16, 3u, 1.0f, nullptr);
-  launch_fill_uniform(wt.p, k * r * s * c, DT_F16, 4u, sqrtf(3.0f / (float)(r * s * c)), nullptr);
-  const uint64_t sx[4] = {n, h, w, c}, sw[4] = {k, r, s, c}, sy[4] = {n, ho, wo, k};
-  TraceaTensorView vx{x.p, 4, sx, nullptr, TRACEA_DTYPE_FLOAT16, 0};
-  TraceaTensorView vw{wt.p, 4, sw, nullptr, TRACEA_DTYPE_FLOAT16, 0};
-  TraceaTensorView vy{y.p, 4, sy, nullptr, TRACEA_DTYPE_FLOAT16, 0};
-  TraceaConv2dParams cp{(uint32_t)stride, (uint32_t)stride, (uint32_t)pad, (uint32_t)pad,
-                        (uint32_t)dilation, (uint32_t)dilation, 1, TRACEA_EPILOGUE_RELU, nullptr};
-  const int saved = forced_variant("conv2d");
-  const double flops = 2.0 * (double)g.m_gemm * (double)g.n_gemm * (double)g.k_gemm;
+  std::string why;
+  if (!conv_dims_ok(n, c, h, w, k, r, s, stride, dilation, &why)) return failure("tune_conv2d: " + why);
+  ConvBenchmark bench;
+  if (!bench.init(n, c, h, w, k, r, s, stride, pad, dilation)) return failure("tune_conv2d: " + bench.error);
   int best = -1;
-  double best_tflops = 0.0;
-  std::string err;
+  float best_tflops = 0.0f;
   for (int i = 0; i < contraction_variant_count(); ++i) {
-    set_forced_variant("conv2d", i);
-    const double t = time_launches(
-        [&]() { return dispatch_conv2d_kind(vx, vw, nullptr, nullptr, &vy, cp) == TRACEA_SUCCESS; }, 3, 10);
-    if (t <= 0.0) {
-      err = last_error_text();
-      continue;
-    }
-    const double tf = flops / t * 1e-12;
+    const float tf = bench.measure(i);
     if (tf > best_tflops) {
       best_tflops = tf;
       best = i;
     }
   }
-  set_forced_variant("conv2d", saved);
-  if (best < 0) return failure("tune_conv2d: no variant ran: " + err);
+  if (best < 0) return failure("tune_conv2d: no variant ran: " + bench.error);
   CacheEntry e;
   e.config = config_for_contraction_variant(best);
   e.config.layout_policy = "NHWC";
-  e.score = (float)best_tflops;
+  e.score = best_tflops;
   e.timestamp = now_seconds();
-  char key[200];
-  snprintf(key, sizeof(key), "conv_%zu_%zu_%zu_%zu_%zu_%zu_%zu_%zu_%zu_%s", n, h, w, c, k, r, s,
-           stride, pad, tuning_device_name());
-  tuning_cache_put(key, e, true);
+  ConvProblem p;
+  p.batch = (uint32_t)n; p.h_in = (uint32_t)h; p.w_in = (uint32_t)w; p.c_in = (uint32_t)c;
+  p.c_out = (uint32_t)k; p.kernel_h = (uint32_t)r; p.kernel_w = (uint32_t)s;
+  p.stride = (uint32_t)stride; p.pad = (uint32_t)pad; p.dilation = (uint32_t)dilation;
+  tuning_cache_put(conv_cache_key(p, tuning_device_name()), e, true);
   return success(e.config, e.score);
+}
+
+// AutoTuner::optimize on the device: cache first, then every candidate
+// (iterations 0) or an expected-improvement-guided subset of them.
+TraceaResult autotune_gemm(size_t m, size_t n, size_t k, uint32_t iterations) {
+  if (!runtime_ready()) return failure("tracea_init has not been called");
+  if (!gemm_dims_ok(m, n, k)) return failure("autotune_gemm: dimensions must be positive, K a multiple of 8");
+  GemmBenchmark bench;
+  bool ready = false;
+  auto measure = [&](const PipelineConfig &cfg) -> float {
+    const int vi = contraction_variant_for_config(cfg);
+    if (vi < 0) return 0.0f;
+    if (!ready) {
+      if (!bench.init(m, n, k)) return 0.0f;
+      ready = true;
+    }
+    return bench.measure(vi);
+  };
+  AutoTuner tuner(HardwareProfile::mi355x());
+  tuner.hardware_id = tuning_device_name();
+  PipelineConfig best;
+  if (iterations == 0) {
+    best = tuner.optimize((uint32_t)m, (uint32_t)n, (uint32_t)k, measure);
+  } else {
+    const std::string key = gemm_cache_key(m, n, k, tuner.hardware_id);
+    CacheEntry hit;
+    if (tuning_cache_get(key, &hit)) return success(hit.config, hit.score);
+    best = tuner.optimize_guided((uint32_t)m, (uint32_t)n, (uint32_t)k,
+                                 propose_gemm_configs((uint32_t)m, (uint32_t)n, (uint32_t)k), measure,
+                                 iterations, AcquisitionFunction::EI);
+    if (tuner.best_score > 0.0f) {
+      CacheEntry e;
+      e.config = best;
+      e.score = tuner.best_score;
+      e.timestamp = now_seconds();
+      tuning_cache_put(key, e, true);
+    }
+  }
+  if (!(tuner.best_score > 0.0f)) return failure("autotune_gemm: no candidate ran: " + bench.error);
+  return success(best, tuner.best_score);
+}
+
+TraceaResult autotune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, size_t s,
+                             size_t stride, size_t pad, size_t dilation, uint32_t iterations) {
+  if (!runtime_ready()) return failure("tracea_init has not been called");
+  std::string why;
+  if (!conv_dims_ok(n, c, h, w, k, r, s, stride, dilation, &why)) return failure("autotune_conv2d: " + why);
+  ConvProblem p;
+  p.batch = (uint32_t)n; p.h_in = (uint32_t)h; p.w_in = (uint32_t)w; p.c_in = (uint32_t)c;
+  p.c_out = (uint32_t)k; p.kernel_h = (uint32_t)r; p.kernel_w = (uint32_t)s;
+  p.stride = (uint32_t)stride; p.pad = (uint32_t)pad; p.dilation = (uint32_t)dilation;
+  ConvBenchmark bench;
+  bool ready = false;
+  auto measure = [&](const PipelineConfig &cfg) -> float {
+    const int vi = contraction_variant_for_config(cfg);
+    if (vi < 0) return 0.0f;
+    if (!ready) {
+      if (!bench.init(n, c, h, w, k, r, s, stride, pad, dilation)) return 0.0f;
+      ready = true;
+    }
+    return bench.measure(vi);
+  };
+  AutoTuner tuner(HardwareProfile::mi355x());
+  tuner.hardware_id = tuning_device_name();
+  PipelineConfig best;
+  if (iterations == 0) {
+    best = tuner.optimize_conv(p, measure).base;
+  } else {
+    const std::string key = conv_cache_key(p, tuner.hardware_id);
+    CacheEntry hit;
+    if (tuning_cache_get(key, &hit)) return success(hit.config, hit.score);
+    const uint32_t mg = p.batch * p.h_out() * p.w_out(), kg = p.c_in * p.kernel_h * p.kernel_w;
+    best = tuner.optimize_guided(mg, p.c_out, kg, propose_conv_configs(mg, p.c_out, kg), measure, iterations,
+                                 AcquisitionFunction::EI);
+    if (tuner.best_score > 0.0f) {
+      CacheEntry e;
+      e.config = best;
+      e.score = tuner.best_score;
+      e.timestamp = now_seconds();
+      tuning_cache_put(key, e, true);
+    }
+  }
+  if (!(tuner.best_score > 0.0f)) return failure("autotune_conv2d: no candidate ran: " + bench.error);
+  best.layout_policy = "NHWC";
+  return success(best, tuner.best_score);
 }
 
 TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
