@@ -1,0 +1,83 @@
+"""Tuning entry points on the device: the exhaustive tracea_tune_* of the
+reference's FFI (src/interface/ffi.rs), and the cache-first AutoTuner adapters.
+The winner must be a compiled variant, be recorded under the reference's cache
+key, and be the variant the operator then runs."""
+import json
+
+import numpy as np
+import pytest
+
+import oracle
+from helpers import round_f16, tol_half, assert_close_scaled
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def cache_file(tmp_path, monkeypatch):
+    from tracea_amd import tuner as T
+    path = tmp_path / "tuning_cache_v2.json"
+    monkeypatch.setenv("TRACEA_TUNING_CACHE", str(path))
+    T.cache_reload()
+    yield path
+    monkeypatch.delenv("TRACEA_TUNING_CACHE")
+    T.cache_reload()
+
+
+def _device_name():
+    return torch.cuda.get_device_properties(0).name
+
+
+def test_tune_gemm_records_a_runnable_winner(tracea_gpu, cache_file):
+    from tracea_amd import capi, tuner as T
+    ok, score, cfg, err = capi.take_result(capi.lib().tracea_tune_gemm(1024, 1024, 512))
+    assert ok, err
+    cfg = json.loads(cfg)
+    assert score > 1.0  # TFLOP/s; any MFMA variant clears this on 1024x1024x512
+    assert T.validate(cfg) is None and T.variant_for_config(cfg) >= 0
+    disk = json.loads(cache_file.read_text())
+    keys = [k for k in disk if k.startswith("gemm_1024_1024_512_")]
+    assert len(keys) == 1
+    assert disk[keys[0]]["config"] == cfg and disk[keys[0]]["score"] == pytest.approx(score)
+    # the operator still computes the right product afterwards (forced variant restored)
+    rng = np.random.default_rng(5)
+    a = round_f16(rng.standard_normal((1024, 512)).astype(np.float32) / np.sqrt(512))
+    b = round_f16(rng.standard_normal((512, 1024)).astype(np.float32))
+    c = tracea_gpu.gemm(torch.from_numpy(a).cuda().half(), torch.from_numpy(b).cuda().half())
+    assert_close_scaled(c.float().cpu().numpy(), oracle.gemm_f64(a, b), tol_half(512, "f16"), "after tune")
+
+
+def test_autotune_gemm_is_cache_first_and_budgeted(tracea_gpu, cache_file):
+    from tracea_amd import tuner as T
+    best, score = T.autotune_gemm(512, 512, 256, iterations=4)
+    assert score > 0.2 and T.variant_for_config(best) >= 0
+    disk = json.loads(cache_file.read_text())
+    key = [k for k in disk if k.startswith("gemm_512_512_256_")][0]
+    # a planted entry under the same key is what the next call returns, unmeasured
+    planted = T.propose_gemm_configs(512, 512, 256)[-1]
+    T.cache_put(key, planted, 123.0, 1)
+    again, score2 = T.autotune_gemm(512, 512, 256, iterations=0)
+    assert again == planted and score2 == 123.0
+
+
+def test_autotune_conv2d_and_tune_conv2d_agree_on_the_key(tracea_gpu, cache_file):
+    from tracea_amd import capi, tuner as T
+    best, score = T.autotune_conv2d(2, 32, 16, 16, 32, 3, 3, stride=1, pad=1, iterations=0)
+    assert score > 0.01 and best["layout_policy"] == "NHWC"
+    ok, score2, cfg, err = capi.take_result(capi.lib().tracea_tune_conv2d(2, 32, 16, 16, 32, 3, 3, 1, 1, 1))
+    assert ok, err
+    disk = json.loads(cache_file.read_text())
+    keys = [k for k in disk if k.startswith("conv_2_16_16_32_32_3_3_1_1_")]
+    assert len(keys) == 1  # both wrote the reference's key conv_B_H_W_C_K_R_S_stride_pad_device
+    assert T.variant_for_config(json.loads(cfg)) >= 0
+
+
+def test_tune_fa2_returns_a_flash_variant(tracea_gpu, cache_file):
+    from tracea_amd import capi
+    ok, score, cfg, err = capi.take_result(capi.lib().tracea_tune_fa2(1, 2, 256, 64, True))
+    assert ok, err
+    cfg = json.loads(cfg)
+    assert cfg["attention_variant"] == "FlashV2" and score > 0.0
+    ok, _, _, err = capi.take_result(capi.lib().tracea_tune_fa2(1, 2, 256, 96, True))
+    assert not ok and "D 64 or 128" in err
