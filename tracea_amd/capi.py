@@ -149,6 +149,8 @@ SIGNATURES.update({
                                         MEASURE_FN, C.c_void_p, C.c_uint32, C.c_int, C.c_uint64]),
     "tracea_autotune_gemm": (Result, [C.c_size_t] * 3 + [C.c_uint32]),
     "tracea_autotune_conv2d": (Result, [C.c_size_t] * 10 + [C.c_uint32]),
+    # include/tracea_graph.h
+    "tracea_graph_fuse": (_STR, [C.c_char_p]),
 })
 
 _lib = None
