@@ -4,6 +4,7 @@ exports every symbol include/tracea.h and include/tracea_tuner.h declare, and it
 import ctypes as C
 import os
 import re
+import subprocess
 
 import numpy as np
 import pytest
@@ -140,3 +141,21 @@ def test_cpp_header_compiles_and_links(tmp_path):
                            "-L", libdir, "-ltracea", "-Wl,-rpath," + libdir])
     out = subprocess.check_output([str(exe)]).decode()
     assert "tracea.hpp ok" in out
+
+
+def test_tuner_cli_usage_and_failure_without_a_device(tmp_path):
+    """tracea-tuner keeps the reference CLI's sub-commands (src/bin/tuner.rs:11-30) and fails
+    cleanly when no device can be initialised."""
+    exe = os.path.join(ROOT, "tracea_amd", "bin", "tracea-tuner")
+    assert os.path.exists(exe), "run `python -m tracea_amd.build`"
+    r = subprocess.run([exe], capture_output=True, text=True)
+    assert r.returncode == 0 and "gemm <m> <n> <k> [--out <file>]" in r.stderr
+    r = subprocess.run([exe, "pool", "1"], capture_output=True, text=True)
+    assert r.returncode == 2 and "Unknown subcommand: pool" in r.stderr
+    r = subprocess.run([exe, "gemm", "64", "x"], capture_output=True, text=True)
+    assert r.returncode == 2
+    import torch
+    if not torch.cuda.is_available():
+        out = tmp_path / "r.json"
+        r = subprocess.run([exe, "gemm", "64", "64", "64", "--out", str(out)], capture_output=True, text=True)
+        assert r.returncode == 1 and "Runtime init failed" in r.stderr and not out.exists()

@@ -81,3 +81,26 @@ def test_tune_fa2_returns_a_flash_variant(tracea_gpu, cache_file):
     assert cfg["attention_variant"] == "FlashV2" and score > 0.0
     ok, _, _, err = capi.take_result(capi.lib().tracea_tune_fa2(1, 2, 256, 96, True))
     assert not ok and "D 64 or 128" in err
+
+
+def test_tuner_cli_writes_the_reference_record(tracea_gpu, cache_file, tmp_path):
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tracea_amd", "bin", "tracea-tuner")
+    out = tmp_path / "bench_results.json"
+    r = subprocess.run([exe, "gemm", "512", "512", "256", "--out", str(out)], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode == 0, r.stderr
+    assert "Starting Tuner for GEMM 512x512x256" in r.stdout and "Results saved to" in r.stdout
+    rec = json.loads(out.read_text())
+    assert list(rec)[:4] == ["timestamp", "kernel", "problem", "best_config"]  # src/bin/tuner.rs:93-102
+    assert rec["kernel"] == "gemm" and rec["problem"] == {"m": 512, "n": 512, "k": 256}
+    from tracea_amd import tuner as T
+    assert T.variant_for_config(rec["best_config"]) >= 0 and rec["score_tflops"] > 0
+    # the child process wrote the cache file this process points at
+    assert any(k.startswith("gemm_512_512_256_") for k in json.loads(cache_file.read_text()))
+    r = subprocess.run([exe, "attention", "1", "2", "256", "64", "--causal", "--out", str(out)], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    rec = json.loads(out.read_text())
+    assert rec["kernel"] == "attention" and rec["problem"]["causal"] is True

@@ -21,6 +21,8 @@ _OUT = os.environ.get("TRACEA_BUILD_OUT") or HERE
 OBJ = os.path.join(_OUT, "_obj")
 LIB_DIR = os.path.join(_OUT, "lib")
 LIB = os.path.join(LIB_DIR, "libtracea.so")
+BIN_DIR = os.path.join(_OUT, "bin")
+TUNER_BIN = os.path.join(BIN_DIR, "tracea-tuner")
 
 ARCH = "gfx950"
 # -packed-fp32-ops: keep the compiler from forming packed fp32 VALU instructions.
@@ -107,6 +109,16 @@ def build(force=False, jobs=None, verbose=True):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stderr[-4000:])
+    # command-line tuner: plain C++ over the public headers, linked against the library
+    os.makedirs(BIN_DIR, exist_ok=True)
+    src = os.path.join(CSRC, "tools", "tuner_main.cpp")
+    if (rebuilt or force or not os.path.exists(TUNER_BIN)
+            or os.path.getmtime(TUNER_BIN) < os.path.getmtime(src)):
+        cmd = ["g++", "-std=c++17", "-O2", "-Wall", "-I", INCLUDE, src, "-o", TUNER_BIN, "-L", LIB_DIR, "-ltracea",
+               "-Wl,-rpath,$ORIGIN/../lib"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("tuner link failed:\n" + r.stderr[-4000:])
     if verbose:
         print("libtracea.so: %d of %d objects rebuilt -> %s" % (rebuilt, len(todo), LIB))
     return LIB
