@@ -247,6 +247,11 @@ int32_t tracea_force_variant(const char *op, int32_t index);    /* 0 ok, -1 bad 
  * its implicit-GEMM view (m rows, n channels, k reduction), K-contiguous B, before
  * any forced variant is applied; -1 on a bad argument. */
 int32_t tracea_select_variant(const char *op, int64_t m, int64_t n, int64_t k);
+/* The variant the calling thread's most recent call of `op` actually launched
+ * (a forced or cached variant that cannot run a problem is replaced by the
+ * nearest one that can); -1 before any call, or when the call was served by a
+ * kernel outside the variant table (fp32 and strided GEMM). */
+int32_t tracea_last_variant(const char *op);
 
 /* The 80-byte ConvParams block of the reference (src/emitter/cuda/conv.rs:134-142;
  * packing src/interface/python.rs:423-435) as this library computes it, for

@@ -56,7 +56,7 @@ SMALL = [  # n, h, w, c, k, r, s, stride, pad, dilation
 ]
 
 
-@pytest.mark.parametrize("variant", range(16))
+@pytest.mark.parametrize("variant", range(24))
 def test_small_shapes_every_variant_both_filter_layouts(tracea_gpu, variant):
     from tracea_amd import capi
     names = capi.variants("conv2d")
@@ -84,6 +84,55 @@ def test_small_shapes_every_variant_both_filter_layouts(tracea_gpu, variant):
             assert_close_scaled(y.float().cpu().numpy(), want, tol, "%s rsck %s" % (names[variant], shape))
     finally:
         capi.force_variant("conv2d", -1)
+
+
+PATCH_SHAPES = [  # n, h, w, c, k, r, s, stride, pad, dilation: all with C % 16 == 0
+    (2, 20, 20, 64, 64, 3, 3, 1, 1, 1),    # 400 pixels: several tiles per image, last one partial
+    (1, 33, 17, 32, 72, 3, 3, 1, 1, 1),    # K = 288: partial last filter tile, N not a tile multiple
+    (3, 14, 14, 64, 128, 3, 3, 2, 1, 1),   # stride 2
+    (2, 12, 12, 16, 40, 5, 3, 1, 2, 1),    # 5x3 taps, K = 240
+    (2, 13, 11, 48, 24, 3, 3, 1, 2, 2),    # dilation 2, C/8 even -> padded pixel pitch
+    (4, 9, 9, 128, 96, 1, 1, 1, 0, 1),     # 1x1
+    (1, 40, 40, 16, 16, 3, 3, (2, 1), (0, 2), 1),  # asymmetric stride and padding
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_patch_resident_variants(tracea_gpu, dtype):
+    """The LDS-patch convolution kernels against the oracle, forced one by one (a variant
+    whose patch does not fit a shape falls back to the streamed kernel of the same tile)."""
+    from tracea_amd import capi
+    names = capi.variants("conv2d")
+    patch = [i for i, nm in enumerate(names) if nm.endswith("_patch")]
+    assert patch, "no patch-resident variant in the build"
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rnd = round_f16 if dtype == "f16" else round_bf16
+    ran = set()
+    try:
+        for vi in patch:
+            capi.force_variant("conv2d", vi)
+            for shape in PATCH_SHAPES:
+                n, h, w, c, k, r, s, stride, pad, dil = shape
+                rng = np.random.default_rng(vi * 1000 + h * 7 + c)
+                x = rnd(rng.standard_normal((n, h, w, c)))
+                wk = rnd(rng.standard_normal((k, r, s, c)) * np.sqrt(2.0 / (r * s * c)))
+                bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+                ref = torch.nn.functional.conv2d(
+                    torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
+                    bias=torch.from_numpy(bias).double(), stride=stride, padding=pad, dilation=dil)
+                ref = torch.relu(ref).permute(0, 2, 3, 1).numpy()
+                if isinstance(stride, int):  # the oracle takes symmetric geometry: cross-check torch with it once
+                    acc = oracle.conv2d_nhwc(x, np.ascontiguousarray(wk.transpose(1, 2, 3, 0)), stride, pad, dil)
+                    want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+                    assert np.abs(want - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+                y = tracea_gpu.conv2d(_dev(x, tdt), _dev(wk, tdt), bias=_dev(bias), stride=stride, padding=pad,
+                                      dilation=dil, epilogue="bias+relu")
+                assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(r * s * c, dtype),
+                                    "%s %s %s" % (names[vi], dtype, shape))
+                ran.add(capi.last_variant("conv2d"))
+    finally:
+        capi.force_variant("conv2d", -1)
+    assert {names[i] for i in patch} <= ran, "a patch-resident variant never ran: %s" % sorted(ran)
 
 
 def test_asymmetric_stride_and_padding_bf16(tracea_gpu):

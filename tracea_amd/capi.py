@@ -99,6 +99,7 @@ SIGNATURES = {
     "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),
     "tracea_force_variant": (C.c_int32, [C.c_char_p, C.c_int32]),
     "tracea_select_variant": (C.c_int32, [C.c_char_p, C.c_int64, C.c_int64, C.c_int64]),
+    "tracea_last_variant": (C.c_int32, [C.c_char_p]),
     "tracea_conv_params_pack": (C.c_int, [C.c_int32] * 10 + [C.POINTER(ConvParamsBlock)]),
     "tracea_conv_coords_device": (C.c_int, [C.POINTER(ConvParamsBlock), C.c_void_p, C.c_void_p,
                                             C.c_void_p, C.c_void_p]),
@@ -228,6 +229,12 @@ def take_string(ptr):
 def variants(op):
     n = lib().tracea_variant_count(op.encode())
     return [lib().tracea_variant_name(op.encode(), i).decode() for i in range(max(n, 0))]
+
+
+def last_variant(op):
+    """Name of the variant the latest call of `op` on this thread launched, or None."""
+    i = lib().tracea_last_variant(op.encode())
+    return variants(op)[i] if i >= 0 else None
 
 
 def force_variant(op, index_or_name):

@@ -142,6 +142,8 @@ int32_t tracea_force_variant(const char *op, int32_t index) {
   return 0;
 }
 
+int32_t tracea_last_variant(const char *op) { return op == nullptr ? -1 : last_variant(op); }
+
 int32_t tracea_select_variant(const char *op, int64_t m, int64_t n, int64_t k) {
   if (op == nullptr || m <= 0 || n <= 0 || k <= 0 || m >= (1ll << 31) || n >= (1ll << 31) || k >= (1ll << 31))
     return -1;

@@ -43,6 +43,12 @@ struct ContractionArgs {
   int h_in, w_in, c_in, h_out, w_out, s_sz;
   int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
   unsigned hw_m, hw_s, w_m, w_s, sc_m, sc_s, c_m, c_s;
+  // patch-resident convolution (pipeline 4) only: filter rows, M tiles per image,
+  // padded row width W + 2 pad_w, 16-byte chunks per patch pixel (odd), patch
+  // load iterations per thread, LDS bytes reserved for the patch, and the
+  // reciprocals of the chunk count and of the padded width
+  int r_sz, p_tiles, p_pw, p_cpp, p_iters, p_np_bytes;
+  unsigned p_cpp_m, p_cpp_s, p_pw_m, p_pw_s;
   EpilogueChain epi;
 };
 
@@ -65,6 +71,7 @@ struct ContractionVariant {
   int pipeline;  // 0: operands read just in time; 1: read one k-step ahead, across the barrier;
                  // 2: as 1, with direct-to-LDS tile loads (K-contiguous B only);
                  // 3: ring of `stages` LDS buffers, direct-to-LDS loads stages-1 tiles ahead
+                 // 4: convolution only: input patch resident in LDS, filter tiles through a ring of `stages`
   size_t lds_bytes;
   // launch: returns hipError_t as int
   int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);

@@ -2,6 +2,7 @@
 // compiles this file once per line of contraction_variants.def with
 // -DV_NAME=... -DV_BM=... -DV_BN=... -DV_BK=... -DV_WM=... -DV_WN=... -DV_STAGES=... -DV_DIRECT=<pipeline mode>
 #include "contraction_kernel.hpp"
+#include "conv_patch_kernel.hpp"
 
 #define TRACEA_CAT2(a, b) a##b
 #define TRACEA_CAT(a, b) TRACEA_CAT2(a, b)
@@ -13,8 +14,13 @@ namespace tracea_amd {
 const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
   static const ContractionVariant v = {
       TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT,
+#if V_DIRECT == 4
+      (size_t)V_STAGES * V_BN * V_BK * 2,  // filter ring only; the patch size depends on the problem
+      &launch_conv_patch<V_BM, V_BN, V_WM, V_WN, V_STAGES>};
+#else
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
       &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT>};
+#endif
   return v;
 }
 }  // namespace tracea_amd

@@ -237,6 +237,9 @@ TraceaStatus check_bias_residual(const char *what, const TraceaTensorView *bias,
 std::atomic<int> g_forced_contraction{-1};
 std::atomic<int> g_forced_conv{-1};
 std::atomic<int> g_forced_attention{-1};
+// variant the calling thread's latest launch of each operator used (-1: none,
+// or a kernel outside the variant tables)
+thread_local int t_last_contraction = -1, t_last_conv = -1, t_last_attention = -1;
 
 TraceaStatus hip_status(const char *what, int e) {
   if (e == 0) return TRACEA_SUCCESS;
@@ -249,6 +252,12 @@ void set_forced_variant(const char *op, int index) {
   if (!strcmp(op, "gemm")) g_forced_contraction.store(index);
   else if (!strcmp(op, "conv2d")) g_forced_conv.store(index);
   else if (!strcmp(op, "attention")) g_forced_attention.store(index);
+}
+int last_variant(const char *op) {
+  if (!strcmp(op, "gemm")) return t_last_contraction;
+  if (!strcmp(op, "conv2d")) return t_last_conv;
+  if (!strcmp(op, "attention")) return t_last_attention;
+  return -1;
 }
 int forced_variant(const char *op) {
   if (!strcmp(op, "gemm")) return g_forced_contraction.load();
@@ -324,6 +333,7 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
   double best_cost = 0.0;
   for (int i = 0; i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
+    if (v.pipeline == 4) continue;  // needs the convolution geometry: see plan_conv_patch
     const double gm = (double)((m + v.bm - 1) / v.bm), gn = (double)((n + v.bn - 1) / v.bn);
     const double tiles = gm * gn;
     const double exact = tiles / cus > 1.0 ? tiles / cus : 1.0;
@@ -370,6 +380,7 @@ int twin(int vi, int pipeline) {
 // pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
 int resolve_variant(int vi, bool conv, bool b_ncontig, bool k_exact) {
   int pipe = contraction_variant(vi).pipeline;
+  if (pipe == 4) pipe = 2;  // the caller found the patch-resident kernel unusable: same tile, streamed operands
   if (pipe >= 2 && b_ncontig) pipe = 1;
   if (pipe == 1 && !conv && !k_exact) pipe = 0;
   if (pipe == contraction_variant(vi).pipeline) return vi;
@@ -396,6 +407,7 @@ void fill_grid(ContractionArgs *a, const ContractionVariant &v) {
 TraceaStatus run_gemm(const View &a, const View &b, const View &c, const EpilogueChain &chain,
                       hipStream_t stream) {
   const long long M = a.shape[0], K = a.shape[1], N = b.shape[1];
+  t_last_contraction = -1;
   if (M == 0 || N == 0) return TRACEA_SUCCESS;
   DeviceScope scope(c.device);
   if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
@@ -427,6 +439,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.a_bytes = (unsigned)(small ? a_extent : 0);
       args.b_bytes = (unsigned)(small ? b_extent : 0);
       fill_grid(&args, v);
+      t_last_contraction = vi;
       return hip_status("gemm launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
     }
   }
@@ -583,6 +596,61 @@ TraceaStatus conv_common(const TraceaTensorView &tx, const TraceaTensorView &tw,
   return TRACEA_SUCCESS;
 }
 
+// Fills the patch-resident convolution fields of `a` for variant `v` and sets
+// the grid; false when the kernel cannot run this problem (then nothing the
+// caller relies on has been changed).
+//   * K-contiguous filters, C a multiple of 16 (a 16-wide k-step stays inside
+//     one tap);
+//   * one image and the filter bank each below 2 GiB (32-bit buffer offsets);
+//   * the patch of the worst tile plus the filter ring fits in LDS.
+// The patch bound: BM consecutive output pixels take at most nw row wraps; a
+// step inside a row advances the padded linear index by stride_w, a wrap by
+// stride_h*PW - (Wo-1)*stride_w; the taps add (R-1)*dil_h*PW + (S-1)*dil_w.
+bool plan_conv_patch(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  const TraceaConvParamsBlock &b = g.block;
+  const int C = b.c_in;
+  if (v.pipeline != 4 || w_ncontig || C % 16 != 0) return false;
+  const long long img_bytes = (long long)b.h_in * b.w_in * C * 2;
+  const long long w_bytes = (long long)g.n_gemm * g.k_gemm * 2;
+  if (img_bytes >= (1ll << 31) || w_bytes >= (1ll << 31)) return false;
+  const long long pw = (long long)b.w_in + 2ll * g.pad_w;
+  const long long ph = (long long)b.h_in + 2ll * g.pad_h;
+  if (pw * ph >= (1ll << 30)) return false;
+  const int hw = b.h_out * b.w_out;
+  const int tm = v.bm < hw ? v.bm : hw;
+  const long long steps = tm - 1;
+  long long nw = (steps + b.w_out - 1) / b.w_out;
+  if (nw > steps) nw = steps;
+  if (nw > b.h_out - 1) nw = b.h_out - 1;
+  const long long in_row = g.stride_w;
+  long long wrap = (long long)g.stride_h * pw - (long long)(b.w_out - 1) * g.stride_w;
+  if (wrap < in_row) wrap = in_row;
+  const long long span = (steps - nw) * in_row + nw * wrap;
+  const long long taps = (long long)(b.r_sz - 1) * g.dil_h * pw + (long long)(b.s_sz - 1) * g.dil_w;
+  const long long np = span + taps + 1;
+  const int cpp = (C / 8) | 1;
+  const int nt = v.waves_m * v.waves_n * 64;
+  const long long chunks = np * cpp;
+  const long long iters = (chunks + nt - 1) / nt;
+  const long long patch_bytes = iters * nt * 16;
+  const long long ring = (long long)v.stages * v.bn * 128;
+  if (patch_bytes + ring > 160 * 1024) return false;
+  a->r_sz = b.r_sz;
+  a->p_tiles = (hw + v.bm - 1) / v.bm;
+  a->p_pw = (int)pw;
+  a->p_cpp = cpp;
+  a->p_iters = (int)iters;
+  a->p_np_bytes = (int)patch_bytes;
+  magic_for_divisor((uint32_t)cpp, (uint64_t)(iters * nt), &a->p_cpp_m, &a->p_cpp_s);
+  magic_for_divisor((uint32_t)pw, (uint64_t)(pw * ph + np), &a->p_pw_m, &a->p_pw_s);
+  a->grid_m = b.batch * a->p_tiles;
+  a->grid_n = (g.n_gemm + v.bn - 1) / v.bn;
+  a->group_m = 1;
+  a->b_bytes = (unsigned)w_bytes;
+  a->a_bytes = 0;
+  return true;
+}
+
 TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStream_t stream) {
   const ConvGeometry &g = plan.geo;
   DeviceScope scope(plan.out.device);
@@ -608,11 +676,17 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   const long long x_extent = (long long)g.block.batch * g.block.h_in * g.block.w_in * g.block.c_in * 2;
   const long long w_extent = (long long)g.n_gemm * g.k_gemm * 2;
   const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
+  if (contraction_variant(vi).pipeline == 4 && plan_conv_patch(g, contraction_variant(vi), plan.w_ncontig, &a)) {
+    t_last_conv = vi;
+    return hip_status("conv2d launch",
+                      contraction_variant(vi).launch(a, true, plan.x.dtype, false, stream));
+  }
   vi = resolve_variant(vi, true, plan.w_ncontig || !small, true);
   const ContractionVariant &v = contraction_variant(vi);
   a.a_bytes = (unsigned)(small ? x_extent : 0);
   a.b_bytes = (unsigned)(small ? w_extent : 0);
   fill_grid(&a, v);
+  t_last_conv = vi;
   return hip_status("conv2d launch", v.launch(a, true, plan.x.dtype, plan.w_ncontig, stream));
 }
 
@@ -711,6 +785,7 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
   if (vi < 0) return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: no kernel variant fits");
   DeviceScope scope(o.device);
   if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  t_last_attention = vi;
   return hip_status("attention launch",
                     attention_variant(vi).launch(a, q.dtype, (hipStream_t)params.stream));
 }

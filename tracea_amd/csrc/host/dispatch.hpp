@@ -31,6 +31,8 @@ void magic_for_divisor(uint32_t d, uint64_t n_max, uint32_t *magic, uint32_t *sh
 
 void set_forced_variant(const char *op, int index);
 int forced_variant(const char *op);
+// Variant index the calling thread's latest launch of `op` used, -1 if none.
+int last_variant(const char *op);
 
 TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorView &b,
                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
