@@ -22,6 +22,8 @@
 //     regroups the accumulators through LDS into 8 consecutive channels per
 //     lane, applies the fused operator chain on fp32 and stores 16 bytes.
 #pragma once
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace tracea_amd {
@@ -34,6 +36,17 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+// Compile-time loop: body(std::integral_constant<int, I>) for I = 0..N-1.  Used where an
+// accumulator array must be indexed by constants however large the loop body is
+// (a run-time index would move the whole array to scratch memory).
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&body) {
+  if constexpr (I < N) {
+    body(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(body);
+  }
+}
 
 template <int DT>
 struct Mfma32;
@@ -118,13 +131,12 @@ __device__ __forceinline__ void load_as_float(const void *base, int dtype, long 
   }
 }
 
-// Applies the operator chain, in order, to V consecutive channels n..n+V-1 of
-// output row m (fp32 in, fp32 out).
+// Applies one operator to V consecutive channels n..n+V-1 of output row m
+// (fp32 in, fp32 out), reading its operands from global memory.
 template <int V>
-__device__ __forceinline__ void apply_epilogue(float (&v)[V], long long m, int n, int nvalid,
-                                               const EpilogueChain &chain) {
-  for (int o = 0; o < chain.n_ops; ++o) {
-    const EpilogueOpDev &op = chain.ops[o];
+__device__ __forceinline__ void apply_epilogue_one(float (&v)[V], long long m, int n, int nvalid,
+                                                   const EpilogueOpDev &op) {
+  {
     float t[V];
     switch (op.kind) {
       case TRACEA_EPI_OP_BIAS_ADD:
@@ -181,6 +193,14 @@ __device__ __forceinline__ void apply_epilogue(float (&v)[V], long long m, int n
   }
 }
 
+// Applies the operator chain, in order, to V consecutive channels n..n+V-1 of
+// output row m (fp32 in, fp32 out), every operand read from global memory.
+template <int V>
+__device__ __forceinline__ void apply_epilogue(float (&v)[V], long long m, int n, int nvalid,
+                                               const EpilogueChain &chain) {
+  for (int o = 0; o < chain.n_ops; ++o) apply_epilogue_one<V>(v, m, n, nvalid, chain.ops[o]);
+}
+
 // Converts V floats to the output type (round to nearest even) and stores
 // them at element index idx; only the first nvalid are written.
 template <int V>
@@ -231,6 +251,190 @@ __device__ __forceinline__ void store_from_float(void *base, int dtype, long lon
       for (int e = 0; e < V; ++e)
         if (e < nvalid) p[e] = h[e];
     }
+  }
+}
+
+// ---- per-channel operands of the chain, staged in LDS ----------------------------
+// In the tile epilogue every row a lane stores needs the same per-channel
+// operands (bias, BatchNorm or scale/shift vectors).  Reading them from global
+// memory inside the row loop makes that loop a chain of dependent L2 round
+// trips, one per row.  Instead each thread loads a few entries of a small
+// table before the main loop (the loads complete under it), the table is
+// written to LDS once the main loop has released it, and the row loop reads its
+// operands from there.  Layout: table[(o * 2 + which) * BN + channel], fp32;
+// which 0 = bias or scale, which 1 = shift.  BatchNorm is folded to
+// scale = gamma / sqrt(var + eps), shift = beta - mean * scale (one fp32
+// rounding away from the unfolded form).
+__device__ __forceinline__ float chain_table_value(const EpilogueChain &chain, int o, int which, int n, int N) {
+  if (o >= chain.n_ops || n >= N) return 0.0f;
+  const EpilogueOpDev &op = chain.ops[o];
+  float one[1];
+  if (op.kind == TRACEA_EPI_OP_BIAS_ADD || op.kind == TRACEA_EPI_OP_BIAS_ADD_SILU) {
+    if (which != 0) return 0.0f;
+    load_as_float<1>(op.p0, op.dtype, n, 1, one);
+    return one[0];
+  }
+  if (op.kind == TRACEA_EPI_OP_SCALE_SHIFT) return ((const float *)(which == 0 ? op.p0 : op.p1))[n];
+  if (op.kind == TRACEA_EPI_OP_BATCHNORM) {
+    const float scale = ((const float *)op.p0)[n] * (1.0f / sqrtf(((const float *)op.p3)[n] + op.epsilon));
+    return which == 0 ? scale : ((const float *)op.p1)[n] - ((const float *)op.p2)[n] * scale;
+  }
+  return 0.0f;
+}
+
+// The chain as the row loop needs it, read once from the kernel arguments: the
+// operator kinds and the descriptor of the first residual operator.  Indexing
+// args.epi.ops[] with a run-time operator number inside the row loop re-reads
+// kind, pointer, dtype and stride through dependent scalar loads for every
+// (row, operator) pair, which cost more than everything else in the epilogue.
+struct ChainPlan {
+  unsigned kinds;      // operator o in bits 4o..4o+3 (TraceaEpilogueOpKind < 16), 0 past the end
+  int n_ops;
+  int res_index;       // first residual operator, -1 if none
+  const void *res_ptr;
+  int res_dtype;
+  long long res_ld;
+};
+
+__device__ __forceinline__ ChainPlan chain_plan(const EpilogueChain &chain) {
+  ChainPlan p;
+  p.kinds = 0;
+  p.n_ops = chain.n_ops;
+  p.res_index = -1;
+  p.res_ptr = nullptr;
+  p.res_dtype = DT_F32;
+  p.res_ld = 0;
+#pragma unroll
+  for (int o = TRACEA_MAX_EPILOGUE_OPS - 1; o >= 0; --o) {
+    const int kind = o < chain.n_ops ? chain.ops[o].kind : (int)TRACEA_EPI_OP_NONE;
+    p.kinds |= (unsigned)(kind & 15) << (4 * o);
+    if (kind == TRACEA_EPI_OP_RESIDUAL_ADD) {
+      p.res_index = o;
+      p.res_ptr = chain.ops[o].p0;
+      p.res_dtype = chain.ops[o].dtype;
+      p.res_ld = chain.ops[o].ld;
+    }
+  }
+  return p;
+}
+
+// The chain on 8 consecutive channels of row m; per-channel operands come from
+// the LDS table (tab points at this lane's first channel, vectors bn apart),
+// the first residual tensor through the plan, any further one from the
+// kernel arguments.  The operator loop is a real loop (its body is emitted
+// once) over kinds held in one scalar.
+__device__ __forceinline__ void apply_epilogue_tab(float (&v)[8], long long m, int n, int nvalid,
+                                                   const EpilogueChain &chain, const ChainPlan &plan,
+                                                   const float *tab, int bn) {
+#pragma nounroll
+  for (int o = 0; o < plan.n_ops; ++o) {
+    const int kind = (int)((plan.kinds >> (4 * o)) & 15u);
+    if (kind == TRACEA_EPI_OP_RELU) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = fmaxf(0.0f, v[e]);
+    } else if (kind == TRACEA_EPI_OP_BIAS_ADD || kind == TRACEA_EPI_OP_BIAS_ADD_SILU ||
+               kind == TRACEA_EPI_OP_SCALE_SHIFT || kind == TRACEA_EPI_OP_BATCHNORM) {
+      const float *pa = tab + (o * 2) * bn;
+      const f32x4 a0 = *(const f32x4 *)pa, a1 = *(const f32x4 *)(pa + 4);
+      const f32x4 b0 = *(const f32x4 *)(pa + bn), b1 = *(const f32x4 *)(pa + bn + 4);  // zeros for a bias
+      const float a[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+      const float b[8] = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+      if (kind == TRACEA_EPI_OP_BIAS_ADD) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] + a[e];
+      } else if (kind == TRACEA_EPI_OP_BIAS_ADD_SILU) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float x = v[e] + a[e];
+          v[e] = x / (1.0f + expf(-x));
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] * a[e] + b[e];
+      }
+    } else if (kind == TRACEA_EPI_OP_RESIDUAL_ADD && o == plan.res_index) {
+      float t[8];
+      load_as_float<8>(plan.res_ptr, plan.res_dtype, m * plan.res_ld + n, nvalid, t);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = v[e] + t[e];
+    } else {
+      apply_epilogue_one<8>(v, m, n, nvalid, chain.ops[o]);  // GELU, SiLU, a second residual
+    }
+  }
+}
+
+// ---- specialised row body ------------------------------------------------------------
+// The general row body above carries every fallback inline (partial channel
+// vectors, unaligned rows, per-element loads and stores, GELU / SiLU): several
+// thousand instructions and hundreds of branches per row, more than the
+// instruction cache holds.  Nearly every call needs none of it: all 8 channels
+// of every lane exist, rows of C (and of the residual) are 16-byte aligned, and
+// the chain is made of bias / scale-shift / BatchNorm / ReLU / one residual.
+// Whether that holds is the same for the whole workgroup, so it is decided
+// once and the row loops are emitted twice, each behind a uniform branch.
+__device__ __forceinline__ bool chain_is_simple(const ChainPlan &plan, const ContractionArgs &args, int n0, int bn) {
+  bool ok = n0 + bn <= args.N && (args.ldc & 7) == 0 && (((uintptr_t)args.C) & 15) == 0 &&
+            args.out_dtype != DT_F32;
+#pragma unroll
+  for (int o = 0; o < TRACEA_MAX_EPILOGUE_OPS; ++o) {
+    const int kind = (int)((plan.kinds >> (4 * o)) & 15u);
+    ok = ok && (kind == TRACEA_EPI_OP_NONE || kind == TRACEA_EPI_OP_BIAS_ADD || kind == TRACEA_EPI_OP_RELU ||
+                kind == TRACEA_EPI_OP_SCALE_SHIFT || kind == TRACEA_EPI_OP_BATCHNORM ||
+                (kind == TRACEA_EPI_OP_RESIDUAL_ADD && o == plan.res_index));
+  }
+  if (plan.res_index >= 0)
+    ok = ok && plan.res_dtype != DT_F32 && (plan.res_ld & 7) == 0 && (((uintptr_t)plan.res_ptr) & 15) == 0;
+  return ok;
+}
+
+// One row on the specialised path: 8 channels, 16-bit output, every access a
+// single 16-byte operation.
+template <int DT>
+__device__ __forceinline__ void simple_row(float (&v)[8], long long m, int n, const ContractionArgs &args,
+                                           const ChainPlan &plan, const float *tab, int bn) {
+#pragma nounroll
+  for (int o = 0; o < plan.n_ops; ++o) {
+    const int kind = (int)((plan.kinds >> (4 * o)) & 15u);
+    if (kind == TRACEA_EPI_OP_RELU) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = fmaxf(0.0f, v[e]);
+    } else if (kind == TRACEA_EPI_OP_RESIDUAL_ADD) {
+      const u32x4 raw = *(const u32x4 *)((const unsigned short *)plan.res_ptr + m * plan.res_ld + n);
+      if (plan.res_dtype == DT_F16) {
+        const f16x8 h = __builtin_bit_cast(f16x8, raw);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] + (float)h[e];
+      } else {
+        const bf16x8 h = __builtin_bit_cast(bf16x8, raw);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] + (float)h[e];
+      }
+    } else {  // bias: v + a; scale/shift and BatchNorm: v * a + b
+      const float *pa = tab + (o * 2) * bn;
+      const f32x4 a0 = *(const f32x4 *)pa, a1 = *(const f32x4 *)(pa + 4);
+      const float a[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+      if (kind == TRACEA_EPI_OP_BIAS_ADD) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] + a[e];
+      } else {
+        const f32x4 b0 = *(const f32x4 *)(pa + bn), b1 = *(const f32x4 *)(pa + bn + 4);
+        const float b[8] = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = v[e] * a[e] + b[e];
+      }
+    }
+  }
+  unsigned short *dst = (unsigned short *)args.C + m * args.ldc + n;
+  if constexpr (DT == DT_F16) {
+    f16x8 h;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[e];
+    *(f16x8 *)dst = h;
+  } else {
+    bf16x8 h;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) h[e] = (__bf16)v[e];
+    *(bf16x8 *)dst = h;
   }
 }
 
@@ -348,6 +552,17 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int NCH = BN / 8;
 
   u32x4 ra[NA], rb[NB];
+
+  // This thread's entries of the epilogue operand table (see chain_table_value):
+  // requested here so that they arrive under the main loop.
+  constexpr int TAB_ENTRIES = TRACEA_MAX_EPILOGUE_OPS * 2 * BN;
+  constexpr int TPT = (TAB_ENTRIES + NT - 1) / NT;
+  float tabr[TPT];
+#pragma unroll
+  for (int i = 0; i < TPT; ++i) {
+    const int idx = tid + i * NT;
+    tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;
+  }
 
   // Every load is issued unconditionally from an address that is always
   // inside the tensor (the real one, or the tensor base when the piece lies in
@@ -805,45 +1020,73 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int EP_PITCH = TN + 4;                 // floats
   constexpr int LPR = TN / 8;                      // lanes per output row
   constexpr int RPI = 64 / LPR;                    // rows per pass
-  static_assert((size_t)WM * WN * 32 * EP_PITCH * 4 <= (size_t)NS * STAGE, "staging must fit");
+  constexpr int STAGING_FLOATS = WM * WN * 32 * EP_PITCH;
+  static_assert((size_t)(STAGING_FLOATS + TAB_ENTRIES) * 4 <= (size_t)NS * STAGE, "staging and operand table must fit");
   float *stage = (float *)smem + wave * (32 * EP_PITCH);
+  float *table = (float *)smem + STAGING_FLOATS;
   const int er = lane / LPR, ec = (lane % LPR) * 8;
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
+  for (int i = 0; i < TPT; ++i)
+    if (tid + i * NT < TAB_ENTRIES) table[tid + i * NT] = tabr[i];
+  __syncthreads();
+  const float *tab = table + wn * TN + ec;
+  const ChainPlan plan = chain_plan(args.epi);
+  // the output type equals the operand type on the specialised path (simple_row<DT> stores DT)
+  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
+  static_for<0, FM>([&](auto blk) {
+    constexpr int i = decltype(blk)::value;
+    static_for<0, FN>([&](auto col) {
+      constexpr int j = decltype(col)::value;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
                    acc[i][j][g * 4 + 3]};
         *(f32x4 *)(stage + lrow * EP_PITCH + j * 32 + g * 8 + lhalf * 4) = v;
       }
+    });
     // The staging area is private to the wave and a wave's LDS operations
     // complete in program order: a compiler-level fence is all that is needed
     // between the writes above and the reads below (and before the next pass
     // overwrites what this one reads).
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    for (int r = er; r < 32; r += RPI) {
-      const int m = m0 + wm * TM + i * 32 + r;
-      const int n = n0 + wn * TN + ec;
-      if (m < M && n < N) {
-        float v[8];
-        const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
-        const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
+    if (simple) {
+      for (int r = er; r < 32; r += RPI) {
+        const int m = m0 + wm * TM + i * 32 + r;
+        if (m < M) {
+          float v[8];
+          const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
+          const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = lo[e];
-          v[4 + e] = hi[e];
+          for (int e = 0; e < 4; ++e) {
+            v[e] = lo[e];
+            v[4 + e] = hi[e];
+          }
+          simple_row<DT>(v, m, n0 + wn * TN + ec, args, plan, tab, BN);
         }
-        const int nvalid = N - n;
-        apply_epilogue<8>(v, m, n, nvalid, args.epi);
-        store_from_float<8>(args.C, args.out_dtype, (long long)m * args.ldc + n, nvalid, v);
+      }
+    } else {
+      for (int r = er; r < 32; r += RPI) {
+        const int m = m0 + wm * TM + i * 32 + r;
+        const int n = n0 + wn * TN + ec;
+        if (m < M && n < N) {
+          float v[8];
+          const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
+          const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = lo[e];
+            v[4 + e] = hi[e];
+          }
+          const int nvalid = N - n;
+          apply_epilogue_tab(v, m, n, nvalid, args.epi, plan, tab, BN);
+          store_from_float<8>(args.C, args.out_dtype, (long long)m * args.ldc + n, nvalid, v);
+        }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-  }
+  });
 }
 
 template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE>

@@ -122,6 +122,16 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
 #pragma unroll
   for (int st = 0; st < NSB - 1; ++st) dma_b(st, (st < nk ? st : nk - 1) * BK);
 
+  // this thread's entries of the epilogue operand table, requested under the main loop
+  constexpr int TAB_ENTRIES = TRACEA_MAX_EPILOGUE_OPS * 2 * BN;
+  constexpr int TPT = (TAB_ENTRIES + NT - 1) / NT;
+  float tabr[TPT];
+#pragma unroll
+  for (int i = 0; i < TPT; ++i) {
+    const int idx = tid + i * NT;
+    tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;
+  }
+
   // ---- per-lane operand addresses ----
   // A: the lane's pixel of each 32-row block (rows past the tile re-read its last pixel)
   int a_base[FM];
@@ -211,48 +221,77 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
   constexpr int EP_PITCH = TN + 4;
   constexpr int LPR = TN / 8;
   constexpr int RPI = 64 / LPR;
+  constexpr int STAGING_FLOATS = WM * WN * 32 * EP_PITCH;
   float *stage = (float *)smem + wave_u * (32 * EP_PITCH);
+  float *table = (float *)smem + STAGING_FLOATS;
   const int er = lane / LPR, ec = (lane % LPR) * 8;
   const long long m_img = (long long)img * hw + p0;
 #pragma unroll
-  for (int i = 0; i < FM; ++i) {
-#pragma unroll
-    for (int j = 0; j < FN; ++j)
+  for (int i = 0; i < TPT; ++i)
+    if (tid + i * NT < TAB_ENTRIES) table[tid + i * NT] = tabr[i];
+  __syncthreads();
+  const float *tab = table + wn * TN + ec;
+  const ChainPlan plan = chain_plan(args.epi);
+  // the output type equals the operand type on the specialised path (simple_row<DT> stores DT)
+  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
+  static_for<0, FM>([&](auto blk) {
+    constexpr int i = decltype(blk)::value;
+    static_for<0, FN>([&](auto col) {
+      constexpr int j = decltype(col)::value;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
         *(f32x4 *)(stage + lrow * EP_PITCH + j * 32 + g * 8 + lhalf * 4) = v;
       }
+    });
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    for (int r = er; r < 32; r += RPI) {
-      const int pr = wm * TMW + i * 32 + r;
-      const int n = n0 + wn * TN + ec;
-      if (pr < npix && n < N) {
-        float v[8];
-        const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
-        const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
+    if (simple) {
+      for (int r = er; r < 32; r += RPI) {
+        const int pr = wm * TMW + i * 32 + r;
+        if (pr < npix) {
+          float v[8];
+          const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
+          const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          v[e] = lo[e];
-          v[4 + e] = hi[e];
+          for (int e = 0; e < 4; ++e) {
+            v[e] = lo[e];
+            v[4 + e] = hi[e];
+          }
+          simple_row<DT>(v, m_img + pr, n0 + wn * TN + ec, args, plan, tab, BN);
         }
-        const int nvalid = N - n;
-        const long long m = m_img + pr;
-        apply_epilogue<8>(v, m, n, nvalid, args.epi);
-        store_from_float<8>(args.C, args.out_dtype, m * args.ldc + n, nvalid, v);
+      }
+    } else {
+      for (int r = er; r < 32; r += RPI) {
+        const int pr = wm * TMW + i * 32 + r;
+        const int n = n0 + wn * TN + ec;
+        if (pr < npix && n < N) {
+          float v[8];
+          const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
+          const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = lo[e];
+            v[4 + e] = hi[e];
+          }
+          const int nvalid = N - n;
+          const long long m = m_img + pr;
+          apply_epilogue_tab(v, m, n, nvalid, args.epi, plan, tab, BN);
+          store_from_float<8>(args.C, args.out_dtype, m * args.ldc + n, nvalid, v);
+        }
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-  }
+  });
 }
 
 // LDS bytes of one filter stage and of the epilogue staging, for the host-side plan.
 template <int TM, int BN, int WM, int WN, int NSB>
 int launch_conv_patch(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig, hipStream_t stream) {
   if (!conv || b_ncontig || a.p_np_bytes <= 0) return (int)hipErrorInvalidValue;
-  const size_t staging = (size_t)WM * WN * 32 * (BN / WN + 4) * 4;
+  // epilogue: wave-private staging areas followed by the operand table
+  const size_t staging = ((size_t)WM * WN * 32 * (BN / WN + 4) + (size_t)TRACEA_MAX_EPILOGUE_OPS * 2 * BN) * 4;
   size_t lds = (size_t)a.p_np_bytes + (size_t)NSB * BN * 128;
   if (lds < staging) lds = staging;
   const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(WM * WN * 64);

@@ -673,6 +673,24 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
            g.pad_h, tuning_device_name());
   int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
   if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
+  // Default choice of a patch-resident variant.  Measured on MI355X it beats the
+  // streamed tiles only where the filter bank is narrow and an image holds
+  // several full tiles (N32 56x56x64 -> 64, 3x3: 21.9 us against 23.1 us); with
+  // 128 filters, stride 2 or 14x14 images the streamed 128x64 tiles are faster.
+  // One shape is thin evidence: a tuning-cache entry or a forced variant wins
+  // over this rule, and tracea_autotune_conv2d measures every variant.
+  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && a.N <= 64 &&
+      g.stride_h == 1 && g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 &&
+      (long long)g.block.h_out * g.block.w_out >= 4 * 256) {
+    for (int i = 0; i < contraction_variant_count(); ++i) {
+      const ContractionVariant &cv = contraction_variant(i);
+      if (cv.pipeline == 4 && cv.bm == 256 && cv.bn == 64) {
+        ContractionArgs probe = a;
+        if (plan_conv_patch(g, cv, plan.w_ncontig, &probe)) vi = i;
+        break;
+      }
+    }
+  }
   const long long x_extent = (long long)g.block.batch * g.block.h_in * g.block.w_in * g.block.c_in * 2;
   const long long w_extent = (long long)g.n_gemm * g.k_gemm * 2;
   const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
