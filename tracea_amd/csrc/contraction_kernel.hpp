@@ -387,55 +387,99 @@ __device__ __forceinline__ bool chain_is_simple(const ChainPlan &plan, const Con
   return ok;
 }
 
-// One row on the specialised path: 8 channels, 16-bit output, every access a
-// single 16-byte operation.
-template <int DT>
-__device__ __forceinline__ void simple_row(float (&v)[8], long long m, int n, const ContractionArgs &args,
-                                           const ChainPlan &plan, const float *tab, int bn) {
-#pragma nounroll
-  for (int o = 0; o < plan.n_ops; ++o) {
-    const int kind = (int)((plan.kinds >> (4 * o)) & 15u);
-    if (kind == TRACEA_EPI_OP_RELU) {
+// The specialised path for the 32 staged rows of one accumulator block: the
+// rows a lane handles (er, er+RPI, ...) are processed GROUP at a time -- all
+// their staged values are read first, each operator's operands are read once
+// and applied to every row of the group, residual loads are issued together,
+// stores come last.  One row at a time, every row paid an LDS round trip for
+// its staged values and one more per operator, back to back.
+// row_of(r) gives the output row of staged row r, or -1 if it does not exist.
+template <int DT, int TN, typename RowOf>
+__device__ __forceinline__ void simple_rows(const float *stage, int lane, int n, const ContractionArgs &args,
+                                            const ChainPlan &plan, const float *tab, int bn, RowOf row_of) {
+  constexpr int EP_PITCH = TN + 4, LPR = TN / 8, RPI = 64 / LPR, NIT = 32 / RPI;
+  constexpr int GROUP = NIT < 4 ? NIT : 4;
+  const int er = lane / LPR, ec = (lane % LPR) * 8;
+  static_for<0, NIT / GROUP>([&](auto grp) {
+    constexpr int it0 = decltype(grp)::value * GROUP;
+    float v[GROUP][8];
+    long long m[GROUP];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = fmaxf(0.0f, v[e]);
-    } else if (kind == TRACEA_EPI_OP_RESIDUAL_ADD) {
-      const u32x4 raw = *(const u32x4 *)((const unsigned short *)plan.res_ptr + m * plan.res_ld + n);
-      if (plan.res_dtype == DT_F16) {
-        const f16x8 h = __builtin_bit_cast(f16x8, raw);
+    for (int g = 0; g < GROUP; ++g) {
+      const int r = er + (it0 + g) * RPI;
+      m[g] = row_of(r);
+      const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
+      const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = v[e] + (float)h[e];
-      } else {
-        const bf16x8 h = __builtin_bit_cast(bf16x8, raw);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = v[e] + (float)h[e];
-      }
-    } else {  // bias: v + a; scale/shift and BatchNorm: v * a + b
-      const float *pa = tab + (o * 2) * bn;
-      const f32x4 a0 = *(const f32x4 *)pa, a1 = *(const f32x4 *)(pa + 4);
-      const float a[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-      if (kind == TRACEA_EPI_OP_BIAS_ADD) {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = v[e] + a[e];
-      } else {
-        const f32x4 b0 = *(const f32x4 *)(pa + bn), b1 = *(const f32x4 *)(pa + bn + 4);
-        const float b[8] = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = v[e] * a[e] + b[e];
+      for (int e = 0; e < 4; ++e) {
+        v[g][e] = lo[e];
+        v[g][4 + e] = hi[e];
       }
     }
-  }
-  unsigned short *dst = (unsigned short *)args.C + m * args.ldc + n;
-  if constexpr (DT == DT_F16) {
-    f16x8 h;
+#pragma nounroll
+    for (int o = 0; o < plan.n_ops; ++o) {
+      const int kind = (int)((plan.kinds >> (4 * o)) & 15u);
+      if (kind == TRACEA_EPI_OP_RELU) {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[e];
-    *(f16x8 *)dst = h;
-  } else {
-    bf16x8 h;
+        for (int g = 0; g < GROUP; ++g)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) h[e] = (__bf16)v[e];
-    *(bf16x8 *)dst = h;
-  }
+          for (int e = 0; e < 8; ++e) v[g][e] = fmaxf(0.0f, v[g][e]);
+      } else if (kind == TRACEA_EPI_OP_RESIDUAL_ADD) {
+        u32x4 raw[GROUP];
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+          const long long mm = m[g] >= 0 ? m[g] : 0;  // a row that does not exist re-reads row 0, result discarded
+          raw[g] = *(const u32x4 *)((const unsigned short *)plan.res_ptr + mm * plan.res_ld + n);
+        }
+#pragma unroll
+        for (int g = 0; g < GROUP; ++g) {
+          if (plan.res_dtype == DT_F16) {
+            const f16x8 h = __builtin_bit_cast(f16x8, raw[g]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[g][e] = v[g][e] + (float)h[e];
+          } else {
+            const bf16x8 h = __builtin_bit_cast(bf16x8, raw[g]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[g][e] = v[g][e] + (float)h[e];
+          }
+        }
+      } else {  // bias: v + a; scale/shift and BatchNorm: v * a + b
+        const float *pa = tab + (o * 2) * bn;
+        const f32x4 a0 = *(const f32x4 *)pa, a1 = *(const f32x4 *)(pa + 4);
+        const f32x4 b0 = *(const f32x4 *)(pa + bn), b1 = *(const f32x4 *)(pa + bn + 4);  // zeros for a bias
+        const float a[8] = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+        const float b[8] = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+        if (kind == TRACEA_EPI_OP_BIAS_ADD) {
+#pragma unroll
+          for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[g][e] = v[g][e] + a[e];
+        } else {
+#pragma unroll
+          for (int g = 0; g < GROUP; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[g][e] = v[g][e] * a[e] + b[e];
+        }
+      }
+    }
+#pragma unroll
+    for (int g = 0; g < GROUP; ++g) {
+      if (m[g] >= 0) {
+        unsigned short *dst = (unsigned short *)args.C + m[g] * args.ldc + n;
+        if constexpr (DT == DT_F16) {
+          f16x8 h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[g][e];
+          *(f16x8 *)dst = h;
+        } else {
+          bf16x8 h;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) h[e] = (__bf16)v[g][e];
+          *(bf16x8 *)dst = h;
+        }
+      }
+    }
+  });
 }
 
 // ---- tile order ---------------------------------------------------------------
@@ -552,6 +596,12 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int NCH = BN / 8;
 
   u32x4 ra[NA], rb[NB];
+
+  // The chain as the epilogue needs it, and the choice of its row body, are worked
+  // out here: their scalar loads complete under the main loop instead of after it.
+  // (The output type equals the operand type on the specialised path.)
+  const ChainPlan plan = chain_plan(args.epi);
+  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
 
   // This thread's entries of the epilogue operand table (see chain_table_value):
   // requested here so that they arrive under the main loop.
@@ -1030,9 +1080,6 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     if (tid + i * NT < TAB_ENTRIES) table[tid + i * NT] = tabr[i];
   __syncthreads();
   const float *tab = table + wn * TN + ec;
-  const ChainPlan plan = chain_plan(args.epi);
-  // the output type equals the operand type on the specialised path (simple_row<DT> stores DT)
-  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
   static_for<0, FM>([&](auto blk) {
     constexpr int i = decltype(blk)::value;
     static_for<0, FN>([&](auto col) {
@@ -1051,20 +1098,9 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
     if (simple) {
-      for (int r = er; r < 32; r += RPI) {
-        const int m = m0 + wm * TM + i * 32 + r;
-        if (m < M) {
-          float v[8];
-          const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
-          const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] = lo[e];
-            v[4 + e] = hi[e];
-          }
-          simple_row<DT>(v, m, n0 + wn * TN + ec, args, plan, tab, BN);
-        }
-      }
+      const int mb = m0 + wm * TM + i * 32;
+      simple_rows<DT, TN>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN,
+                          [&](int r) -> long long { return mb + r < M ? (long long)(mb + r) : -1ll; });
     } else {
       for (int r = er; r < 32; r += RPI) {
         const int m = m0 + wm * TM + i * 32 + r;

@@ -122,6 +122,10 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
 #pragma unroll
   for (int st = 0; st < NSB - 1; ++st) dma_b(st, (st < nk ? st : nk - 1) * BK);
 
+  // chain description and choice of the row body: read here, under the main loop
+  const ChainPlan plan = chain_plan(args.epi);
+  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
+
   // this thread's entries of the epilogue operand table, requested under the main loop
   constexpr int TAB_ENTRIES = TRACEA_MAX_EPILOGUE_OPS * 2 * BN;
   constexpr int TPT = (TAB_ENTRIES + NT - 1) / NT;
@@ -231,9 +235,6 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
     if (tid + i * NT < TAB_ENTRIES) table[tid + i * NT] = tabr[i];
   __syncthreads();
   const float *tab = table + wn * TN + ec;
-  const ChainPlan plan = chain_plan(args.epi);
-  // the output type equals the operand type on the specialised path (simple_row<DT> stores DT)
-  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
   static_for<0, FM>([&](auto blk) {
     constexpr int i = decltype(blk)::value;
     static_for<0, FN>([&](auto col) {
@@ -247,20 +248,9 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
     if (simple) {
-      for (int r = er; r < 32; r += RPI) {
-        const int pr = wm * TMW + i * 32 + r;
-        if (pr < npix) {
-          float v[8];
-          const f32x4 lo = *(const f32x4 *)(stage + r * EP_PITCH + ec);
-          const f32x4 hi = *(const f32x4 *)(stage + r * EP_PITCH + ec + 4);
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            v[e] = lo[e];
-            v[4 + e] = hi[e];
-          }
-          simple_row<DT>(v, m_img + pr, n0 + wn * TN + ec, args, plan, tab, BN);
-        }
-      }
+      const int pb = wm * TMW + i * 32;
+      simple_rows<DT, TN>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN,
+                          [&](int r) -> long long { return pb + r < npix ? m_img + pb + r : -1ll; });
     } else {
       for (int r = er; r < 32; r += RPI) {
         const int pr = wm * TMW + i * 32 + r;
