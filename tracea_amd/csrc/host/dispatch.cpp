@@ -380,7 +380,7 @@ int twin(int vi, int pipeline) {
 // pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
 int resolve_variant(int vi, bool conv, bool b_ncontig, bool k_exact) {
   int pipe = contraction_variant(vi).pipeline;
-  if (pipe == 4) pipe = 2;  // the caller found the patch-resident kernel unusable: same tile, streamed operands
+  if (pipe == 4) pipe = 2;  // a convolution-only kernel asked for a GEMM: same tile with streamed operands, if any
   if (pipe >= 2 && b_ncontig) pipe = 1;
   if (pipe == 1 && !conv && !k_exact) pipe = 0;
   if (pipe == contraction_variant(vi).pipeline) return vi;
@@ -698,6 +698,13 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
     t_last_conv = vi;
     return hip_status("conv2d launch",
                       contraction_variant(vi).launch(a, true, plan.x.dtype, false, stream));
+  }
+  // a patch-resident variant that cannot run this problem (asked for by a forced
+  // index or a cache entry) gives way to the selector's choice, not to whatever
+  // shares its tile shape
+  if (contraction_variant(vi).pipeline == 4) {
+    vi = select_contraction_variant(a.M, a.N, a.K, true);
+    if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
   }
   vi = resolve_variant(vi, true, plan.w_ncontig || !small, true);
   const ContractionVariant &v = contraction_variant(vi);
