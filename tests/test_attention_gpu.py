@@ -25,7 +25,7 @@ def _tol(d, dtype):
     return tol_for_k(d) + (2.0 ** -8 if dtype == "bf16" else 2.0 ** -11) * 2
 
 
-@pytest.mark.parametrize("variant", ["pipe", "tr", "u16"])
+@pytest.mark.parametrize("variant", ["pipe", "pipe2", "tr", "u16"])
 @pytest.mark.parametrize("d", [64, 128])
 @pytest.mark.parametrize("dtype", ["bf16", "f16"])
 def test_small_and_edge_lengths(tracea_gpu, variant, d, dtype):

@@ -328,8 +328,18 @@ fa2_fwd_kernel(const AttentionArgs a) {
 // that publishes K(t+1) and V(t) and retires K(t) and V(t-1); K(t+2) and
 // V(t+1) are then requested into the retired stages, a whole iteration before
 // they are needed.
+//
+// EARLY_MAX: an iteration of the form above has three phases -- running maximum
+// of tile t (vector ALU only), score product of t+1 with the exponentials of t
+// (both pipes), P.V of t (matrix pipe only).  The maximum of tile t+1 depends
+// only on S(t+1), which is complete after the second phase, so with EARLY_MAX it
+// is computed under the P.V MFMAs of tile t (whose operand reads then run one
+// step ahead): two phases, both pipes busy in each.  Only the rescale of O,
+// which needs P.V(t) finished, stays between iterations.  The last iteration
+// takes the maximum of a tile past the end, all of whose scores are masked:
+// nothing moves.
 // ---------------------------------------------------------------------------
-template <int DT, int D>
+template <int DT, int D, bool EARLY_MAX>
 __global__ void __launch_bounds__(FA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fa2_fwd_pipe_kernel(const AttentionArgs a) {
   constexpr int ROW_BYTES = D * 2;
@@ -453,20 +463,15 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   f32x16 s_cur[2], s_nxt[2];
   scores(sKbase, s_cur);
 
-  // One iteration, compiled twice: EDGE tiles (sequence end or causal diagonal)
-  // mask scores with selects, interior tiles do not test at all.  Either body is
-  // branch-free up to the optional rescale, so the MFMAs of the next tile's score
-  // product can be interleaved instruction by instruction with the vector-ALU
-  // work of this tile's softmax.
-  auto iteration = [&](int t, auto edge_tag) {
+  // Masks tile `tile`'s scores in s (EDGE only) and folds them into the running
+  // maximum.  The maximum is taken over the raw scores (the scale is positive);
+  // the scale is folded into the exponent's multiply-add.  Leaves the rescale
+  // factor of the earlier tiles in `alpha` (exactly 1 where the maximum did not
+  // move) and returns whether this lane's maximum moved.
+  float alpha = 1.0f;
+  auto take_max = [&](int tile, auto edge_tag, f32x16 (&s)[2]) -> bool {
     constexpr bool EDGE = decltype(edge_tag)::value;
-    const unsigned char *sV = sVbase + (t & 1) * TILE_BYTES;
-    const unsigned char *sKn = sKbase + ((t + 1) & 1) * TILE_BYTES;
-    const int kv0 = t * FA_BKV;
-
-    // phase 1: mask, running maximum.  The maximum is taken over the raw scores
-    // (the scale is positive) and the scale is folded into the exponent's
-    // multiply-add of phase 2.
+    const int kv0 = tile * FA_BKV;
     float mx = -INFINITY;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
@@ -475,27 +480,33 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         if constexpr (EDGE) {
           const int kv = kv0 + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
           const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine));
-          s_cur[blk][e] = dead ? -INFINITY : s_cur[blk][e];
+          s[blk][e] = dead ? -INFINITY : s[blk][e];
         }
-        mx = fmaxf(mx, s_cur[blk][e]);
+        mx = fmaxf(mx, s[blk][e]);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx * a.scale_log2);
     const bool moved = m_new > m_run;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     m_run = m_new;
-    // alpha is exactly 1 for every lane whose maximum did not move: skip the
-    // 16*DB multiplies unless some lane of the wave needs them
+    return moved;
+  };
+  // alpha is exactly 1 for every lane whose maximum did not move: the 16*DB
+  // multiplies are skipped unless some lane of the wave needs them
+  auto rescale = [&](bool moved) {
     if (__any(moved)) {
 #pragma unroll
       for (int d = 0; d < DB; ++d)
 #pragma unroll
         for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
     }
-    __builtin_amdgcn_sched_barrier(0);
-
-    // phase 2, one scheduling region: the score product of the NEXT tile on the
-    // matrix pipe, the exponentials and row sums of THIS tile on the vector ALU
+  };
+  // One scheduling region: the score product of tile t+1 on the matrix pipe, the
+  // exponentials and row sums of tile t (maximum m_run, rescale factor alpha) on
+  // the vector ALU.
+  u32x4 pf[4];
+  auto softmax_and_next_scores = [&](int t) {
+    const unsigned char *sKn = sKbase + ((t + 1) & 1) * TILE_BYTES;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -508,7 +519,6 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         s_nxt[blk] = Mfma32<DT>::run(kf, qf[ks], s_nxt[blk]);
       }
     float lsum = 0.0f;
-    u32x4 pf[4];
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -516,7 +526,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         float p[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[blk][hh * 8 + j], a.scale_log2, -m_new));
+          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[blk][hh * 8 + j], a.scale_log2, -m_run));
           lsum += p[j];
         }
         pf[blk * 2 + hh] = pack8<DT>(p);
@@ -524,25 +534,117 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     l_run = l_run * alpha + lsum;
     Interleave3<0, 2 * KS>::run();
     __builtin_amdgcn_sched_barrier(0);
+  };
+  // The transposed V operand of P.V step (kk, d): V rows kk*16.., head-dim block d.
+  auto read_v = [&](const unsigned char *sV, int kk, int d) -> u32x4 {
+    const int r = lane & 15;
+    const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
+    const int row_lo = kk * 16 + g * 4 + (r >> 2);
+    const int row_hi = row_lo + 8;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_lo, col >> 3) + (col & 7) * 2));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_hi, col >> 3) + (col & 7) * 2));
+    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 vf;
+    vf[0] = lo2[0]; vf[1] = lo2[1]; vf[2] = hi2[0]; vf[3] = hi2[1];
+    return vf;
+  };
 
-    // ---- O^T += V^T P^T ----
+  // One iteration, compiled twice: EDGE tiles (sequence end or causal diagonal)
+  // mask scores with selects, interior tiles do not test at all.  Either body is
+  // branch-free up to the optional rescale, so MFMAs and vector-ALU work can be
+  // interleaved instruction by instruction.  For EARLY_MAX the tag describes
+  // tile t+1, the one whose maximum the iteration takes.
+  auto iteration = [&](int t, auto edge_tag) {
+    const unsigned char *sV = sVbase + (t & 1) * TILE_BYTES;
+    if constexpr (!EARLY_MAX) {
+      const bool moved = take_max(t, edge_tag, s_cur);
+      rescale(moved);
+      __builtin_amdgcn_sched_barrier(0);
+      softmax_and_next_scores(t);
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+      for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-      for (int d = 0; d < DB; ++d) {
-        const int r = lane & 15;
-        const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
-        const int row_lo = kk * 16 + g * 4 + (r >> 2);
-        const int row_hi = row_lo + 8;
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_lo, col >> 3) + (col & 7) * 2));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_hi, col >> 3) + (col & 7) * 2));
-        const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
-        u32x4 vf;
-        vf[0] = lo2[0]; vf[1] = lo2[1]; vf[2] = hi2[0]; vf[3] = hi2[1];
-        o[d] = Mfma32<DT>::run(vf, pf[kk], o[d]);
+        for (int d = 0; d < DB; ++d) o[d] = Mfma32<DT>::run(read_v(sV, kk, d), pf[kk], o[d]);
+    } else {
+      // Both phases are written as short chunks -- a few MFMAs and their share of
+      // the vector-ALU work -- each closed by a full scheduling fence: MFMA issue
+      // is asynchronous, so the vector instructions of a chunk execute while the
+      // matrix pipe works on its MFMAs, whatever order the compiler gives them
+      // inside the chunk.
+      constexpr bool EDGE = decltype(edge_tag)::value;
+      const unsigned char *sKn = sKbase + ((t + 1) & 1) * TILE_BYTES;
+      // ---- phase A: S^T(t+1) = K(t+1) Q^T  with  P(t) = exp2(S(t)*scale - m), row sums ----
+      // chunk ks: the two MFMAs of k-step ks (operands read one chunk ahead) and
+      // 32/KS of the 32 exponentials
+      constexpr int EPC = 32 / KS;  // exponentials per chunk
+      static_assert(32 % KS == 0 && (EPC == 4 || EPC == 8), "exponentials must divide over the k-steps");
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s_nxt[blk][e] = 0.0f;
+      u32x4 kf0 = *(const u32x4 *)(sKn + k_piece(lrow, g));
+      u32x4 kf1 = *(const u32x4 *)(sKn + k_piece(32 + lrow, g));
+      float lsum = 0.0f;
+      float p[8];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4 kn0 = kf0, kn1 = kf1;
+        if (ks + 1 < KS) {
+          kn0 = *(const u32x4 *)(sKn + k_piece(lrow, (ks + 1) * 2 + g));
+          kn1 = *(const u32x4 *)(sKn + k_piece(32 + lrow, (ks + 1) * 2 + g));
+        }
+        s_nxt[0] = Mfma32<DT>::run(kf0, qf[ks], s_nxt[0]);
+        s_nxt[1] = Mfma32<DT>::run(kf1, qf[ks], s_nxt[1]);
+#pragma unroll
+        for (int j = 0; j < EPC; ++j) {
+          const int idx = ks * EPC + j;  // 0..31 over (blk, hh, j8): blk = idx/16, element idx%16
+          const float x = __builtin_amdgcn_exp2f(fmaf(s_cur[idx >> 4][idx & 15], a.scale_log2, -m_run));
+          p[idx & 7] = x;
+          lsum += x;
+          if ((idx & 7) == 7) pf[idx >> 3] = pack8<DT>(p);
+        }
+        kf0 = kn0;
+        kf1 = kn1;
+        __builtin_amdgcn_sched_barrier(0);
       }
+      l_run = l_run * alpha + lsum;
+
+      // ---- phase B: O^T += V^T(t) P^T(t)  with  the running maximum of tile t+1 ----
+      // chunk kk: the DB MFMAs of key block kk (operand reads one MFMA ahead) and
+      // the maximum over 8 of the 32 scores of S(t+1)
+      const int kv0n = (t + 1) * FA_BKV;
+      float mx = -INFINITY;
+      u32x4 vf = read_v(sV, 0, 0);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+#pragma unroll
+        for (int d = 0; d < DB; ++d) {
+          const int nxt = kk * DB + d + 1;
+          const u32x4 vn = nxt < 4 * DB ? read_v(sV, nxt / DB, nxt % DB) : vf;
+          o[d] = Mfma32<DT>::run(vf, pf[kk], o[d]);
+          vf = vn;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int idx = kk * 8 + j, blk = idx >> 4, e = idx & 15;
+          if constexpr (EDGE) {
+            const int kv = kv0n + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+            const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine));
+            s_nxt[blk][e] = dead ? -INFINITY : s_nxt[blk][e];
+          }
+          mx = fmaxf(mx, s_nxt[blk][e]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx * a.scale_log2);
+      const bool moved = m_new > m_run;
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      rescale(moved);
     }
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) s_cur[blk] = s_nxt[blk];
@@ -558,8 +660,16 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     first_edge = fe < first_edge ? fe : first_edge;
   }
   first_edge = __builtin_amdgcn_readfirstlane(first_edge);
+  if constexpr (EARLY_MAX) {
+    // the maximum of tile 0 has no P.V to hide under; O is still zero, no rescale
+    if (first_edge == 0) (void)take_max(0, std::true_type{}, s_cur);
+    else (void)take_max(0, std::false_type{}, s_cur);
+  }
+  // iteration t handles tile t, and with EARLY_MAX the maximum of tile t+1: its
+  // body is the interior one while that tile is interior
+  const int interior_end = EARLY_MAX ? first_edge - 1 : first_edge;
   int t = 0;
-  for (; t < first_edge; ++t) {
+  for (; t < interior_end; ++t) {
     __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1) and V(t), requested one iteration ago
     __syncthreads();
     load_k(t + 2, sKbase + (t & 1) * TILE_BYTES);
@@ -607,14 +717,14 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   }
 }
 
-template <int D>
+template <int D, bool EARLY_MAX>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
   constexpr size_t lds = 4 * (size_t)FA_BKV * D * 2;
   const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
   const dim3 grid((unsigned)(nqb * a.B * a.H)), block(FA_WAVES * 64);
 #define TRACEA_FA_LAUNCH(DTV)                                                                  \
   do {                                                                                         \
-    auto kfn = fa2_fwd_pipe_kernel<DTV, D>;                                                    \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX>;                                                    \
     static bool attr_done = false;                                                             \
     if (!attr_done) {                                                                          \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
@@ -667,8 +777,11 @@ static bool feasible_d128(const AttentionArgs &a) { return a.D == 128; }
 static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 
 static const AttentionVariant kAttentionVariants[] = {
-    {"fa2_q128_kv64_d128_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<128>, &feasible_pipe_d128},
-    {"fa2_q128_kv64_d64_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<64>, &feasible_pipe_d64},
+    // the first feasible entry is the default
+    {"fa2_q128_kv64_d128_pipe2", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<128, true>, &feasible_pipe_d128},
+    {"fa2_q128_kv64_d64_pipe2", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<64, true>, &feasible_pipe_d64},
+    {"fa2_q128_kv64_d128_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<128, false>, &feasible_pipe_d128},
+    {"fa2_q128_kv64_d64_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<64, false>, &feasible_pipe_d64},
     {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, true>, &feasible_d128},
     {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, false>, &feasible_d128},
     {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<64, true>, &feasible_d64},
