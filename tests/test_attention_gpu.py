@@ -46,6 +46,43 @@ def test_small_and_edge_lengths(tracea_gpu, variant, d, dtype):
         capi.force_variant("attention", -1)
 
 
+@pytest.mark.parametrize("variant", ["pipe", "pipe2", "tr", "u16"])
+@pytest.mark.parametrize("dom_mod8", [1, 5])
+def test_dominant_key_needs_the_true_running_maximum(tracea_gpu, variant, dom_mod8):
+    """One key scores about 2^250 times the others for every query row that can see it; the exact output is that
+    key's V row.
+    In the kernels a query's keys are split between lanes l and l+32 (keys with kv % 8 in 0..3 and in
+    4..7); a running maximum that is consistent between the two but not the true one cancels out of an
+    ordinary softmax and passes every comparison with the oracle, yet here exp2 of (score - too small a
+    maximum) overflows.  The dominant key is placed once in each half."""
+    from tracea_amd import capi
+    b, h, s, d = 1, 2, 384, 128
+    rng = np.random.default_rng(77 + dom_mod8)
+    q = np.zeros((b, h, s, d), np.float32)
+    k = round_bf16(rng.standard_normal((b, h, s, d)) * 0.05)
+    v = round_bf16(rng.standard_normal((b, h, s, d)))
+    q[...] = 4.0
+    # a single dominant key per run, visible to every row (under the causal mask: to the rows at or after it)
+    gk = 64 * 2 + 8 * 3 + dom_mod8          # tile 2, lane-half chosen by dom_mod8
+    k[:, :, gk, :] = 4.0                    # q.k = 128 * 16 = 2048; others ~ N(0, (4*0.05)^2 * 128) ~ +-2.3
+    name = "fa2_q128_kv64_d%d_%s" % (d, variant)
+    capi.force_variant("attention", name)
+    try:
+        for causal in (False, True):
+            got = tracea_gpu.attention(_dev(q, torch.bfloat16), _dev(k, torch.bfloat16), _dev(v, torch.bfloat16),
+                                       causal=causal).float().cpu().numpy()
+            assert np.isfinite(got).all(), "%s causal=%s: non-finite output" % (name, causal)
+            rows = slice(gk, s) if causal else slice(0, s)   # causal rows before gk cannot see it
+            expect = np.broadcast_to(v[:, :, gk:gk + 1, :], got[:, :, rows, :].shape)
+            # softmax weight of the dominant key is 1 - O(2^-250): the output is its V row up to bf16 rounding
+            assert np.abs(got[:, :, rows, :] - expect).max() <= 2.0 ** -7 * np.abs(v).max(), (name, causal)
+            if causal:  # the rows that cannot see it still match the oracle
+                ref = oracle.attention_bhsd(q, k, v, 1.0 / np.sqrt(d), True)
+                assert_close_scaled(got[:, :, :gk, :], ref[:, :, :gk, :], _tol(d, "bf16"), name + " before the dominant key")
+    finally:
+        capi.force_variant("attention", -1)
+
+
 def test_reference_gpu_check_shape(tracea_gpu):
     # examples/verify_fa2_gpu.rs:67-162: B1 H4 S512 D64 causal, inputs U[0,0.2), tolerance 2e-3
     rng = np.random.default_rng(42)
