@@ -22,7 +22,7 @@ PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
 # HBM-side bytes per launch of the dominant kernel of each workload, from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
 # (profiles/bench_kernels_mi355x.md); None where no counter run exists.
-TRAFFIC_BYTES = {"gemm": 235.1e6, "conv": 26.5e6, "attention": 575.9e6, "attention_causal": None, "copy": None}
+TRAFFIC_BYTES = {"gemm": 235.2e6, "conv": 26.5e6, "attention": 537.1e6, "attention_causal": None, "copy": None}
 METRIC = "TFLOPS + % fp16 MFMA peak: GEMM 4096^3, 3x3 implicit-GEMM conv, FA2 fwd"
 
 
