@@ -155,8 +155,24 @@ TraceaStatus tracea_conv2d(TraceaTensorView x, TraceaTensorView w, const TraceaT
                            const TraceaTensorView *residual, TraceaTensorView *out,
                            TraceaConv2dParams params);
 
-/* reference: include/tracea.hpp:133-137.  Outside the accelerated path:
- * always returns TRACEA_UNSUPPORTED_CONFIG. */
+/* ---- transposed convolution: reference include/tracea.hpp:112-137,
+ * src/interface/c_bindings.rs:292-368, kernel src/emitter/conv_transpose.rs:178-266.
+ *   x   [N,H,W,C]   activations, channels innermost (NHWC)
+ *   w   [K,R,S,C]   filters as the reference reads the dims (c_bindings.rs:303-311:
+ *                   K = output channels); the physical order is taken from the
+ *                   strides.  The reference kernel indexes the storage as
+ *                   [C*R*S, K] rows (conv_transpose.rs:236), i.e. strides
+ *                   {1, S*K, K, R*S*K}; that order, torch's [C,K,R,S] and a
+ *                   contiguous [K,R,S,C] are accepted (input channels outermost
+ *                   or innermost, the other three dims dense)
+ *   b   [K]         optional bias; residual optional, shape of out
+ *   out [N,Ho,Wo,K] pre-allocated, Ho = (H-1)*stride - 2*pad + R + output_padding
+ * x and w are both f32 (the reference's only case), both f16 or both bf16;
+ * sums are kept in fp32.  groups and dilation must be 1 (0 = unset), as the
+ * reference states (conv_transpose.rs:26-29).  Stride, padding and output
+ * padding may differ between h and w (the reference reads the _h fields for both).
+ * The call takes a temporary device buffer from the stream-ordered allocator
+ * (hipMallocAsync on params.stream) for the per-tap partial products. */
 TraceaStatus tracea_conv_transpose2d(TraceaTensorView x, TraceaTensorView w,
                                      const TraceaTensorView *b, const TraceaTensorView *residual,
                                      TraceaTensorView *out, TraceaConvTranspose2dParams params);
@@ -225,7 +241,7 @@ typedef struct {
 
 #define TRACEA_MAX_EPILOGUE_OPS 4
 
-/* tracea_conv2d / tracea_gemm with an explicit operator chain (at most
+/* tracea_conv2d / tracea_gemm / tracea_conv_transpose2d with an explicit operator chain (at most
  * TRACEA_MAX_EPILOGUE_OPS entries) instead of a TraceaEpilogueKind; the
  * `epilogue` field of params is ignored.  This is how BatchNorm, which
  * TraceaEpilogueKind cannot name, reaches the fused epilogue
@@ -235,6 +251,9 @@ TraceaStatus tracea_conv2d_ex(TraceaTensorView x, TraceaTensorView w, TraceaTens
                               uint32_t n_ops);
 TraceaStatus tracea_gemm_ex(TraceaTensorView a, TraceaTensorView b, TraceaTensorView *c,
                             TraceaGemmParams params, const TraceaEpilogueOp *ops, uint32_t n_ops);
+TraceaStatus tracea_conv_transpose2d_ex(TraceaTensorView x, TraceaTensorView w, TraceaTensorView *out,
+                                        TraceaConvTranspose2dParams params,
+                                        const TraceaEpilogueOp *ops, uint32_t n_ops);
 
 /* Kernel-variant control for tuners and benchmarks.  `op` is "gemm", "conv2d"
  * or "attention".  A variant forced with tracea_force_variant (index >= 0) is

@@ -179,6 +179,38 @@ def conv2d_nhwc(x, w, stride=1, pad=0, dilation=1, nthreads=None):
     return y
 
 
+def conv_transpose_out_shape(h, w, r, s, stride, pad, output_padding):
+    """(H_out, W_out) of the reference (src/emitter/conv_transpose.rs:36-37)."""
+    sh, sw = _pair(stride)
+    ph, pw = _pair(pad)
+    oh, ow = _pair(output_padding)
+    return (h - 1) * sh - 2 * ph + r + oh, (w - 1) * sw - 2 * pw + s + ow
+
+
+def _pair(v):
+    return (v, v) if isinstance(v, int) else tuple(v)
+
+
+def conv_transpose2d_nhwc(x, w, stride=1, pad=0, output_padding=0, nthreads=None):
+    """x [N,H,W,C], w [C,R,S,K] (the reference kernel's [C*R*S, K] rows) -> [N,Ho,Wo,K] float32."""
+    x, w = _f32(x), _f32(w)
+    n, h, wd, c = x.shape
+    c2, r, s, k = w.shape
+    assert c == c2
+    sh, sw = _pair(stride)
+    ph, pw = _pair(pad)
+    oh, ow = _pair(output_padding)
+    ho, wo = conv_transpose_out_shape(h, wd, r, s, stride, pad, output_padding)
+    if ho <= 0 or wo <= 0:
+        raise ValueError("oracle_conv_transpose2d_nhwc: empty output")
+    y = np.empty((n, ho, wo, k), dtype=np.float32)
+    rc = lib().oracle_conv_transpose2d_nhwc(_ptr(x), _ptr(w), _ptr(y), n, h, wd, c, k, r, s, sh, sw,
+                                            ph, pw, oh, ow, nthreads or default_threads())
+    if rc != 0:
+        raise ValueError("oracle_conv_transpose2d_nhwc: bad argument")
+    return y
+
+
 def attention(q, k, v, scale, causal, rows=None, nthreads=None):
     """One (batch, head) slice: q,k,v [S,D] -> out [len(rows), D] float32."""
     q, k, v = _f32(q), _f32(k), _f32(v)

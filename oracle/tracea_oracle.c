@@ -17,6 +17,11 @@
  *   oracle_conv2d_nhwc       pinned: all-ones interior/border counts, 1x1 == GEMM,
  *                            delta filters == shifts, torch conv2d fp32 fixtures.
  *   oracle_conv_coords       pinned: brute-force nested-loop enumeration.
+ *   oracle_conv_transpose2d  pinned: the reference's minimal case and its scatter-form
+ *                            statement re-derived as brute force, all-ones tap counts,
+ *                            stride 1 == convolution with the flipped filter,
+ *                            adjointness <convT(x), y> == <x, conv(y)>, torch
+ *                            conv_transpose2d fp32.
  *   oracle_attention         pinned: softmax row-sum invariants, causal row 0,
  *                            Q=0 prefix means, torch SDPA fp32 fixtures.
  *
@@ -507,6 +512,80 @@ ORACLE_API int oracle_conv2d_nhwc(const float *x, const float *w, float *y, int 
     for (int t = 0; t < nthreads - 1; ++t)
         if (pthread_create(&th[started], NULL, conv_worker, &j) == 0) ++started;
     conv_worker(&j);
+    for (int t = 0; t < started; ++t) pthread_join(th[t], NULL);
+    return 0;
+}
+
+/* ------------------------------------------------------------------------ */
+/* Transposed convolution, NHWC input, weights [C*R*S, K] (row c*R*S + r*S + s */
+/* as the reference kernel indexes them, src/emitter/conv_transpose.rs:207-   */
+/* 225, 236), NHWK output.  The value is that of the reference's own CPU     */
+/* statement (examples/verify_conv_transpose.rs:12-54: ho = hi*stride - pad  */
+/* + r), written as the gather the kernel performs (hi = (ho + pad - r) /    */
+/* stride where that division is exact).  Accumulates in double.             */
+/* ------------------------------------------------------------------------ */
+typedef struct {
+    const float *x, *w;
+    float *y;
+    int n, h, wd, c, k, r, s, sh, sw, ph, pw, ho, wo;
+    volatile int *next;
+} convt_job;
+
+static void *convt_worker(void *arg)
+{
+    const convt_job *j = (const convt_job *)arg;
+    const int rows = j->n * j->ho;
+    double *acc = (double *)malloc(sizeof(double) * (size_t)j->k);
+    for (;;) {
+        int row = __sync_fetch_and_add(j->next, 1);
+        if (row >= rows) break;
+        const int bi = row / j->ho, oh = row % j->ho;
+        for (int ow = 0; ow < j->wo; ++ow) {
+            for (int ki = 0; ki < j->k; ++ki) acc[ki] = 0.0;
+            for (int ri = 0; ri < j->r; ++ri) {
+                const int th = oh + j->ph - ri;
+                if (th < 0 || th % j->sh != 0 || th / j->sh >= j->h) continue;
+                for (int si = 0; si < j->s; ++si) {
+                    const int tw = ow + j->pw - si;
+                    if (tw < 0 || tw % j->sw != 0 || tw / j->sw >= j->wd) continue;
+                    const float *xin =
+                        j->x + (((size_t)bi * j->h + th / j->sh) * j->wd + tw / j->sw) * j->c;
+                    for (int ci = 0; ci < j->c; ++ci) {
+                        const double xv = xin[ci];
+                        const float *wrow = j->w + ((size_t)(ci * j->r + ri) * j->s + si) * j->k;
+                        for (int ki = 0; ki < j->k; ++ki) acc[ki] += xv * (double)wrow[ki];
+                    }
+                }
+            }
+            float *out = j->y + (((size_t)bi * j->ho + oh) * j->wo + ow) * j->k;
+            for (int ki = 0; ki < j->k; ++ki) out[ki] = (float)acc[ki];
+        }
+    }
+    free(acc);
+    return NULL;
+}
+
+ORACLE_API int oracle_conv_transpose2d_nhwc(const float *x, const float *w, float *y, int n, int h,
+                                            int wd, int c, int k, int r, int s, int stride_h,
+                                            int stride_w, int pad_h, int pad_w, int opad_h,
+                                            int opad_w, int nthreads)
+{
+    if (n <= 0 || h <= 0 || wd <= 0 || c <= 0 || k <= 0 || r <= 0 || s <= 0 || stride_h <= 0 ||
+        stride_w <= 0 || pad_h < 0 || pad_w < 0 || opad_h < 0 || opad_w < 0)
+        return -1;
+    /* H_out = (H_in - 1) * stride - 2 * pad + kernel + output_padding (conv_transpose.rs:36-37) */
+    const int ho = (h - 1) * stride_h - 2 * pad_h + r + opad_h;
+    const int wo = (wd - 1) * stride_w - 2 * pad_w + s + opad_w;
+    if (ho <= 0 || wo <= 0) return -1;
+    if (nthreads < 1) nthreads = 1;
+    if (nthreads > 256) nthreads = 256;
+    volatile int next = 0;
+    convt_job j = {x, w, y, n, h, wd, c, k, r, s, stride_h, stride_w, pad_h, pad_w, ho, wo, &next};
+    pthread_t th[256];
+    int started = 0;
+    for (int t = 0; t < nthreads - 1; ++t)
+        if (pthread_create(&th[started], NULL, convt_worker, &j) == 0) ++started;
+    convt_worker(&j);
     for (int t = 0; t < started; ++t) pthread_join(th[t], NULL);
     return 0;
 }

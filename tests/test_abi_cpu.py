@@ -82,12 +82,16 @@ def test_compute_before_init_is_unknown_error():
     assert "tracea_init" in capi.last_error()
 
 
-def test_conv_transpose_is_unsupported():
+def test_conv_transpose_before_init_is_unknown_error():
+    # src/interface/c_bindings.rs:299: no runtime -> UnknownError, before any view is read
     l = capi.lib()
+    l.tracea_shutdown()
     shape = (C.c_uint64 * 4)(1, 4, 4, 8)
     tv = capi.TensorView(None, 4, shape, None, capi.F16, 0)
     st = l.tracea_conv_transpose2d(tv, tv, None, None, C.byref(tv), capi.ConvTranspose2dParams())
-    assert st == capi.UNSUPPORTED_CONFIG
+    assert st == capi.UNKNOWN_ERROR and "tracea_init" in capi.last_error()
+    st = l.tracea_conv_transpose2d_ex(tv, tv, C.byref(tv), capi.ConvTranspose2dParams(), None, 0)
+    assert st == capi.UNKNOWN_ERROR
 
 
 @pytest.mark.parametrize("shape", [

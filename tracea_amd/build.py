@@ -34,7 +34,7 @@ COMMON = ["-I" + INCLUDE, "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "
 HOST_SOURCES = ["abi.cpp", "tuner_abi.cpp", "graph_abi.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
                 "host/pipeline_config.cpp", "host/gaussian_process.cpp", "host/autotuner.cpp",
                 "host/graph_fusion.cpp"]
-DEVICE_SOURCES = ["support_kernels.hip", "attention_kernels.hip"]
+DEVICE_SOURCES = ["support_kernels.hip", "conv_transpose_kernels.hip", "attention_kernels.hip"]
 
 
 def hipcc():

@@ -91,6 +91,8 @@ SIGNATURES = {
     "tracea_tune_gemm": (Result, [C.c_size_t, C.c_size_t, C.c_size_t]),
     "tracea_tune_fa2": (Result, [C.c_size_t, C.c_size_t, C.c_size_t, C.c_size_t, C.c_bool]),
     "tracea_tune_conv2d": (Result, [C.c_size_t] * 10),
+    "tracea_conv_transpose2d_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), ConvTranspose2dParams,
+                                             C.POINTER(EpilogueOp), C.c_uint32]),
     "tracea_conv2d_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), Conv2dParams,
                                    C.POINTER(EpilogueOp), C.c_uint32]),
     "tracea_gemm_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), GemmParams,

@@ -108,12 +108,16 @@ TraceaStatus tracea_conv2d_ex(TraceaTensorView x, TraceaTensorView w, TraceaTens
   TRACEA_GUARDED(dispatch_conv2d_ops(x, w, out, params, ops, n_ops))
 }
 
-TraceaStatus tracea_conv_transpose2d(TraceaTensorView, TraceaTensorView, const TraceaTensorView *,
-                                     const TraceaTensorView *, TraceaTensorView *,
-                                     TraceaConvTranspose2dParams) {
-  return fail(TRACEA_UNSUPPORTED_CONFIG,
-              "tracea_conv_transpose2d: transposed convolution is outside the accelerated "
-              "GEMM / Conv2d / attention path of this build");
+TraceaStatus tracea_conv_transpose2d(TraceaTensorView x, TraceaTensorView w, const TraceaTensorView *b,
+                                     const TraceaTensorView *residual, TraceaTensorView *out,
+                                     TraceaConvTranspose2dParams params) {
+  TRACEA_GUARDED(dispatch_conv_transpose2d_kind(x, w, b, residual, out, params))
+}
+
+TraceaStatus tracea_conv_transpose2d_ex(TraceaTensorView x, TraceaTensorView w, TraceaTensorView *out,
+                                        TraceaConvTranspose2dParams params, const TraceaEpilogueOp *ops,
+                                        uint32_t n_ops) {
+  TRACEA_GUARDED(dispatch_conv_transpose2d_ops(x, w, out, params, ops, n_ops))
 }
 
 TraceaStatus tracea_attention(TraceaTensorView q, TraceaTensorView k, TraceaTensorView v,

@@ -93,6 +93,23 @@ struct GenericGemmArgs {
 };
 int launch_gemm_generic(const GenericGemmArgs &args, hipStream_t stream);
 
+// Second stage of the transposed convolution: gathers the per-tap partial
+// products `cols` (one row per input pixel, one column per (r, s, k)) into the
+// output pixels and applies the operator chain.
+struct Col2imArgs {
+  const float *cols;
+  void *out;
+  int out_dtype;
+  long long ld_cols;           // row stride of cols, elements
+  long long ldc;               // output pixel pitch, elements
+  long long st_r, st_s, st_k;  // column of (r, s, k) inside a row of cols
+  int b0, nb;                  // images this launch covers: b0 .. b0+nb-1 (cols row 0 is image b0)
+  int h_in, w_in, h_out, w_out, k_out, r_sz, s_sz;
+  int stride_h, stride_w, pad_h, pad_w;
+  EpilogueChain epi;
+};
+int launch_col2im_epilogue(const Col2imArgs &args, hipStream_t stream);
+
 struct AttentionVariant {
   const char *name;
   int block_q, block_kv, waves;

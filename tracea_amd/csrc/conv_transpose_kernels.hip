@@ -1,0 +1,74 @@
+// Transposed convolution, second stage.
+//
+// The reference computes y[b,ho,wo,k] = sum over (c,r,s) of
+// x[b,(ho+pad-r)/stride,(wo+pad-s)/stride,c] * w[c,r,s,k] where both divisions
+// are exact (src/emitter/conv_transpose.rs:207-225), as one implicit GEMM whose
+// K axis runs over every tap, so stride^2 - 1 of every stride^2 products are
+// zeros.  Here the sum is split: a plain GEMM cols[(b,hi,wi),(r,s,k)] =
+// x[(b,hi,wi),c] . w[c,(r,s,k)] does exactly the non-zero products on the matrix
+// cores (NHWC activations and the reference's [C*R*S, K] filter storage are
+// already those two row-major matrices), and this kernel adds, for each output
+// pixel, the ceil(R/stride_h) * ceil(S/stride_w) entries of cols that land on
+// it, runs the operator chain and stores.  It reads cols once and writes the
+// output once: bound by HBM.
+#include "contraction_kernel.hpp"
+
+namespace tracea_amd {
+
+// One thread per output pixel and V consecutive channels (V = 4 when channels
+// are the contiguous column index of cols, else 1).  Consecutive threads take
+// consecutive channel groups, so a wave reads whole rows of cols.
+template <int V>
+__global__ void __launch_bounds__(256) col2im_epilogue_kernel(const Col2imArgs a) {
+  const unsigned groups = (unsigned)(a.k_out + V - 1) / V;
+  const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+  const unsigned total = (unsigned)a.nb * a.h_out * a.w_out * groups;  // < 2^31, checked by the host
+  if (idx >= total) return;
+  const unsigned g = idx % groups, p = idx / groups;
+  const unsigned ow = p % (unsigned)a.w_out, q = p / (unsigned)a.w_out;
+  const unsigned oh = q % (unsigned)a.h_out, bl = q / (unsigned)a.h_out;
+  const int n = (int)g * V;
+  const int nvalid = a.k_out - n;
+
+  float acc[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) acc[e] = 0.0f;
+  // taps r with (oh + pad_h - r) divisible by stride_h: r = r0, r0 + stride_h, ...
+  // and the input row falls by one per step
+  const int th = (int)oh + a.pad_h, tw = (int)ow + a.pad_w;
+  const int r0 = th % a.stride_h, s0 = tw % a.stride_w;
+  const int hi0 = th / a.stride_h, wi0 = tw / a.stride_w;
+  const float *img = a.cols + (long long)bl * a.h_in * a.w_in * a.ld_cols + (long long)n * a.st_k;
+  for (int r = r0, hi = hi0; r < a.r_sz && hi >= 0; r += a.stride_h, --hi) {
+    if (hi >= a.h_in) continue;
+    for (int s = s0, wi = wi0; s < a.s_sz && wi >= 0; s += a.stride_w, --wi) {
+      if (wi >= a.w_in) continue;
+      const float *src = img + ((long long)hi * a.w_in + wi) * a.ld_cols + r * a.st_r + s * a.st_s;
+      if constexpr (V == 4) {
+        const f32x4 t = *(const f32x4 *)src;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] += t[e];
+      } else {
+        acc[0] += src[0];
+      }
+    }
+  }
+  const long long m = ((long long)(a.b0 + (int)bl) * a.h_out + oh) * a.w_out + ow;
+  apply_epilogue<V>(acc, m, n, nvalid, a.epi);
+  store_from_float<V>(a.out, a.out_dtype, m * a.ldc + n, nvalid, acc);
+}
+
+int launch_col2im_epilogue(const Col2imArgs &a, hipStream_t stream) {
+  const bool vec = a.st_k == 1 && a.k_out % 4 == 0 && a.ld_cols % 4 == 0 && a.st_r % 4 == 0 && a.st_s % 4 == 0 &&
+                   (((uintptr_t)a.cols) & 15) == 0;
+  const long long groups = vec ? a.k_out / 4 : a.k_out;
+  const long long total = (long long)a.nb * a.h_out * a.w_out * groups;
+  if (total <= 0) return 0;
+  if (total >= (1ll << 31)) return (int)hipErrorInvalidValue;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (vec) hipLaunchKernelGGL(col2im_epilogue_kernel<4>, grid, block, 0, stream, a);
+  else hipLaunchKernelGGL(col2im_epilogue_kernel<1>, grid, block, 0, stream, a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace tracea_amd

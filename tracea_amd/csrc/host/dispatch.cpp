@@ -6,6 +6,7 @@
 // UNSUPPORTED_CONFIG; host pointers -> CPU_ERROR; HIP failures -> CUDA_ERROR.
 #include "dispatch.hpp"
 
+#include <algorithm>
 #include <atomic>
 #include <cmath>
 #include <cstring>
@@ -412,7 +413,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
   DeviceScope scope(c.device);
   if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
 
-  if (is_half(a.dtype) && K > 0) {
+  if (is_half(a.dtype) && b.dtype == a.dtype && K > 0) {
     const bool a_ok = a.stride[1] == 1 && a.stride[0] % 8 == 0 && K % 8 == 0 && aligned(a.ptr, 16);
     const bool b_kcontig = b.stride[0] == 1 && b.stride[1] % 8 == 0 && aligned(b.ptr, 16);
     const bool b_ncontig = b.stride[1] == 1 && b.stride[0] % 8 == 0 && N % 8 == 0 && aligned(b.ptr, 16);
@@ -443,7 +444,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       return hip_status("gemm launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
     }
   }
-  if (a.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32 && K > 0 &&
+  if (a.dtype == TRACEA_DTYPE_FLOAT32 && b.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32 && K > 0 &&
       a.stride[1] == 1 && b.stride[1] == 1 && c.stride[1] == 1 && K % 4 == 0 && N % 4 == 0 &&
       a.stride[0] % 4 == 0 && b.stride[0] % 4 == 0 && aligned(a.ptr, 16) && aligned(b.ptr, 16)) {
     ContractionArgs args{};
@@ -745,6 +746,209 @@ TraceaStatus dispatch_conv2d_ops(const TraceaTensorView &tx, const TraceaTensorV
   st = lower_chain("tracea_conv2d_ex", ops, n_ops, plan.out.shape[3], plan.out.shape[3], &chain);
   if (st != TRACEA_SUCCESS) return st;
   return run_conv(plan, chain, (hipStream_t)params.stream);
+}
+
+// ---- ConvTranspose2d ---------------------------------------------------------------
+// cols = x[(b,hi,wi), c] . w[c, (k,r,s)] on the GEMM kernels, then the gather
+// kernel sums the taps that land on each output pixel and runs the chain.
+namespace {
+
+// The filter bank [K,R,S,C] seen as the matrix B[c, j], j running densely over
+// (k, r, s) in whatever order the strides give.
+struct FilterMatrix {
+  bool c_inner;        // true: B is K-contiguous (element (c, j) at j*ld + c); false: row-major, (c, j) at c*ld + j
+  long long ld;
+  long long col[3];    // column of one step of k, r, s
+  long long columns;   // K*R*S
+};
+
+bool dense_block(const View &w, long long unit, long long *col) {
+  int order[3] = {0, 1, 2};
+  for (int i = 0; i < 3; ++i)
+    for (int j = i + 1; j < 3; ++j)
+      if (w.stride[order[j]] < w.stride[order[i]]) std::swap(order[i], order[j]);
+  long long expect = unit;
+  for (int i = 0; i < 3; ++i) {
+    const int d = order[i];
+    col[d] = 0;
+    if (w.shape[d] == 1) continue;
+    if (w.stride[d] != expect) return false;
+    col[d] = expect / unit;
+    expect *= w.shape[d];
+  }
+  return true;
+}
+
+bool filter_as_matrix(const View &w, FilterMatrix *f) {
+  const long long C = w.shape[3], J = w.shape[0] * w.shape[1] * w.shape[2];
+  f->columns = J;
+  // input channels outermost: the reference kernel's [C*R*S, K] rows (C, R, S, K), or (C, K, R, S)
+  if (dense_block(w, 1, f->col) && (C == 1 || w.stride[3] >= J)) {
+    f->c_inner = false;
+    f->ld = C == 1 ? J : w.stride[3];
+    return true;
+  }
+  // input channels innermost, e.g. contiguous [K,R,S,C]
+  if (C == 1 || w.stride[3] == 1) {
+    long long unit = 0;
+    for (int d = 0; d < 3; ++d)
+      if (w.shape[d] > 1 && (unit == 0 || w.stride[d] < unit)) unit = w.stride[d];
+    if (unit == 0) unit = C;
+    if (unit >= C && dense_block(w, unit, f->col)) {
+      f->c_inner = true;
+      f->ld = unit;
+      return true;
+    }
+  }
+  return false;
+}
+
+struct ConvTransposePlan {
+  View x, w, out;
+  FilterMatrix fm;
+  int stride_h, stride_w, pad_h, pad_w;
+  long long ldx, ldc;
+};
+
+TraceaStatus conv_transpose_common(const TraceaTensorView &tx, const TraceaTensorView &tw, TraceaTensorView *tout,
+                                   const TraceaConvTranspose2dParams &p, ConvTransposePlan *plan) {
+  const char *me = "tracea_conv_transpose2d";
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "%s: tracea_init has not been called", me);
+  if (tout == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: output view is NULL", me);
+  // the reference states groups = 1 and dilation = 1 as constraints and reads neither
+  // field (src/emitter/conv_transpose.rs:26-29); 0 is taken as "left unset"
+  if (p.groups > 1) return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: groups=%u (only groups=1)", me, p.groups);
+  if (p.dilation_h > 1 || p.dilation_w > 1)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dilation %ux%u (only 1)", me, p.dilation_h, p.dilation_w);
+  if (p.stride_h == 0 || p.stride_w == 0) return fail(TRACEA_INVALID_PARAMS, "%s: stride must be at least 1", me);
+  TraceaStatus st;
+  View &x = plan->x, &w = plan->w, &out = plan->out;
+  if ((st = read_view("tracea_conv_transpose2d: x", tx, 4, &x)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_conv_transpose2d: w", tw, 4, &w)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_conv_transpose2d: out", *tout, 4, &out)) != TRACEA_SUCCESS) return st;
+  if (!is_float_type(x.dtype) || w.dtype != x.dtype)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: activations %s / filters %s; f32, f16 or bf16 (both alike) required",
+                me, dtype_name(x.dtype), dtype_name(w.dtype));
+  if (!is_float_type(out.dtype))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: output dtype %s unsupported", me, dtype_name(out.dtype));
+  if ((st = check_device(me, out.device)) != TRACEA_SUCCESS) return st;
+  if (x.device != out.device || w.device != out.device)
+    return fail(TRACEA_INVALID_PARAMS, "%s: operands live on different devices", me);
+  const long long N = x.shape[0], H = x.shape[1], W = x.shape[2], C = x.shape[3];
+  const long long K = w.shape[0], R = w.shape[1], S = w.shape[2];
+  if (w.shape[3] != C) return fail(TRACEA_INVALID_PARAMS, "%s: x has %lld channels, w expects %lld", me, C, w.shape[3]);
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0)
+    return fail(TRACEA_INVALID_PARAMS, "%s: empty dimension", me);
+  const long long big = 1ll << 31;
+  if (N >= big || H >= big || W >= big || C >= big || K >= big || R >= big || S >= big || K * R * S >= big)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dimension exceeds 2^31-1", me);
+  // H_out = (H_in - 1) * stride - 2 * pad + kernel + output_padding (conv_transpose.rs:36-37)
+  const long long Ho = (H - 1) * p.stride_h - 2ll * p.padding_h + R + p.output_padding_h;
+  const long long Wo = (W - 1) * p.stride_w - 2ll * p.padding_w + S + p.output_padding_w;
+  if (Ho <= 0 || Wo <= 0) return fail(TRACEA_INVALID_PARAMS, "%s: output would be %lldx%lld", me, Ho, Wo);
+  if (Ho >= big || Wo >= big) return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dimension exceeds 2^31-1", me);
+  if (out.shape[0] != N || out.shape[1] != Ho || out.shape[2] != Wo || out.shape[3] != K)
+    return fail(TRACEA_INVALID_PARAMS, "%s: output shape must be [%lld,%lld,%lld,%lld]", me, N, Ho, Wo, K);
+  const long long ldx = x.stride[2];
+  if (!(x.stride[3] == 1 && ldx >= C && x.stride[1] == W * ldx && x.stride[0] == H * W * ldx))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: activations must be channel-contiguous NHWC", me);
+  const long long ldc = out.stride[2];
+  if (!(out.stride[3] == 1 && ldc >= K && out.stride[1] == Wo * ldc && out.stride[0] == Ho * Wo * ldc))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: output must be channel-contiguous NHWK", me);
+  if (!filter_as_matrix(w, &plan->fm))
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "%s: filters (dims [K,R,S,C]) must be stored with the input channels outermost or innermost "
+                "and the other three dims dense, e.g. [C,R,S,K], [C,K,R,S] or [K,R,S,C]", me);
+  plan->stride_h = (int)p.stride_h; plan->stride_w = (int)p.stride_w;
+  plan->pad_h = (int)p.padding_h; plan->pad_w = (int)p.padding_w;
+  plan->ldx = ldx; plan->ldc = ldc;
+  return TRACEA_SUCCESS;
+}
+
+TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueChain &chain, hipStream_t stream) {
+  const View &x = plan.x, &w = plan.w, &out = plan.out;
+  const long long N = x.shape[0], H = x.shape[1], W = x.shape[2], C = x.shape[3];
+  const long long K = w.shape[0], Ho = out.shape[1], Wo = out.shape[2];
+  const long long J = plan.fm.columns;
+  DeviceScope scope(out.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  // Images per pass: the partial products of a pass stay below 512 MiB, the GEMM
+  // rows and the gather kernel's thread count below 2^31.
+  const long long per_image = H * W * J * 4;
+  long long nb = per_image > 0 ? (512ll << 20) / per_image : N;
+  if (nb < 1) nb = 1;
+  if (nb > N) nb = N;
+  const long long lim = (1ll << 31) - 1;
+  while (nb > 1 && (nb * H * W > lim || nb * Ho * Wo * K > lim)) nb = (nb + 1) / 2;
+  if (H * W > lim || Ho * Wo * K > lim || per_image / 4 >= (1ll << 40))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv_transpose2d: one image is too large");
+  float *cols = nullptr;
+  hipError_t e = hipMallocAsync((void **)&cols, (size_t)(nb * per_image), stream);
+  if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+  TraceaStatus st = TRACEA_SUCCESS;
+  for (long long b0 = 0; b0 < N && st == TRACEA_SUCCESS; b0 += nb) {
+    const long long cnt = N - b0 < nb ? N - b0 : nb;
+    View a = x, b = w, c{};
+    a.rank = b.rank = c.rank = 2;
+    a.ptr = (char *)x.ptr + b0 * x.stride[0] * elem_size(x.dtype);
+    a.shape[0] = cnt * H * W; a.shape[1] = C;
+    a.stride[0] = plan.ldx; a.stride[1] = 1;
+    b.shape[0] = C; b.shape[1] = J;
+    if (plan.fm.c_inner) { b.stride[0] = 1; b.stride[1] = plan.fm.ld; }
+    else { b.stride[0] = plan.fm.ld; b.stride[1] = 1; }
+    c.ptr = cols; c.dtype = TRACEA_DTYPE_FLOAT32; c.device = out.device;
+    c.shape[0] = a.shape[0]; c.shape[1] = J;
+    c.stride[0] = J; c.stride[1] = 1;
+    EpilogueChain none{};
+    st = run_gemm(a, b, c, none, stream);
+    if (st != TRACEA_SUCCESS) break;
+    Col2imArgs g{};
+    g.cols = cols; g.out = out.ptr; g.out_dtype = out.dtype;
+    g.ld_cols = J; g.ldc = plan.ldc;
+    g.st_k = plan.fm.col[0]; g.st_r = plan.fm.col[1]; g.st_s = plan.fm.col[2];
+    g.b0 = (int)b0; g.nb = (int)cnt;
+    g.h_in = (int)H; g.w_in = (int)W; g.h_out = (int)Ho; g.w_out = (int)Wo; g.k_out = (int)K;
+    g.r_sz = (int)w.shape[1]; g.s_sz = (int)w.shape[2];
+    g.stride_h = plan.stride_h; g.stride_w = plan.stride_w; g.pad_h = plan.pad_h; g.pad_w = plan.pad_w;
+    g.epi = chain;
+    st = hip_status("conv_transpose2d gather launch", launch_col2im_epilogue(g, stream));
+  }
+  e = hipFreeAsync(cols, stream);
+  if (st == TRACEA_SUCCESS && e != hipSuccess) st = hip_status("tracea_conv_transpose2d: workspace release", (int)e);
+  return st;
+}
+
+}  // namespace
+
+TraceaStatus dispatch_conv_transpose2d_kind(const TraceaTensorView &tx, const TraceaTensorView &tw,
+                                            const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                            TraceaTensorView *tout, const TraceaConvTranspose2dParams &params) {
+  ConvTransposePlan plan;
+  TraceaStatus st = conv_transpose_common(tx, tw, tout, params, &plan);
+  if (st != TRACEA_SUCCESS) return st;
+  TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
+  const int n = kind_to_ops((int)params.epilogue, bias, residual, ops);
+  if (n < 0)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_conv_transpose2d: unknown epilogue kind %d", (int)params.epilogue);
+  st = check_bias_residual("tracea_conv_transpose2d", bias, residual, plan.out.shape[3], plan.out, plan.out.device,
+                           ops, n);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain("tracea_conv_transpose2d", ops, (uint32_t)n, plan.out.shape[3], plan.out.shape[3], &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  return run_conv_transpose(plan, chain, (hipStream_t)params.stream);
+}
+
+TraceaStatus dispatch_conv_transpose2d_ops(const TraceaTensorView &tx, const TraceaTensorView &tw,
+                                           TraceaTensorView *tout, const TraceaConvTranspose2dParams &params,
+                                           const TraceaEpilogueOp *ops, uint32_t n_ops) {
+  ConvTransposePlan plan;
+  TraceaStatus st = conv_transpose_common(tx, tw, tout, params, &plan);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain("tracea_conv_transpose2d_ex", ops, n_ops, plan.out.shape[3], plan.out.shape[3], &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  return run_conv_transpose(plan, chain, (hipStream_t)params.stream);
 }
 
 // ---- attention ---------------------------------------------------------------------

@@ -46,6 +46,12 @@ TraceaStatus dispatch_conv2d_kind(const TraceaTensorView &x, const TraceaTensorV
 TraceaStatus dispatch_conv2d_ops(const TraceaTensorView &x, const TraceaTensorView &w,
                                  TraceaTensorView *out, const TraceaConv2dParams &params,
                                  const TraceaEpilogueOp *ops, uint32_t n_ops);
+TraceaStatus dispatch_conv_transpose2d_kind(const TraceaTensorView &x, const TraceaTensorView &w,
+                                            const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                            TraceaTensorView *out, const TraceaConvTranspose2dParams &params);
+TraceaStatus dispatch_conv_transpose2d_ops(const TraceaTensorView &x, const TraceaTensorView &w,
+                                           TraceaTensorView *out, const TraceaConvTranspose2dParams &params,
+                                           const TraceaEpilogueOp *ops, uint32_t n_ops);
 TraceaStatus dispatch_attention(const TraceaTensorView &q, const TraceaTensorView &k,
                                 const TraceaTensorView &v, TraceaTensorView *o,
                                 const TraceaAttentionParams &params);

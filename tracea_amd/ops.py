@@ -161,6 +161,65 @@ def conv2d_ex(x, w, ops, stride=1, padding=0, dilation=1, out=None, weight_layou
     return out
 
 
+def conv_transpose_out_shape(x_shape, w_shape, stride, padding, output_padding):
+    n, h, w, _ = x_shape
+    k, r, s, _ = w_shape
+    ho = (h - 1) * stride[0] - 2 * padding[0] + r + output_padding[0]
+    wo = (w - 1) * stride[1] - 2 * padding[1] + s + output_padding[1]
+    return (n, ho, wo, k)
+
+
+def _transposed_weight_view(w, layout):
+    """Filter view with dims [K,R,S,C] (K output channels) whatever the storage order."""
+    order = {"crsk": (3, 1, 2, 0),   # the reference kernel's [C*R*S, K] rows
+             "ckrs": (1, 2, 3, 0),   # torch.nn.ConvTranspose2d.weight
+             "krsc": (0, 1, 2, 3)}.get(layout)
+    if order is None:
+        raise ValueError("weight layout must be 'crsk', 'ckrs' or 'krsc'")
+    return _view(w, shape=tuple(w.shape[i] for i in order), stride=tuple(w.stride()[i] for i in order))
+
+
+def _conv_transpose_setup(x, w, stride, padding, output_padding, out, weight_layout, out_dtype):
+    stride, padding, output_padding = _pair(stride), _pair(padding), _pair(output_padding)
+    vw = _transposed_weight_view(w, weight_layout)
+    wshape = tuple(vw.c.shape[i] for i in range(4))
+    if out is None:
+        out = torch.empty(conv_transpose_out_shape(x.shape, wshape, stride, padding, output_padding),
+                          dtype=out_dtype or x.dtype, device=x.device)
+    return vw, out, stride, padding, output_padding
+
+
+def conv_transpose2d(x, w, bias=None, residual=None, stride=1, padding=0, output_padding=0, epilogue="none",
+                     out=None, weight_layout="crsk", out_dtype=None):
+    """x [N,H,W,C] (NHWC); w [C,R,S,K] ('crsk'), [C,K,R,S] ('ckrs') or [K,R,S,C] ('krsc'); out [N,Ho,Wo,K]
+    with Ho = (H-1)*stride - 2*padding + R + output_padding."""
+    vw, out, stride, padding, output_padding = _conv_transpose_setup(x, w, stride, padding, output_padding, out,
+                                                                     weight_layout, out_dtype)
+    vx, vo = _view(x), _view(out)
+    vbias = _view(bias) if bias is not None else None
+    vres = _view(residual) if residual is not None else None
+    params = capi.ConvTranspose2dParams(stride[0], stride[1], padding[0], padding[1], output_padding[0],
+                                        output_padding[1], 1, 1, 1, parse_epilogue(epilogue), _stream(x))
+    st = capi.lib().tracea_conv_transpose2d(vx.c, vw.c, C.byref(vbias.c) if vbias else None,
+                                            C.byref(vres.c) if vres else None, C.byref(vo.c), params)
+    capi.check("tracea_conv_transpose2d", st)
+    return out
+
+
+def conv_transpose2d_ex(x, w, ops, stride=1, padding=0, output_padding=0, out=None, weight_layout="crsk",
+                        out_dtype=None):
+    """Transposed convolution with an explicit operator chain."""
+    vw, out, stride, padding, output_padding = _conv_transpose_setup(x, w, stride, padding, output_padding, out,
+                                                                     weight_layout, out_dtype)
+    vx, vo = _view(x), _view(out)
+    arr, _keep = _ops_array(ops)
+    params = capi.ConvTranspose2dParams(stride[0], stride[1], padding[0], padding[1], output_padding[0],
+                                        output_padding[1], 1, 1, 1, capi.EPI_IDENTITY, _stream(x))
+    st = capi.lib().tracea_conv_transpose2d_ex(vx.c, vw.c, C.byref(vo.c), params, arr, len(ops))
+    capi.check("tracea_conv_transpose2d_ex", st)
+    return out
+
+
 def attention(q, k, v, causal=False, scale=0.0, out=None):
     """q,k,v [B,H,S,D] -> softmax(scale q k^T) v; scale 0 means 1/sqrt(D)."""
     if out is None:
