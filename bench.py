@@ -6,7 +6,7 @@ fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
 FlashAttention-2 forward named by the metric are timed in the same run and
 reported under "also".  Prints one JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|conv|attention|attention_causal|copy]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|conv|attention|attention_causal|conv_transpose|copy]
 """
 import argparse
 import json
@@ -22,7 +22,7 @@ PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
 # HBM-side bytes per launch of the dominant kernel of each workload, from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
 # (profiles/bench_kernels_mi355x.md); None where no counter run exists.
-TRAFFIC_BYTES = {"gemm": 235.2e6, "conv": 26.5e6, "attention": 537.1e6, "attention_causal": None, "copy": None}
+TRAFFIC_BYTES = {"gemm": 235.2e6, "conv": 26.5e6, "attention": 537.1e6, "attention_causal": None, "conv_transpose": None, "copy": None}
 METRIC = "TFLOPS + % fp16 MFMA peak: GEMM 4096^3, 3x3 implicit-GEMM conv, FA2 fwd"
 
 
@@ -55,6 +55,17 @@ def make_workload(name, torch, ops):
         flops = 4.0 * b * h * d * (s * (s + 1) / 2.0 if causal else float(s) * s)
         return ("bf16 FA2 forward B4 H32 S4096 D128 %s" % ("causal" if causal else "dense"),
                 flops, 2.0 * 4 * q.numel(), "bf16", lambda: ops.attention(q, k, v, causal=causal, out=o))
+    if name == "conv_transpose":
+        # the reference's VAE decoder layer at batch 8 (src/optimizer/benchmark.rs:572-575); FLOPs are
+        # the products that are not structurally zero, 1/stride^2 of the reference's 2*M*N*K count
+        n, h, w, cin, cout, r, st, pd = 8, 32, 32, 512, 256, 4, 2, 1
+        x = torch.randn(n, h, w, cin, device=dev, generator=g).half()
+        wt = (torch.randn(cin, r, r, cout, device=dev, generator=g) * (1.0 / (4 * cin)) ** 0.5).half()
+        ho = (h - 1) * st - 2 * pd + r
+        y = torch.empty(n, ho, ho, cout, device=dev, dtype=torch.float16)
+        return ("fp16 NHWC transposed conv N8 32x32x512->64x64x256 4x4 s2 p1",
+                2.0 * n * h * w * cin * r * r * cout, 2.0 * (x.numel() + wt.numel() + y.numel()), "f16",
+                lambda: ops.conv_transpose2d(x, wt, stride=st, padding=pd, out=y))
     if name == "copy":
         # calibration workload for the HBM traffic counters: a plain device copy of known size
         n = 256 << 20
@@ -139,7 +150,7 @@ def main():
     }
     if not args.no_extras:
         also = {}
-        for name in ("gemm", "conv", "attention", "attention_causal"):
+        for name in ("gemm", "conv", "attention", "attention_causal", "conv_transpose"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)

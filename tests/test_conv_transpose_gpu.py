@@ -72,13 +72,13 @@ def test_half_precision_operands(tracea_gpu, shape, dtype):
     assert_close_scaled(y32.cpu().numpy(), want, 1e-5 * math.sqrt(c * taps) + 1e-6, "%s f32 out" % (shape,))
 
 
-@pytest.mark.parametrize("layout", ["crsk", "ckrs", "krsc"])
+@pytest.mark.parametrize("layout", ["crsk", "ckrs", "krsc", "rskc"])
 @pytest.mark.parametrize("tdt", [torch.float32, torch.float16])
 def test_filter_storage_orders_agree(tracea_gpu, layout, tdt):
     shape = (2, 6, 6, 16, 8, 4, 4, 2, 1, 0)
     x, wt = _operands(shape, 3, round_f16)
     want = oracle.conv_transpose2d_nhwc(x, wt, 2, 1, 0)
-    perm = {"crsk": (0, 1, 2, 3), "ckrs": (0, 3, 1, 2), "krsc": (3, 1, 2, 0)}[layout]
+    perm = {"crsk": (0, 1, 2, 3), "ckrs": (0, 3, 1, 2), "krsc": (3, 1, 2, 0), "rskc": (1, 2, 3, 0)}[layout]
     dw = _dev(wt, tdt).permute(*perm).contiguous()
     y = tracea_gpu.conv_transpose2d(_dev(x, tdt), dw, stride=2, padding=1, weight_layout=layout,
                                     out_dtype=torch.float32)

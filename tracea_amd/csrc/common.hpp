@@ -110,6 +110,20 @@ struct Col2imArgs {
 };
 int launch_col2im_epilogue(const Col2imArgs &args, hipStream_t stream);
 
+// Copies a filter bank with dims [K,R,S,C] and arbitrary element strides into
+// the B operand of the transposed convolution's GEMM, columns ordered (r, s, k):
+// [R][S][K][C] (K-contiguous B, for the half-precision kernels) when c_inner,
+// else [C][R][S][K] (row-major B, for the fp32 kernel).
+struct FilterRepackArgs {
+  const void *w;
+  void *out;
+  int elem_bytes;  // 2 or 4
+  int c_inner;
+  int C, K, R, S;
+  long long sc, sk, sr, ss;  // element strides of c, k, r, s in w
+};
+int launch_filter_repack(const FilterRepackArgs &args, hipStream_t stream);
+
 struct AttentionVariant {
   const char *name;
   int block_q, block_kv, waves;

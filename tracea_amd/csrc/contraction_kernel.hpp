@@ -373,8 +373,7 @@ __device__ __forceinline__ void apply_epilogue_tab(float (&v)[8], long long m, i
 // Whether that holds is the same for the whole workgroup, so it is decided
 // once and the row loops are emitted twice, each behind a uniform branch.
 __device__ __forceinline__ bool chain_is_simple(const ChainPlan &plan, const ContractionArgs &args, int n0, int bn) {
-  bool ok = n0 + bn <= args.N && (args.ldc & 7) == 0 && (((uintptr_t)args.C) & 15) == 0 &&
-            args.out_dtype != DT_F32;
+  bool ok = n0 + bn <= args.N && (args.ldc & 7) == 0 && (((uintptr_t)args.C) & 15) == 0;
 #pragma unroll
   for (int o = 0; o < TRACEA_MAX_EPILOGUE_OPS; ++o) {
     const int kind = (int)((plan.kinds >> (4 * o)) & 15u);
@@ -394,7 +393,8 @@ __device__ __forceinline__ bool chain_is_simple(const ChainPlan &plan, const Con
 // stores come last.  One row at a time, every row paid an LDS round trip for
 // its staged values and one more per operator, back to back.
 // row_of(r) gives the output row of staged row r, or -1 if it does not exist.
-template <int DT, int TN, typename RowOf>
+// F32OUT: C holds fp32 (two 16-byte stores per lane and row) instead of DT.
+template <int DT, int TN, bool F32OUT = false, typename RowOf>
 __device__ __forceinline__ void simple_rows(const float *stage, int lane, int n, const ContractionArgs &args,
                                             const ChainPlan &plan, const float *tab, int bn, RowOf row_of) {
   constexpr int EP_PITCH = TN + 4, LPR = TN / 8, RPI = 64 / LPR, NIT = 32 / RPI;
@@ -466,7 +466,12 @@ __device__ __forceinline__ void simple_rows(const float *stage, int lane, int n,
     for (int g = 0; g < GROUP; ++g) {
       if (m[g] >= 0) {
         unsigned short *dst = (unsigned short *)args.C + m[g] * args.ldc + n;
-        if constexpr (DT == DT_F16) {
+        if constexpr (F32OUT) {
+          float *dst32 = (float *)args.C + m[g] * args.ldc + n;
+          const f32x4 lo = {v[g][0], v[g][1], v[g][2], v[g][3]}, hi = {v[g][4], v[g][5], v[g][6], v[g][7]};
+          *(f32x4 *)dst32 = lo;
+          *(f32x4 *)(dst32 + 4) = hi;
+        } else if constexpr (DT == DT_F16) {
           f16x8 h;
 #pragma unroll
           for (int e = 0; e < 8; ++e) h[e] = (_Float16)v[g][e];
@@ -599,9 +604,13 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 
   // The chain as the epilogue needs it, and the choice of its row body, are worked
   // out here: their scalar loads complete under the main loop instead of after it.
-  // (The output type equals the operand type on the specialised path.)
+  // (On the specialised path the output type is the operand type or fp32.)
   const ChainPlan plan = chain_plan(args.epi);
-  const bool simple = chain_is_simple(plan, args, n0, BN) && args.out_dtype == DT;
+  // (fp32 output takes it only where a wave holds at most 8 accumulator blocks: with 16,
+  // a second copy of the row body costs the compiler its register allocation.)
+  constexpr bool F32_SIMPLE = FM * FN <= 8;
+  const bool out_f32 = F32_SIMPLE && args.out_dtype == DT_F32;
+  const bool simple = chain_is_simple(plan, args, n0, BN) && (args.out_dtype == DT || out_f32);
 
   // This thread's entries of the epilogue operand table (see chain_table_value):
   // requested here so that they arrive under the main loop.
@@ -1099,8 +1108,13 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     __builtin_amdgcn_wave_barrier();
     if (simple) {
       const int mb = m0 + wm * TM + i * 32;
-      simple_rows<DT, TN>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN,
-                          [&](int r) -> long long { return mb + r < M ? (long long)(mb + r) : -1ll; });
+      auto row_of = [&](int r) -> long long { return mb + r < M ? (long long)(mb + r) : -1ll; };
+      if constexpr (F32_SIMPLE) {
+        if (out_f32) simple_rows<DT, TN, true>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
+        else simple_rows<DT, TN, false>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
+      } else {
+        simple_rows<DT, TN, false>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
+      }
     } else {
       for (int r = er; r < 32; r += RPI) {
         const int m = m0 + wm * TM + i * 32 + r;

@@ -6,8 +6,9 @@
 // K axis runs over every tap, so stride^2 - 1 of every stride^2 products are
 // zeros.  Here the sum is split: a plain GEMM cols[(b,hi,wi),(r,s,k)] =
 // x[(b,hi,wi),c] . w[c,(r,s,k)] does exactly the non-zero products on the matrix
-// cores (NHWC activations and the reference's [C*R*S, K] filter storage are
-// already those two row-major matrices), and this kernel adds, for each output
+// cores (NHWC activations are already the row-major left matrix; the filter bank
+// is first copied into the K-contiguous order the fast GEMM kernels read, a few
+// megabytes), and the gather kernel adds, for each output
 // pixel, the ceil(R/stride_h) * ceil(S/stride_w) entries of cols that land on
 // it, runs the operator chain and stores.  It reads cols once and writes the
 // output once: bound by HBM.
@@ -68,6 +69,47 @@ int launch_col2im_epilogue(const Col2imArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)((total + 255) / 256)), block(256);
   if (vec) hipLaunchKernelGGL(col2im_epilogue_kernel<4>, grid, block, 0, stream, a);
   else hipLaunchKernelGGL(col2im_epilogue_kernel<1>, grid, block, 0, stream, a);
+  return (int)hipGetLastError();
+}
+
+// Filter repack: a 64 (c) x 64 (k) tile per workgroup and tap, transposed through
+// LDS so that the side with the smaller source stride is read along the lanes and
+// the destination is written along its contiguous side.
+template <typename T>
+__global__ void __launch_bounds__(256) filter_repack_kernel(const FilterRepackArgs a) {
+  __shared__ T tile[64][65];
+  const int c0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int r = blockIdx.z / a.S, s = blockIdx.z % a.S;
+  const int fast = threadIdx.x & 63, slow = threadIdx.x >> 6;
+  const bool k_fast = a.sk <= a.sc;
+  const T *src = (const T *)a.w + (long long)r * a.sr + (long long)s * a.ss;
+  for (int i = 0; i < 16; ++i) {
+    const int kk = k_fast ? fast : slow + i * 4, cc = k_fast ? slow + i * 4 : fast;
+    const int k = k0 + kk, c = c0 + cc;
+    if (k < a.K && c < a.C) tile[cc][kk] = src[(long long)k * a.sk + (long long)c * a.sc];
+  }
+  __syncthreads();
+  if (a.c_inner) {
+    T *dst = (T *)a.out + (long long)blockIdx.z * a.K * a.C;
+    for (int i = 0; i < 16; ++i) {
+      const int kk = slow + i * 4, k = k0 + kk, c = c0 + fast;
+      if (k < a.K && c < a.C) dst[(long long)k * a.C + c] = tile[fast][kk];
+    }
+  } else {
+    T *dst = (T *)a.out + (long long)blockIdx.z * a.K;
+    const long long row = (long long)a.R * a.S * a.K;
+    for (int i = 0; i < 16; ++i) {
+      const int cc = slow + i * 4, c = c0 + cc, k = k0 + fast;
+      if (k < a.K && c < a.C) dst[(long long)c * row + k] = tile[cc][fast];
+    }
+  }
+}
+
+int launch_filter_repack(const FilterRepackArgs &a, hipStream_t stream) {
+  const dim3 grid((unsigned)((a.C + 63) / 64), (unsigned)((a.K + 63) / 64), (unsigned)(a.R * a.S)), block(256);
+  if (grid.y > 65535 || grid.z > 65535) return (int)hipErrorInvalidValue;
+  if (a.elem_bytes == 4) hipLaunchKernelGGL(filter_repack_kernel<unsigned>, grid, block, 0, stream, a);
+  else hipLaunchKernelGGL(filter_repack_kernel<unsigned short>, grid, block, 0, stream, a);
   return (int)hipGetLastError();
 }
 

@@ -882,10 +882,32 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
   while (nb > 1 && (nb * H * W > lim || nb * Ho * Wo * K > lim)) nb = (nb + 1) / 2;
   if (H * W > lim || Ho * Wo * K > lim || per_image / 4 >= (1ll << 40))
     return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv_transpose2d: one image is too large");
-  float *cols = nullptr;
-  hipError_t e = hipMallocAsync((void **)&cols, (size_t)(nb * per_image), stream);
+  // Filters already stored in the order the GEMM reads are used in place; any other order is
+  // copied into it (C*R*S*K elements, next to the partial products in the temporary buffer).
+  const long long R = w.shape[1], S = w.shape[2];
+  // (the fp32 GEMM kernel reads a row-major B: there the order is [C,R,S,K], the reference's own)
+  const bool c_inner = is_half(x.dtype);
+  const bool in_place = plan.fm.c_inner == c_inner && plan.fm.ld == (c_inner ? C : J) &&
+                        (K == 1 || plan.fm.col[0] == 1) && (S == 1 || plan.fm.col[2] == K) &&
+                        (R == 1 || plan.fm.col[1] == S * K);
+  const size_t cols_bytes = (size_t)(nb * per_image);
+  const size_t cols_padded = (cols_bytes + 255) & ~(size_t)255;
+  const size_t filt_bytes = in_place ? 0 : (size_t)(J * C) * elem_size(w.dtype);
+  char *ws = nullptr;
+  hipError_t e = hipMallocAsync((void **)&ws, cols_padded + filt_bytes, stream);
   if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+  float *cols = (float *)ws;
+  const void *filt = w.ptr;
   TraceaStatus st = TRACEA_SUCCESS;
+  if (!in_place) {
+    FilterRepackArgs f{};
+    f.w = w.ptr; f.out = ws + cols_padded; f.elem_bytes = elem_size(w.dtype);
+    f.c_inner = c_inner ? 1 : 0;
+    f.C = (int)C; f.K = (int)K; f.R = (int)R; f.S = (int)S;
+    f.sk = w.stride[0]; f.sr = w.stride[1]; f.ss = w.stride[2]; f.sc = w.stride[3];
+    st = hip_status("conv_transpose2d filter repack launch", launch_filter_repack(f, stream));
+    filt = f.out;
+  }
   for (long long b0 = 0; b0 < N && st == TRACEA_SUCCESS; b0 += nb) {
     const long long cnt = N - b0 < nb ? N - b0 : nb;
     View a = x, b = w, c{};
@@ -893,9 +915,10 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
     a.ptr = (char *)x.ptr + b0 * x.stride[0] * elem_size(x.dtype);
     a.shape[0] = cnt * H * W; a.shape[1] = C;
     a.stride[0] = plan.ldx; a.stride[1] = 1;
+    b.ptr = (void *)filt;
     b.shape[0] = C; b.shape[1] = J;
-    if (plan.fm.c_inner) { b.stride[0] = 1; b.stride[1] = plan.fm.ld; }
-    else { b.stride[0] = plan.fm.ld; b.stride[1] = 1; }
+    if (c_inner) { b.stride[0] = 1; b.stride[1] = C; }
+    else { b.stride[0] = J; b.stride[1] = 1; }
     c.ptr = cols; c.dtype = TRACEA_DTYPE_FLOAT32; c.device = out.device;
     c.shape[0] = a.shape[0]; c.shape[1] = J;
     c.stride[0] = J; c.stride[1] = 1;
@@ -905,15 +928,15 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
     Col2imArgs g{};
     g.cols = cols; g.out = out.ptr; g.out_dtype = out.dtype;
     g.ld_cols = J; g.ldc = plan.ldc;
-    g.st_k = plan.fm.col[0]; g.st_r = plan.fm.col[1]; g.st_s = plan.fm.col[2];
+    g.st_k = 1; g.st_s = K; g.st_r = S * K;
     g.b0 = (int)b0; g.nb = (int)cnt;
     g.h_in = (int)H; g.w_in = (int)W; g.h_out = (int)Ho; g.w_out = (int)Wo; g.k_out = (int)K;
-    g.r_sz = (int)w.shape[1]; g.s_sz = (int)w.shape[2];
+    g.r_sz = (int)R; g.s_sz = (int)S;
     g.stride_h = plan.stride_h; g.stride_w = plan.stride_w; g.pad_h = plan.pad_h; g.pad_w = plan.pad_w;
     g.epi = chain;
     st = hip_status("conv_transpose2d gather launch", launch_col2im_epilogue(g, stream));
   }
-  e = hipFreeAsync(cols, stream);
+  e = hipFreeAsync(ws, stream);
   if (st == TRACEA_SUCCESS && e != hipSuccess) st = hip_status("tracea_conv_transpose2d: workspace release", (int)e);
   return st;
 }

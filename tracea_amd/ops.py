@@ -173,9 +173,10 @@ def _transposed_weight_view(w, layout):
     """Filter view with dims [K,R,S,C] (K output channels) whatever the storage order."""
     order = {"crsk": (3, 1, 2, 0),   # the reference kernel's [C*R*S, K] rows
              "ckrs": (1, 2, 3, 0),   # torch.nn.ConvTranspose2d.weight
-             "krsc": (0, 1, 2, 3)}.get(layout)
+             "krsc": (0, 1, 2, 3),
+             "rskc": (2, 0, 1, 3)}.get(layout)  # what the half-precision GEMM stage reads in place
     if order is None:
-        raise ValueError("weight layout must be 'crsk', 'ckrs' or 'krsc'")
+        raise ValueError("weight layout must be 'crsk', 'ckrs', 'krsc' or 'rskc'")
     return _view(w, shape=tuple(w.shape[i] for i in order), stride=tuple(w.stride()[i] for i in order))
 
 
@@ -191,7 +192,8 @@ def _conv_transpose_setup(x, w, stride, padding, output_padding, out, weight_lay
 
 def conv_transpose2d(x, w, bias=None, residual=None, stride=1, padding=0, output_padding=0, epilogue="none",
                      out=None, weight_layout="crsk", out_dtype=None):
-    """x [N,H,W,C] (NHWC); w [C,R,S,K] ('crsk'), [C,K,R,S] ('ckrs') or [K,R,S,C] ('krsc'); out [N,Ho,Wo,K]
+    """x [N,H,W,C] (NHWC); w [C,R,S,K] ('crsk'), [C,K,R,S] ('ckrs'), [K,R,S,C] ('krsc') or [R,S,K,C]
+    ('rskc'); out [N,Ho,Wo,K]
     with Ho = (H-1)*stride - 2*padding + R + output_padding."""
     vw, out, stride, padding, output_padding = _conv_transpose_setup(x, w, stride, padding, output_padding, out,
                                                                      weight_layout, out_dtype)
