@@ -69,7 +69,8 @@ struct ContractionVariant {
   const char *name;
   int bm, bn, bk, waves_m, waves_n, stages;
   int pipeline;  // 0: operands read just in time; 1: read one k-step ahead, across the barrier;
-                 // 2: as 1, with direct-to-LDS tile loads (K-contiguous B only);
+                 // 2: as 1, with direct-to-LDS tile loads (an N-contiguous B is kept [k][n] in LDS
+                 //    and fetched with transposing LDS reads);
                  // 3: ring of `stages` LDS buffers, direct-to-LDS loads stages-1 tiles ahead
                  // 4: convolution only: input patch resident in LDS, filter tiles through a ring of `stages`
   size_t lds_bytes;

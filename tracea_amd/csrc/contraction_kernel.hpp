@@ -30,6 +30,7 @@ namespace tracea_amd {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -563,7 +564,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // piece is fixed (row tid/CH + i*PR_STEP, 16-byte column tid%CH) and the
   // swizzle is applied to the GLOBAL column instead.  PR_STEP is a multiple of
   // RP*CH, hence the swizzle term is the same for all pieces of a thread.
-  static_assert(PIPE < 2 || (PR_STEP % (RP * CH) == 0 && !B_NCONTIG), "bad shape for direct-to-LDS loads");
+  static_assert(PIPE < 2 || PR_STEP % (RP * CH) == 0, "bad shape for direct-to-LDS loads");
   static_assert(PIPE == 3 ? NS >= 3 : NS == 2, "stage count does not fit the pipeline mode");
   const int gpc = PIPE >= 2 ? (pc ^ ((prow / RP) & (CH - 1))) : pc;
 
@@ -599,6 +600,13 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   }
   // N-contiguous B: piece q covers k row q / (BN/8), channels (q % (BN/8))*8..+7
   constexpr int NCH = BN / 8;
+
+  // B tile of the direct-to-LDS N-contiguous path: row pitch and pieces per k row.  One
+  // transposing read (below) takes 64 B from each of 4 consecutive k rows per half-wave; the
+  // 16-byte column is XORed with a function of the row so that those four land in the four
+  // different 64-byte bank groups.
+  constexpr int NB_ROWB = BN * 2, NB_CH = BN / 8;
+  auto nb_swz = [](int krow) -> int { return NB_ROWB >= 256 ? ((krow & 3) << 2) : (((krow >> 1) & 1) << 2); };
 
   u32x4 ra[NA], rb[NB];
 
@@ -691,8 +699,21 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
     for (int i = 0; i < NA; ++i)
       a_voff[i] = CONV ? (unsigned)(a_off[i] * 2) : (unsigned)((a_off[i] + gpc * 8) * 2);
+    if constexpr (!B_NCONTIG) {
 #pragma unroll
-    for (int i = 0; i < NB; ++i) b_voff[i] = (unsigned)((b_off[i] + gpc * 8) * 2);
+      for (int i = 0; i < NB; ++i) b_voff[i] = (unsigned)((b_off[i] + gpc * 8) * 2);
+    } else {
+      // N-contiguous B: the tile stays as it lies in memory, BK rows of BN channels.  Piece q
+      // of the tile (LDS byte 16q) is k row q / NB_CH, 16-byte column q % NB_CH, and holds
+      // the channels of global column (q % NB_CH) ^ nb_swz(row) (see nb_swz below).
+#pragma unroll
+      for (int i = 0; i < NB; ++i) {
+        const int q = tid + i * NT;
+        const int krow = q / NB_CH;
+        const int n = n0 + (((q % NB_CH) ^ nb_swz(krow)) << 3);
+        b_voff[i] = n < N ? (unsigned)(((long long)krow * args.ldb + n) * 2) : OOB;
+      }
+    }
   }
   // Only pieces lo <= index < hi of the thread's list (A pieces first, then B)
   // are requested, so that the requests of one tile can be spread over several
@@ -730,11 +751,45 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       if (NA + i < lo || NA + i >= hi) continue;
-      const unsigned voff = kvalid ? b_voff[i] : OOB;
       unsigned char *dst = sB + (i * PR_STEP + wave_u * RPI) * ROW_BYTES;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16,
-                                               (int)voff, k0 * 2, 0, 0);
+      if constexpr (!B_NCONTIG) {
+        const unsigned voff = kvalid ? b_voff[i] : OOB;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16,
+                                                 (int)voff, k0 * 2, 0, 0);
+      } else {
+        // rows at or beyond K must read as zero; the scalar offset takes no part in the
+        // hardware's range check, so the row is tested here
+        const unsigned voff = k0 + (tid + i * NT) / NB_CH < K ? b_voff[i] : OOB;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16,
+                                                 (int)voff, (int)((long long)k0 * args.ldb * 2), 0, 0);
+      }
     }
+  };
+
+  // Operand fetch from the [k][n] tile: ds_read_b64_tr_b16 hands lane i of a 16-lane group
+  // column i of a 4-row x 16-column block, i.e. 4 consecutive k of one channel; lane r of
+  // the group supplies the address of row r/4, columns 4*(r%4).  Lanes 0-31 take k 0-7 of
+  // the 16-wide k-step, lanes 32-63 k 8-15, in two reads of 4 rows each, which is the
+  // operand layout of the K-contiguous path.
+  int tr_off[B_NCONTIG && PIPE >= 2 ? FN : 1];
+  if constexpr (B_NCONTIG && PIPE >= 2) {
+    const int r = lane & 15;
+    const int row = (lane >> 5) * 8 + (r >> 2);
+#pragma unroll
+    for (int j = 0; j < FN; ++j) {
+      const int col = wn * TN + j * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
+      tr_off[j] = row * NB_ROWB + (((col >> 3) ^ nb_swz(row)) << 4) + (col & 7) * 2;
+    }
+  }
+  auto read_b_tr = [&](const unsigned char *sB, int j, int ks) -> u32x4 {
+    const unsigned char *p = sB + tr_off[j] + ks * 16 * NB_ROWB;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
+    const s16x4 hi =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p + 4 * NB_ROWB));
+    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 v;
+    v[0] = lo2[0]; v[1] = lo2[1]; v[2] = hi2[0]; v[3] = hi2[1];
+    return v;
   };
 
   auto lds_piece = [&](int row, int c) -> int {
@@ -918,7 +973,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // barrier.
     constexpr int KS = BK / 16;
     static_assert(KS >= 2 && KS % 2 == 0, "pipelined loop needs an even number of k-steps");
-    constexpr int R = FM * FN, D = FM + FN, L = NA + NB;
+    constexpr int R = FM * FN, D = FM + (B_NCONTIG ? 2 * FN : FN), L = NA + NB;
     u32x4 fa[2][FM], fb[2][FN];
     auto read_operands = [&](int set, const unsigned char *sA, const unsigned char *sB, int ks) {
       const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
@@ -927,7 +982,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
       for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
 #pragma unroll
-      for (int j = 0; j < FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+      for (int j = 0; j < FN; ++j) {
+        if constexpr (B_NCONTIG) fb[set][j] = read_b_tr(sB, j, ks);
+        else fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+      }
     };
     auto mma = [&](int set) {
 #pragma unroll
@@ -997,7 +1055,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // over the k-steps of the tile that overlaps them.
     constexpr int KS = BK / 16;
     static_assert(KS >= 2 && KS % 2 == 0, "pipelined loop needs an even number of k-steps");
-    constexpr int R = FM * FN, D = FM + FN, L = NA + NB;
+    constexpr int R = FM * FN, D = FM + (B_NCONTIG ? 2 * FN : FN), L = NA + NB;
     constexpr int LAST_SHARE = L - ((KS - 1) * L) / KS;          // pieces issued after the barrier
     constexpr int IN_FLIGHT = (NS - 3) * L + (L - LAST_SHARE);   // requests newer than tile t+1 at barrier t
     static_assert(IN_FLIGHT <= 63, "vmcnt is a 6-bit counter");
@@ -1013,7 +1071,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
       for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
 #pragma unroll
-      for (int j = 0; j < FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+      for (int j = 0; j < FN; ++j) {
+        if constexpr (B_NCONTIG) fb[set][j] = read_b_tr(sB, j, ks);
+        else fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+      }
     };
     auto mma = [&](int set) {
 #pragma unroll
@@ -1157,16 +1218,7 @@ int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_nc
     hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                    \
     return (int)hipGetLastError();                                                           \
   } while (0)
-  if constexpr (PIPE >= 2) {
-    // direct-to-LDS loads cannot transpose: K-contiguous B only (the dispatcher
-    // routes an N-contiguous B to the register-staged twin)
-    if (b_ncontig) return (int)hipErrorInvalidValue;
-    if (dtype == DT_F16) {
-      if (conv) TRACEA_LAUNCH(DT_F16, true, false); else TRACEA_LAUNCH(DT_F16, false, false);
-    } else {
-      if (conv) TRACEA_LAUNCH(DT_BF16, true, false); else TRACEA_LAUNCH(DT_BF16, false, false);
-    }
-  } else if (dtype == DT_F16) {
+  if (dtype == DT_F16) {
     if (conv) { if (b_ncontig) TRACEA_LAUNCH(DT_F16, true, true); else TRACEA_LAUNCH(DT_F16, true, false); }
     else      { if (b_ncontig) TRACEA_LAUNCH(DT_F16, false, true); else TRACEA_LAUNCH(DT_F16, false, false); }
   } else {

@@ -377,12 +377,13 @@ int twin(int vi, int pipeline) {
 }
 
 // Replaces a variant that cannot run the problem by the nearest one that can:
-// direct-to-LDS loads (pipeline 2) need a K-contiguous B; the register-staged
-// pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
-int resolve_variant(int vi, bool conv, bool b_ncontig, bool k_exact) {
+// direct-to-LDS loads (pipelines 2 and 3) address operands with 32-bit byte
+// offsets, so operands of 2 GiB and more go through registers (`staged`); the
+// register-staged pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
+int resolve_variant(int vi, bool conv, bool staged, bool k_exact) {
   int pipe = contraction_variant(vi).pipeline;
   if (pipe == 4) pipe = 2;  // a convolution-only kernel asked for a GEMM: same tile with streamed operands, if any
-  if (pipe >= 2 && b_ncontig) pipe = 1;
+  if (pipe >= 2 && staged) pipe = 1;
   if (pipe == 1 && !conv && !k_exact) pipe = 0;
   if (pipe == contraction_variant(vi).pipeline) return vi;
   for (int want = pipe; want >= 0; --want) {
@@ -435,7 +436,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       const long long a_extent = ((M - 1) * a.stride[0] + K) * 2;
       const long long b_extent = b_kcontig ? ((N - 1) * b.stride[1] + K) * 2 : ((K - 1) * b.stride[0] + N) * 2;
       const bool small = a_extent < (1ll << 31) && b_extent < (1ll << 31);
-      vi = resolve_variant(vi, false, !b_kcontig || !small, K % contraction_variant(vi).bk == 0);
+      vi = resolve_variant(vi, false, !small, K % contraction_variant(vi).bk == 0);
       const ContractionVariant &v = contraction_variant(vi);
       args.a_bytes = (unsigned)(small ? a_extent : 0);
       args.b_bytes = (unsigned)(small ? b_extent : 0);
@@ -707,7 +708,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
     vi = select_contraction_variant(a.M, a.N, a.K, true);
     if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
   }
-  vi = resolve_variant(vi, true, plan.w_ncontig || !small, true);
+  vi = resolve_variant(vi, true, !small, true);
   const ContractionVariant &v = contraction_variant(vi);
   a.a_bytes = (unsigned)(small ? x_extent : 0);
   a.b_bytes = (unsigned)(small ? w_extent : 0);
