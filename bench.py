@@ -6,7 +6,7 @@ fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
 FlashAttention-2 forward named by the metric are timed in the same run and
 reported under "also".  Prints one JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|conv|attention|attention_causal|conv_transpose|copy]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_rowmajor|conv|attention|attention_causal|conv_transpose|copy]
 """
 import argparse
 import json
@@ -22,7 +22,7 @@ PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
 # HBM-side bytes per launch of the dominant kernel of each workload, from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
 # (profiles/bench_kernels_mi355x.md); None where no counter run exists.
-TRAFFIC_BYTES = {"gemm": 235.2e6, "conv": 26.5e6, "attention": 537.1e6, "attention_causal": None, "conv_transpose": None, "copy": None}
+TRAFFIC_BYTES = {"gemm": 235.2e6, "conv": 26.5e6, "attention": 537.1e6, "attention_causal": None, "gemm_rowmajor": None, "conv_transpose": None, "copy": None}
 METRIC = "TFLOPS + % fp16 MFMA peak: GEMM 4096^3, 3x3 implicit-GEMM conv, FA2 fwd"
 
 
@@ -37,6 +37,14 @@ def make_workload(name, torch, ops):
         c = torch.empty(m, n, device=dev, dtype=torch.float16)
         b = bt.t()
         return ("fp16 GEMM 4096x4096x4096, A row-major, B column-major, fp32 acc, fp16 out",
+                2.0 * m * n * k, 2.0 * (m * k + k * n + m * n), "f16", lambda: ops.gemm(a, b, out=c))
+    if name == "gemm_rowmajor":
+        # the same product with B stored [K,N] row-major, the layout the reference's tracea_gemm documents
+        m = n = k = 4096
+        a = (torch.randn(m, k, device=dev, generator=g) / k ** 0.5).half()
+        b = (torch.randn(k, n, device=dev, generator=g) / k ** 0.5).half()
+        c = torch.empty(m, n, device=dev, dtype=torch.float16)
+        return ("fp16 GEMM 4096x4096x4096, A and B row-major, fp32 acc, fp16 out",
                 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n), "f16", lambda: ops.gemm(a, b, out=c))
     if name == "conv":
         n, h, w, cin, cout = 32, 56, 56, 64, 64
@@ -150,7 +158,7 @@ def main():
     }
     if not args.no_extras:
         also = {}
-        for name in ("gemm", "conv", "attention", "attention_causal", "conv_transpose"):
+        for name in ("gemm", "gemm_rowmajor", "conv", "attention", "attention_causal", "conv_transpose"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)

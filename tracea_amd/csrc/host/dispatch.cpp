@@ -886,11 +886,16 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
   // Filters already stored in the order the GEMM reads are used in place; any other order is
   // copied into it (C*R*S*K elements, next to the partial products in the temporary buffer).
   const long long R = w.shape[1], S = w.shape[2];
-  // (the fp32 GEMM kernel reads a row-major B: there the order is [C,R,S,K], the reference's own)
-  const bool c_inner = is_half(x.dtype);
-  const bool in_place = plan.fm.c_inner == c_inner && plan.fm.ld == (c_inner ? C : J) &&
-                        (K == 1 || plan.fm.col[0] == 1) && (S == 1 || plan.fm.col[2] == K) &&
-                        (R == 1 || plan.fm.col[1] == S * K);
+  // The gather kernel wants the columns ordered (r, s, k).  The half-precision GEMM kernels
+  // read either orientation of B at nearly the same speed, so [R,S,K,C] and [C,R,S,K] (the
+  // reference's own order) are both used in place; the fp32 kernel reads a row-major B only.
+  const bool cols_ok = (K == 1 || plan.fm.col[0] == 1) && (S == 1 || plan.fm.col[2] == K) &&
+                       (R == 1 || plan.fm.col[1] == S * K);
+  const bool half = is_half(x.dtype);
+  const bool in_place = cols_ok && (plan.fm.c_inner ? (half && plan.fm.ld == C)
+                                                    : (plan.fm.ld % 8 == 0 && aligned(w.ptr, 16)));
+  const bool c_inner = in_place ? plan.fm.c_inner : half;
+  const long long ldw = in_place ? plan.fm.ld : (c_inner ? C : J);
   const size_t cols_bytes = (size_t)(nb * per_image);
   const size_t cols_padded = (cols_bytes + 255) & ~(size_t)255;
   const size_t filt_bytes = in_place ? 0 : (size_t)(J * C) * elem_size(w.dtype);
@@ -918,8 +923,8 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
     a.stride[0] = plan.ldx; a.stride[1] = 1;
     b.ptr = (void *)filt;
     b.shape[0] = C; b.shape[1] = J;
-    if (c_inner) { b.stride[0] = 1; b.stride[1] = C; }
-    else { b.stride[0] = J; b.stride[1] = 1; }
+    if (c_inner) { b.stride[0] = 1; b.stride[1] = ldw; }
+    else { b.stride[0] = ldw; b.stride[1] = 1; }
     c.ptr = cols; c.dtype = TRACEA_DTYPE_FLOAT32; c.device = out.device;
     c.shape[0] = a.shape[0]; c.shape[1] = J;
     c.stride[0] = J; c.stride[1] = 1;
