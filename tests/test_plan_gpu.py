@@ -1,0 +1,201 @@
+"""Execution plans on the device: a fused ResNet block against the CPU oracle, the
+standalone node kernels against numpy, the reference's ResNet-18 benchmark graph
+(src/bin/network_bench.rs:41-215) end to end against torch in fp32, and HIP-graph
+replays of a plan against its eager run."""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import assert_close_scaled, round_f16, tol_for_k
+from test_graph_cpu import basic_block
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+
+def _bn_params(rng, ch):
+    return [rng.uniform(0.5, 1.5, ch).astype(np.float32), (rng.standard_normal(ch) * 0.1).astype(np.float32),
+            (rng.standard_normal(ch) * 0.1).astype(np.float32), rng.uniform(0.5, 1.5, ch).astype(np.float32)]
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_basic_block_plan_matches_the_oracle(tracea_gpu, fused):
+    from tracea_amd import graph as G, plan as P
+    n, ch, hw = 4, 64, 14
+    rng = np.random.default_rng(0x7ACEA020)
+    x = round_f16(rng.standard_normal((n, hw, hw, ch)))
+    w = {1: round_f16(rng.standard_normal((3, 3, ch, ch)) * np.sqrt(2.0 / (9 * ch))),
+         4: round_f16(rng.standard_normal((3, 3, ch, ch)) * np.sqrt(2.0 / (9 * ch)))}
+    bn = {20: _bn_params(rng, ch), 30: _bn_params(rng, ch)}
+
+    def bn_op(base):
+        return (oracle.EPI_BATCHNORM,) + tuple(bn[base]) + (1e-5,)
+
+    y1 = round_f16(oracle.epilogue_apply(oracle.conv2d_nhwc(x, w[1], 1, 1), [bn_op(20), (oracle.EPI_RELU,)]))
+    y2 = oracle.epilogue_apply(oracle.conv2d_nhwc(y1, w[4], 1, 1),
+                               [bn_op(30), (oracle.EPI_RESIDUAL_ADD, x.reshape(-1, ch)), (oracle.EPI_RELU,)])
+    graph = basic_block(n, ch, hw)
+    plan = P.Plan(G.fuse(graph) if fused else graph)
+    assert len(plan.describe()["steps"]) == (2 if fused else 7)
+    plan.bind(0, torch.from_numpy(x).cuda().half())
+    for base, params in bn.items():
+        for i, v in enumerate(params):
+            plan.bind(base + i, torch.from_numpy(v).cuda())
+    plan.bind(1, torch.from_numpy(w[1]).cuda().half(), "weight_rsck")
+    plan.bind(4, torch.from_numpy(w[4]).cuda().half().permute(3, 0, 1, 2).contiguous(), "weight")
+    plan.run()
+    last = plan.describe()["steps"][-1]["op_id"]
+    got = plan.output(last, (n, hw, hw, ch)).float().cpu().numpy()
+    # unfused, every node rounds its result to f16: one more rounding per node
+    assert_close_scaled(got, y2, (2 if fused else 3) * tol_for_k(9 * ch), "block output, fused=%s" % fused)
+
+
+def test_standalone_nodes_against_numpy(tracea_gpu):
+    from tracea_amd import graph as G, plan as P
+    n, c, h = 3, 40, 5
+    rng = np.random.default_rng(7)
+    x = round_f16(rng.standard_normal((n, h, h, c)))
+    g = {"operators": [G.input_node(1, "x"), G.relu_node(2, "relu", x.size), G.add_node(3, "add", x.size),
+                       G.global_avg_pool_node(4, "gap", n, c, h, h), G.softmax_node(5, "softmax"),
+                       G.linear_node(6, "fc", n, 1, 24, c), G.softmax_node(7, "probs")],
+         "dependencies": [[1, 2], [2, 3], [1, 3], [3, 4], [4, 5], [4, 6], [6, 7]]}
+    wt = round_f16(rng.standard_normal((c, 24)) * 0.2)
+    plan = P.Plan(g).bind(1, torch.from_numpy(x).cuda().half())
+    plan.bind(6, torch.from_numpy(wt).cuda().half(), "weight")
+    plan.run()
+    relu = np.maximum(x, 0)
+    add = round_f16(round_f16(relu) + x)
+    gap = round_f16(add.reshape(n, h * h, c).mean(axis=1))
+
+    def softmax(v):
+        e = np.exp(v - v.max(axis=-1, keepdims=True))
+        return e / e.sum(axis=-1, keepdims=True)
+
+    # intermediates give their bytes back after their last consumer; only results nobody reads
+    # (here the two softmax nodes) are still in the arena after the run
+    np.testing.assert_allclose(plan.output(5, (n, c)).float().cpu().numpy(), softmax(gap), atol=1e-3)
+    fc = round_f16(gap.astype(np.float64) @ wt.astype(np.float64))
+    probs = plan.output(7, (n, 24)).float().cpu().numpy()
+    np.testing.assert_allclose(probs, softmax(fc), atol=2e-3)
+    np.testing.assert_allclose(probs.sum(axis=1), 1.0, atol=2e-3)
+    # each kernel on its own, as the single result of a one-node plan
+    dx = torch.from_numpy(x).cuda().half()
+    one = P.Plan({"operators": [G.input_node(1, "x"), G.relu_node(2, "relu", x.size)], "dependencies": [[1, 2]]})
+    one.bind(1, dx).run()
+    np.testing.assert_array_equal(one.output(2, x.shape).float().cpu().numpy(), relu)
+    one = P.Plan({"operators": [G.input_node(1, "x"), G.input_node(2, "y"), G.add_node(3, "add", x.size)],
+                  "dependencies": [[1, 3], [2, 3]]})
+    one.bind(1, dx).bind(2, torch.from_numpy(relu).cuda().half()).run()
+    np.testing.assert_array_equal(one.output(3, x.shape).float().cpu().numpy(), round_f16(x + round_f16(relu)))
+    one = P.Plan({"operators": [G.input_node(1, "x"), G.global_avg_pool_node(4, "gap", n, c, h, h)],
+                  "dependencies": [[1, 4]]})
+    one.bind(1, dx).run()
+    np.testing.assert_allclose(one.output(4, (n, c)).float().cpu().numpy(), x.reshape(n, h * h, c).mean(axis=1),
+                               atol=1e-3)
+    params = _bn_params(rng, c)
+    bn_graph = {"operators": [G.input_node(1, "x")] + [G.input_node(10 + i, "p%d" % i) for i in range(4)] +
+                             [G.batchnorm_node(2, "bn", n, c, h, h)],
+                "dependencies": [[1, 2], [10, 2], [11, 2], [12, 2], [13, 2]]}
+    one = P.Plan(bn_graph).bind(1, dx)
+    for i, v in enumerate(params):
+        one.bind(10 + i, torch.from_numpy(v).cuda())
+    one.run()
+    want = oracle.epilogue_apply(x.reshape(-1, c), [(oracle.EPI_BATCHNORM,) + tuple(params) + (1e-5,)])
+    np.testing.assert_allclose(one.output(2, (n * h * h, c)).float().cpu().numpy(), want, atol=4e-3)
+
+
+def _resnet18(batch, seed):
+    """Plan, bound tensors and a torch fp32 model of the same network."""
+    from tracea_amd import graph as G, plan as P
+    graph, info = G.resnet18_graph(batch)
+    fused = G.fuse(graph)
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    plan = P.Plan(fused)
+    image = torch.zeros(batch, 224, 224, 8, device="cuda", dtype=torch.float16)
+    image[..., :3] = torch.randn(batch, 224, 224, 3, device="cuda", generator=gen).half()
+    plan.bind(info["input"], image)
+    weights, bns = {}, {}
+    for oid, (k, r, s, c) in info["convs"].items():
+        w = (torch.randn(k, r, s, c, device="cuda", generator=gen) * (2.0 / (r * s * c)) ** 0.5).half()
+        if c == 8:
+            w[..., 3:] = 0
+        weights[oid] = w
+        plan.bind(oid, w, "weight")
+    for oid, (params, c) in info["bn"].items():
+        vals = [torch.rand(c, device="cuda", generator=gen) * 0.5 + 0.75, torch.randn(c, device="cuda", generator=gen) * 0.1,
+                torch.randn(c, device="cuda", generator=gen) * 0.1, torch.rand(c, device="cuda", generator=gen) * 0.5 + 0.75]
+        bns[oid] = vals
+        for pid, v in zip(params, vals):
+            plan.bind(pid, v)
+    fc = (torch.randn(512, 1000, device="cuda", generator=gen) * 512 ** -0.5).half()
+    plan.bind(info["fc"], fc, "weight")
+
+    def reference():
+        # the unfused graph, node by node, in fp32 (NCHW for torch's convolution)
+        F = torch.nn.functional
+        vals = {info["input"]: image.float().permute(0, 3, 1, 2)}
+        prod = {}
+        for src, dst in graph["dependencies"]:
+            prod.setdefault(dst, []).append(src)
+        for node in graph["operators"]:
+            (kind, body), = node.items()
+            oid = body["op_id"]
+            if kind == "Input":
+                continue
+            ins = prod[oid]
+            if kind == "Conv2d":
+                vals[oid] = F.conv2d(vals[ins[0]], weights[oid].float().permute(0, 3, 1, 2), stride=body["stride"],
+                                     padding=body["padding"])
+            elif kind == "BatchNorm":
+                g_, b_, m_, v_ = bns[oid]
+                vals[oid] = F.batch_norm(vals[ins[0]], m_, v_, g_, b_, False, 0.0, body["epsilon"])
+            elif kind == "Relu":
+                vals[oid] = torch.relu(vals[ins[0]])
+            elif kind == "Elementwise":
+                vals[oid] = vals[ins[0]] + vals[ins[1]]
+            elif kind == "GlobalAveragePool":
+                vals[oid] = vals[ins[0]].mean(dim=(2, 3))
+            elif kind == "Linear":
+                vals[oid] = vals[ins[0]] @ fc.float()
+        return vals[info["output"]]
+
+    return plan, info, reference
+
+
+def test_resnet18_end_to_end_against_torch_fp32(tracea_gpu):
+    plan, info, reference = _resnet18(batch=2, seed=11)
+    want = reference()
+    plan.run()
+    got = plan.output(info["output"], (2, 1000)).float()
+    scale = float(want.abs().max())
+    assert scale > 0.1
+    # 20 half-precision layers deep: errors relative to the size of the logits
+    assert float((got - want).abs().max()) <= 3e-2 * scale
+    assert torch.equal(got.argmax(dim=1), want.argmax(dim=1))
+
+
+def test_hip_graph_replays_equal_the_eager_run(tracea_gpu):
+    plan, info, _ = _resnet18(batch=1, seed=12)
+    plan.run()
+    torch.cuda.synchronize()
+    eager = plan.output(info["output"], (1, 1000)).clone()
+    plan.capture()
+    scratch = torch.zeros(1 << 20, device="cuda")
+    for i in range(4):
+        plan.output(info["output"]).zero_()          # a replay must write the result again
+        scratch.add_(1.0)                            # eager work and a synchronisation between replays
+        torch.cuda.synchronize()
+        plan.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(plan.output(info["output"], (1, 1000)), eager), "replay %d" % i
+    assert float(scratch[0]) == 4.0
+
+
+def test_unbound_inputs_are_reported_before_any_launch(tracea_gpu):
+    from tracea_amd import graph as G, plan as P
+    plan = P.Plan(G.fuse(basic_block(1, 16, 8)))
+    with pytest.raises(RuntimeError, match="is not bound"):
+        plan.run()
+    plan.bind(0, torch.zeros(1, 8, 8, 16, device="cuda", dtype=torch.float16))
+    with pytest.raises(RuntimeError, match="not bound|no weight bound"):
+        plan.run()

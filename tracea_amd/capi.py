@@ -97,6 +97,13 @@ SIGNATURES = {
                                    C.POINTER(EpilogueOp), C.c_uint32]),
     "tracea_gemm_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), GemmParams,
                                  C.POINTER(EpilogueOp), C.c_uint32]),
+    "tracea_plan_compile": (C.c_void_p, [C.c_char_p, C.c_int]),
+    "tracea_plan_destroy": (None, [C.c_void_p]),
+    "tracea_plan_arena_size": (C.c_size_t, [C.c_void_p]),
+    "tracea_plan_describe": (C.c_void_p, [C.c_void_p]),
+    "tracea_plan_output": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "tracea_plan_bind": (C.c_int, [C.c_void_p, C.c_uint64, C.c_char_p, C.c_void_p]),
+    "tracea_plan_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "tracea_variant_count": (C.c_int32, [C.c_char_p]),
     "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),
     "tracea_force_variant": (C.c_int32, [C.c_char_p, C.c_int32]),

@@ -125,6 +125,25 @@ struct FilterRepackArgs {
 };
 int launch_filter_repack(const FilterRepackArgs &args, hipStream_t stream);
 
+// Operators of a graph that were not merged into a contraction (standalone ReLU,
+// BatchNorm, Add: src/policy/types.rs:60-84) run as an operator chain over an
+// existing tensor: out[m, n] = chain(x[m, n]), rows of `channels` elements.
+struct ChainApplyArgs {
+  const void *x;
+  void *out;
+  int x_dtype, out_dtype;
+  long long rows;
+  int channels;
+  EpilogueChain epi;
+};
+int launch_chain_apply(const ChainApplyArgs &args, hipStream_t stream);
+// out[b, c] = mean over hw of x[b, hw, c] (NHWC), fp32 sums.
+int launch_global_avg_pool(const void *x, void *out, int dtype, int out_dtype, int batch, int hw, int channels,
+                           hipStream_t stream);
+// Row-wise softmax over the last axis, fp32 arithmetic.
+int launch_softmax_rows(const void *x, void *out, int dtype, int out_dtype, long long rows, int cols,
+                        hipStream_t stream);
+
 struct AttentionVariant {
   const char *name;
   int block_q, block_kv, waves;

@@ -168,6 +168,29 @@ bool fuse_graph(Json *graph, std::string *err) {
     current.swap(next);
   }
 
+  // A skip tensor named by a ResidualAdd entry may itself have been merged away in a later
+  // sweep (in a chain of residual blocks, the ReLU that ends block i is the skip input of
+  // block i+1 and is absorbed by block i's last convolution one sweep after block i+1
+  // recorded it).  The reference leaves the stale id in place (src/core/optimizer.rs:139-147
+  // resolves only at the time of the merge); an id that names no node cannot be executed,
+  // so it is resolved here to the node that now produces that tensor.
+  for (Node &n : current) {
+    if (removed.count(n.id)) continue;
+    Json *epi = nullptr;
+    for (auto &kv : n.body.obj)
+      if (kv.first == "epilogue") epi = &kv.second;
+    if (epi == nullptr || epi->type != Json::Array) continue;
+    for (Json &e : epi->arr) {
+      if (e.type != Json::Object || e.obj.size() != 1 || e.obj[0].first != "ResidualAdd") continue;
+      for (auto &f : e.obj[0].second.obj)
+        if (f.first == "residual_ptr" && f.second.type == Json::Number) {
+          Id skip = (Id)f.second.num;
+          for (auto it = fused_into.find(skip); it != fused_into.end(); it = fused_into.find(skip)) skip = it->second;
+          f.second = Json::make_num((double)skip);
+        }
+    }
+  }
+
   Json ops_out = Json::make_arr();
   for (const Node &n : current) {
     if (removed.count(n.id)) continue;

@@ -113,3 +113,93 @@ def execute(graph, tensors, weights):
         if not progressed:
             raise ValueError("graph has a cycle or an input without a tensor")
     return tensors
+
+
+def global_avg_pool_node(op_id, name, n, c, h, w):
+    return {"GlobalAveragePool": dict(op_id=op_id, name=name, n=n, c=c, h=h, w=w)}
+
+
+def linear_node(op_id, name, batch, m, n, k):
+    return {"Linear": dict(op_id=op_id, name=name, batch=batch, m=m, n=n, k=k, epilogue=[])}
+
+
+def softmax_node(op_id, name, axis=-1):
+    return {"Softmax": dict(op_id=op_id, name=name, axis=axis)}
+
+
+def resnet18_graph(batch=1, in_channels=8, classes=1000):
+    """The ResNet-18 graph of the reference's network benchmark (src/bin/network_bench.rs:41-215):
+    7x7 stride-4 stem on 224x224 (no max-pool), four stages of two basic blocks (64/128/256/512
+    filters, the first block of stages 2-4 at stride 2 with a 1x1 shortcut), global average pool,
+    1000-way linear layer.  Two differences, both needed to run it on the matrix-core kernels:
+    every BatchNorm carries its four parameter vectors as Input nodes, so that the fusion rules
+    merge it (the reference's benchmark graph leaves them out and its BatchNorms stay
+    standalone), and the image has 8 channels (3 used, 5 zero) because the convolution reads
+    16-byte channel groups.
+
+    Returns (graph, info): info["convs"] maps op_id -> (k, r, s, c), info["bn"] maps the op_id of
+    every BatchNorm to its 4 parameter Input ids and channel count, info["input"] / ["fc"] /
+    ["output"] name the image Input, the Linear node and the last node."""
+    ops, deps = [], []
+    info = {"convs": {}, "bn": {}}
+    counter = [0]
+
+    def new_id():
+        counter[0] += 1
+        return counter[0]
+
+    def add(node, *producers):
+        oid = _kind(node)[1]["op_id"]
+        ops.append(node)
+        for p in producers:
+            deps.append([p, oid])
+        return oid
+
+    def conv(name, src, c, h, k, r, stride, pad):
+        oid = new_id()
+        info["convs"][oid] = (k, r, r, c)
+        return add(conv2d_node(oid, name, batch, c, h, h, k, r, r, stride, pad), src)
+
+    def bn(name, src, c, h):
+        oid = new_id()
+        params = []
+        for p in ("gamma", "beta", "mean", "var"):
+            pid = new_id()
+            ops.append(input_node(pid, "%s_%s" % (name, p)))
+            params.append(pid)
+        info["bn"][oid] = (params, c)
+        return add(batchnorm_node(oid, name, batch, c, h, h), src, *params)
+
+    def relu(name, src, c, h):
+        return add(relu_node(new_id(), name, batch * c * h * h), src)
+
+    image = new_id()
+    ops.append(input_node(image, "input"))
+    info["input"] = image
+    cur = conv("stem_conv", image, in_channels, 224, 64, 7, 4, 3)
+    cur = bn("stem_bn", cur, 64, 56)
+    cur = relu("stem_relu", cur, 64, 56)
+    size = 56
+    for in_c, out_c, stride in ((64, 64, 1), (64, 128, 2), (128, 256, 2), (256, 512, 2)):
+        block_in = in_c
+        for i in range(2):
+            s = stride if i == 0 else 1
+            out_size = (size + 2 - 3) // s + 1
+            shortcut = cur
+            tag = "layer_%d_block_%d" % (out_c, i)
+            cur = conv(tag + "_conv1", cur, block_in, size, out_c, 3, s, 1)
+            cur = bn(tag + "_bn1", cur, out_c, out_size)
+            cur = relu(tag + "_relu1", cur, out_c, out_size)
+            cur = conv(tag + "_conv2", cur, out_c, out_size, out_c, 3, 1, 1)
+            main = bn(tag + "_bn2", cur, out_c, out_size)
+            if block_in != out_c or s != 1:
+                sc = conv(tag + "_shortcut_conv", shortcut, block_in, size, out_c, 1, s, 0)
+                shortcut = bn(tag + "_shortcut_bn", sc, out_c, out_size)
+            cur = add(add_node(new_id(), tag + "_add", batch * out_c * out_size * out_size), main, shortcut)
+            cur = relu(tag + "_relu2", cur, out_c, out_size)
+            block_in, size = out_c, out_size
+    cur = add(global_avg_pool_node(new_id(), "avgpool", batch, 512, size, size), cur)
+    fc = add(linear_node(new_id(), "fc", batch, 1, classes, 512), cur)
+    info["fc"] = fc
+    info["output"] = fc
+    return {"operators": ops, "dependencies": deps}, info
