@@ -104,6 +104,8 @@ SIGNATURES = {
     "tracea_plan_output": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "tracea_plan_bind": (C.c_int, [C.c_void_p, C.c_uint64, C.c_char_p, C.c_void_p]),
     "tracea_plan_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "tracea_set_split_k": (None, [C.c_int32]),
+    "tracea_last_split_k": (C.c_int32, []),
     "tracea_variant_count": (C.c_int32, [C.c_char_p]),
     "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),
     "tracea_force_variant": (C.c_int32, [C.c_char_p, C.c_int32]),

@@ -125,6 +125,9 @@ TraceaStatus tracea_attention(TraceaTensorView q, TraceaTensorView k, TraceaTens
   TRACEA_GUARDED(dispatch_attention(q, k, v, o, params))
 }
 
+void tracea_set_split_k(int32_t enabled) { set_split_k_enabled(enabled != 0); }
+int32_t tracea_last_split_k(void) { return last_split_k(); }
+
 int32_t tracea_variant_count(const char *op) {
   if (op == nullptr) return -1;
   if (!strcmp(op, "gemm") || !strcmp(op, "conv2d")) return contraction_variant_count();

@@ -38,6 +38,8 @@ struct ContractionArgs {
   int out_dtype;       // DataType of C
   unsigned a_bytes, b_bytes;  // extent of A and B in bytes (bounds of the direct-to-LDS buffer loads)
   int grid_m, grid_n;  // tiles along M and N
+  int k_split;         // 0: one workgroup per tile runs all of K; else the K extent of one split (a multiple
+                       // of the variant's BK): grid.y = ceil(K / k_split), C is the [splits][M][ldc] workspace
   int group_m;         // tile-order group height
   // convolution geometry (ConvParams of the reference, h/w split)
   int h_in, w_in, c_in, h_out, w_out, s_sz;
@@ -93,6 +95,17 @@ struct GenericGemmArgs {
   EpilogueChain epi;
 };
 int launch_gemm_generic(const GenericGemmArgs &args, hipStream_t stream);
+
+// Second stage of a split-K contraction: out[m, n] = chain(sum over z of partial[z][m][n]).
+struct SplitKReduceArgs {
+  const float *partial;  // [splits][M][N] fp32
+  void *out;
+  int out_dtype;
+  int splits, M, N;
+  long long ldc;
+  EpilogueChain epi;
+};
+int launch_splitk_reduce(const SplitKReduceArgs &args, hipStream_t stream);
 
 // Second stage of the transposed convolution: gathers the per-tap partial
 // products `cols` (one row per input pixel, one column per (r, s, k)) into the

@@ -553,7 +553,13 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   int tile_m, tile_n;
   tile_coordinates(args, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int M = args.M, N = args.N, K = args.K;
+  const int M = args.M, N = args.N;
+  // Split-K: workgroups with blockIdx.y = z multiply the K range [z*k_split, (z+1)*k_split)
+  // and write their fp32 partial product to rows z*M.. of C, which is then a workspace that
+  // a reduction kernel sums.  kb is added to every K offset below; K is the end of the range.
+  const int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
+  const int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
+  const long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
 
   // ---- per-thread source coordinates of the pieces this thread moves ----
   const int pc = tid % CH;      // 16-byte column of every A piece of this thread
@@ -640,6 +646,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   unsigned a_ok = 0, b_ok = 0;  // bit i: piece i holds real data
   auto fetch = [&](int k0) {
+    k0 += kb;
     const int kg = k0 + gpc * 8;
     const bool kvalid = kg < K;
     const int k0c = kvalid ? kg : 0;  // column of this thread's piece, or a safe one
@@ -720,6 +727,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // k-steps.
   auto dma = [&](unsigned char *sA, unsigned char *sB, int k0, int lo, int hi) {
     constexpr int RPI = 64 / CH;  // tile rows one wave instruction covers
+    k0 += kb;
     const int kg = k0 + gpc * 8;
     const bool kvalid = kg < K;
     int dh = 0, dw = 0, ci = 0;
@@ -802,7 +810,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // there the decision is made at compile time: always for a convolution, never
   // for a GEMM, and the dispatcher only picks a pipelined GEMM variant when K is
   // a multiple of BK.
-  const bool mask_rt = (K % BK) != 0;
+  const bool mask_rt = ((K - kb) % BK) != 0;
   auto stash = [&](unsigned char *sA, unsigned char *sB) {
     const bool mask_a = PIPE != 0 ? CONV : (CONV || mask_rt);
     const bool mask_b = PIPE != 0 ? CONV : (CONV || mask_rt);
@@ -871,7 +879,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 
   // ---- main loop: two LDS stages ----
   static_assert(NA <= 32 && NB <= 32, "piece masks are 32 bits");
-  const int nk = (K + BK - 1) / BK;
+  const int nk = (K - kb + BK - 1) / BK;
   if constexpr (PIPE < 2) {
     fetch(0);
     stash(smem, smem + A_STAGE);
@@ -1169,7 +1177,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     __builtin_amdgcn_wave_barrier();
     if (simple) {
       const int mb = m0 + wm * TM + i * 32;
-      auto row_of = [&](int r) -> long long { return mb + r < M ? (long long)(mb + r) : -1ll; };
+      auto row_of = [&](int r) -> long long { return mb + r < M ? zrow + (mb + r) : -1ll; };
       if constexpr (F32_SIMPLE) {
         if (out_f32) simple_rows<DT, TN, true>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
         else simple_rows<DT, TN, false>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
@@ -1190,8 +1198,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
             v[4 + e] = hi[e];
           }
           const int nvalid = N - n;
-          apply_epilogue_tab(v, m, n, nvalid, args.epi, plan, tab, BN);
-          store_from_float<8>(args.C, args.out_dtype, (long long)m * args.ldc + n, nvalid, v);
+          apply_epilogue_tab(v, zrow + m, n, nvalid, args.epi, plan, tab, BN);
+          store_from_float<8>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, nvalid, v);
         }
       }
     }
@@ -1204,7 +1212,8 @@ template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE>
 int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
                        hipStream_t stream) {
   constexpr size_t lds = (size_t)NS * (BM + BN) * BK * 2;
-  const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(WM * WN * 64);
+  const dim3 grid((unsigned)(a.grid_m * a.grid_n), (unsigned)(a.k_split > 0 ? (a.K + a.k_split - 1) / a.k_split : 1)),
+      block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \
     auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, NS, PIPE, CONVV, NCV>;                      \

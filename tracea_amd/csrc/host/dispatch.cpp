@@ -10,6 +10,7 @@
 #include <atomic>
 #include <cmath>
 #include <cstring>
+#include <map>
 #include <mutex>
 
 #include "tuning_cache.hpp"
@@ -238,9 +239,11 @@ TraceaStatus check_bias_residual(const char *what, const TraceaTensorView *bias,
 std::atomic<int> g_forced_contraction{-1};
 std::atomic<int> g_forced_conv{-1};
 std::atomic<int> g_forced_attention{-1};
+std::atomic<bool> g_split_k_enabled{true};
 // variant the calling thread's latest launch of each operator used (-1: none,
 // or a kernel outside the variant tables)
 thread_local int t_last_contraction = -1, t_last_conv = -1, t_last_attention = -1;
+thread_local int t_last_splits = 1;  // K ranges of the calling thread's latest gemm / conv2d launch
 
 TraceaStatus hip_status(const char *what, int e) {
   if (e == 0) return TRACEA_SUCCESS;
@@ -248,6 +251,9 @@ TraceaStatus hip_status(const char *what, int e) {
 }
 
 }  // namespace
+
+void set_split_k_enabled(bool on) { g_split_k_enabled.store(on); }
+int last_split_k() { return t_last_splits; }
 
 void set_forced_variant(const char *op, int index) {
   if (!strcmp(op, "gemm")) g_forced_contraction.store(index);
@@ -405,6 +411,86 @@ void fill_grid(ContractionArgs *a, const ContractionVariant &v) {
   if (a->group_m > a->grid_m) a->group_m = a->grid_m;
 }
 
+// ---- split-K ---------------------------------------------------------------------
+// A problem with few output tiles and a long K leaves most of the 256 CUs idle while a
+// handful of workgroups walk K serially (a 3x3 convolution on a 7x7 image with 512
+// channels: 8 tiles, 72 K tiles each).  Such a launch is split along K over blockIdx.y;
+// the fp32 partial products go to a scratch buffer and a second kernel sums them and runs
+// the operator chain.  The scratch buffer is kept per (device, stream), grows on demand up
+// to 64 MiB and is never allocated while the stream is being captured into a graph.
+constexpr size_t kSplitScratchCap = 64u << 20;
+std::mutex g_scratch_mu;
+std::map<std::pair<int, void *>, std::pair<void *, size_t>> g_scratch;
+
+void *splitk_scratch(int device, hipStream_t stream, size_t bytes) {
+  if (bytes > kSplitScratchCap) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  auto &slot = g_scratch[{device, (void *)stream}];
+  if (slot.second >= bytes) return slot.first;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (slot.first != nullptr) {
+    // launches queued on this stream may still write the old buffer
+    if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
+    (void)hipFree(slot.first);
+    slot = {nullptr, 0};
+  }
+  size_t want = 1u << 20;
+  while (want < bytes) want <<= 1;
+  void *p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  slot = {p, want};
+  return p;
+}
+
+// Number of K ranges for a launch of variant v (1: no split) and the extent of one range.
+int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split) {
+  const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+  const int nk = (K + v.bk - 1) / v.bk;
+  if (v.pipeline == 4 || tiles * 2 > 256 || nk < 8) return 1;
+  long long splits = 256 / tiles;
+  if (splits > nk / 4) splits = nk / 4;  // at least 4 K tiles per range
+  if (splits < 2) return 1;
+  const int per = (int)((nk + splits - 1) / splits);
+  *k_split = per * v.bk;
+  return (nk + per - 1) / per;
+}
+
+// Launches `args` on variant v, split along K when that pays; `chain` is the operator chain
+// of the call (args.epi is ignored).
+TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, ContractionArgs args,
+                                const EpilogueChain &chain, bool conv, int dtype, bool b_ncontig, int device,
+                                hipStream_t stream) {
+  int k_split = 0;
+  const int splits = g_split_k_enabled.load() ? choose_split(v, args.M, args.N, args.K, &k_split) : 1;
+  void *scratch = splits > 1 ? splitk_scratch(device, stream, (size_t)splits * args.M * args.N * 4) : nullptr;
+  t_last_splits = scratch != nullptr ? splits : 1;
+  if (scratch == nullptr) {
+    args.epi = chain;
+    args.k_split = 0;
+    return hip_status(what, v.launch(args, conv, dtype, b_ncontig, stream));
+  }
+  SplitKReduceArgs r{};
+  r.partial = (const float *)scratch;
+  r.out = args.C; r.out_dtype = args.out_dtype;
+  r.splits = splits; r.M = args.M; r.N = args.N; r.ldc = args.ldc;
+  r.epi = chain;
+  args.C = scratch;
+  args.ldc = args.N;
+  args.out_dtype = DT_F32;
+  args.epi = EpilogueChain{};
+  args.k_split = k_split;
+  TraceaStatus st = hip_status(what, v.launch(args, conv, dtype, b_ncontig, stream));
+  if (st != TRACEA_SUCCESS) return st;
+  return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
+}
+
 // ---- GEMM ----------------------------------------------------------------------
 TraceaStatus run_gemm(const View &a, const View &b, const View &c, const EpilogueChain &chain,
                       hipStream_t stream) {
@@ -442,7 +528,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.b_bytes = (unsigned)(small ? b_extent : 0);
       fill_grid(&args, v);
       t_last_contraction = vi;
-      return hip_status("gemm launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
+      return launch_maybe_split("gemm launch", v, args, chain, false, a.dtype, !b_kcontig, c.device, stream);
     }
   }
   if (a.dtype == TRACEA_DTYPE_FLOAT32 && b.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32 && K > 0 &&
@@ -680,10 +766,12 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // several full tiles (N32 56x56x64 -> 64, 3x3: 21.9 us against 23.1 us); with
   // 128 filters, stride 2 or 14x14 images the streamed 128x64 tiles are faster.
   // One shape is thin evidence: a tuning-cache entry or a forced variant wins
-  // over this rule, and tracea_autotune_conv2d measures every variant.
+  // over this rule, and tracea_autotune_conv2d measures every variant.  Below 256
+  // tiles of 256 pixels the kernel cannot fill the device (it has no split along
+  // K): a single 56x56 image is 13 workgroups.
   if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && a.N <= 64 &&
       g.stride_h == 1 && g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 &&
-      (long long)g.block.h_out * g.block.w_out >= 4 * 256) {
+      (long long)g.block.h_out * g.block.w_out >= 4 * 256 && (long long)a.M >= 256ll * 256) {
     for (int i = 0; i < contraction_variant_count(); ++i) {
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline == 4 && cv.bm == 256 && cv.bn == 64) {
@@ -714,7 +802,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   a.b_bytes = (unsigned)(small ? w_extent : 0);
   fill_grid(&a, v);
   t_last_conv = vi;
-  return hip_status("conv2d launch", v.launch(a, true, plan.x.dtype, plan.w_ncontig, stream));
+  return launch_maybe_split("conv2d launch", v, a, chain, true, plan.x.dtype, plan.w_ncontig, plan.out.device, stream);
 }
 
 }  // namespace

@@ -33,6 +33,10 @@ void set_forced_variant(const char *op, int index);
 int forced_variant(const char *op);
 // Variant index the calling thread's latest launch of `op` used, -1 if none.
 int last_variant(const char *op);
+// Split-K of launches with few output tiles and a long K (on by default), and the number of
+// K ranges the calling thread's latest gemm / conv2d launch was split into (1: not split).
+void set_split_k_enabled(bool on);
+int last_split_k();
 
 TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorView &b,
                                 const TraceaTensorView *bias, const TraceaTensorView *residual,

@@ -154,6 +154,67 @@ int launch_gemm_generic(const GenericGemmArgs &a, hipStream_t stream) {
 }
 
 // ---------------------------------------------------------------------------
+// Split-K reduction: sums the fp32 partial products of the K ranges, applies the
+// operator chain and stores.  One thread per row and 4 channels (1 when N % 4).
+// ---------------------------------------------------------------------------
+template <int V>
+__global__ void __launch_bounds__(256) splitk_reduce_kernel(const SplitKReduceArgs a) {
+  const int groups = (a.N + V - 1) / V;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)a.M * groups) return;
+  const long long m = idx / groups;
+  const int n = (int)(idx % groups) * V;
+  const int nvalid = a.N - n;
+  float v[V];
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = 0.0f;
+  const float *p = a.partial + m * a.N + n;
+  const long long plane = (long long)a.M * a.N;
+  // eight planes at a time, loads first: with a few thousand threads and a serial chain of
+  // loads per thread the kernel would be bound by memory latency times the split count
+  int z = 0;
+  for (; z + 8 <= a.splits; z += 8) {
+    if constexpr (V == 4) {
+      f32x4 t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) t[u] = *(const f32x4 *)(p + (z + u) * plane);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += t[u][e];
+    } else {
+      float t[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) t[u] = p[(z + u) * plane];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[0] += t[u];
+    }
+  }
+  for (; z < a.splits; ++z) {
+    if constexpr (V == 4) {
+      const f32x4 t = *(const f32x4 *)(p + z * plane);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] += t[e];
+    } else {
+      v[0] += p[z * plane];
+    }
+  }
+  apply_epilogue<V>(v, m, n, nvalid, a.epi);
+  store_from_float<V>(a.out, a.out_dtype, m * a.ldc + n, nvalid, v);
+}
+
+int launch_splitk_reduce(const SplitKReduceArgs &a, hipStream_t stream) {
+  const bool vec = a.N % 4 == 0 && (((uintptr_t)a.partial) & 15) == 0;
+  const long long groups = vec ? a.N / 4 : a.N;
+  const long long blocks = ((long long)a.M * groups + 255) / 256;
+  if (blocks <= 0) return 0;
+  if (blocks >= (1ll << 31)) return (int)hipErrorInvalidValue;
+  if (vec) hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
 // Coordinate tables of the convolution, computed on the device with the same
 // fast_divmod the contraction kernel uses, for bit-exact comparison with the
 // CPU statement of src/emitter/cuda/conv.rs:176-191, 208-210.

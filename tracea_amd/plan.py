@@ -34,7 +34,10 @@ class Plan:
     def __del__(self):
         h, self._h = getattr(self, "_h", None), None
         if h:
-            capi.lib().tracea_plan_destroy(h)
+            try:
+                capi.lib().tracea_plan_destroy(h)
+            except Exception:  # interpreter shutdown: the module globals are already gone
+                pass
 
     @property
     def arena_size(self):
@@ -78,10 +81,16 @@ class Plan:
     def capture(self):
         """Records one run into a HIP graph; ``replay()`` then re-issues it.  Everything a run
         touches (arena, bound tensors) must stay where it is."""
-        self.run()                      # first-use work (function attributes) outside the capture
+        # First-use work happens outside the capture and on the capture's own stream: kernel
+        # attributes, and the split-K scratch buffer, which the library keeps per stream and
+        # never allocates while a stream is being captured.
+        side = torch.cuda.Stream(self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            self.run()
         torch.cuda.synchronize(self.device)
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with torch.cuda.graph(g, stream=side):
             self.run()
         self._graph = g
         return self
