@@ -6,7 +6,7 @@ fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
 FlashAttention-2 forward named by the metric are timed in the same run and
 reported under "also".  Prints one JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_rowmajor|conv|attention|attention_causal|conv_transpose|copy]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_rowmajor|conv|attention|attention_causal|conv_transpose|resnet18_b1|resnet18_b32|copy]
 """
 import argparse
 import json
@@ -74,6 +74,35 @@ def make_workload(name, torch, ops):
         return ("fp16 NHWC transposed conv N8 32x32x512->64x64x256 4x4 s2 p1",
                 2.0 * n * h * w * cin * r * r * cout, 2.0 * (x.numel() + wt.numel() + y.numel()), "f16",
                 lambda: ops.conv_transpose2d(x, wt, stride=st, padding=pd, out=y))
+    if name in ("resnet18_b1", "resnet18_b32"):
+        # the reference's network benchmark graph (src/bin/network_bench.rs:41-215), fused, compiled into
+        # an execution plan and replayed as one HIP graph; random weights, BatchNorm parameters near identity
+        from tracea_amd import graph as G, plan as P
+        batch = 1 if name.endswith("b1") else 32
+        graph, info = G.resnet18_graph(batch)
+        plan = P.Plan(G.fuse(graph))
+        image = torch.zeros(batch, 224, 224, 8, device=dev, dtype=torch.float16)
+        image[..., :3] = torch.randn(batch, 224, 224, 3, device=dev, generator=g).half()
+        plan.bind(info["input"], image)
+        flops = 0.0
+        for node in graph["operators"]:
+            (kind, body), = node.items()
+            if kind == "Conv2d":
+                ho = (body["h"] + 2 * body["padding"] - body["r"]) // body["stride"] + 1
+                flops += 2.0 * body["n"] * ho * ho * body["k"] * body["r"] * body["s"] * (3 if body["c"] == 8 else body["c"])
+        flops += 2.0 * batch * 512 * 1000
+        for oid, (k, r, s_, c) in info["convs"].items():
+            w = (torch.randn(k, r, s_, c, device=dev, generator=g) * (2.0 / (r * s_ * c)) ** 0.5).half()
+            plan.bind(oid, w, "weight")
+        for oid, (params, c) in info["bn"].items():
+            vals = [torch.rand(c, device=dev, generator=g) * 0.5 + 0.75, torch.randn(c, device=dev, generator=g) * 0.1,
+                    torch.randn(c, device=dev, generator=g) * 0.1, torch.rand(c, device=dev, generator=g) * 0.5 + 0.75]
+            for pid, v in zip(params, vals):
+                plan.bind(pid, v)
+        plan.bind(info["fc"], (torch.randn(512, 1000, device=dev, generator=g) * 512 ** -0.5).half(), "weight")
+        plan.capture()
+        return ("fp16 ResNet-18 forward, batch %d, 224x224, %d fused launches replayed as one HIP graph"
+                % (batch, len(plan.describe()["steps"])), flops, 0.0, "f16", plan.replay)
     if name == "copy":
         # calibration workload for the HBM traffic counters: a plain device copy of known size
         n = 256 << 20
@@ -158,7 +187,8 @@ def main():
     }
     if not args.no_extras:
         also = {}
-        for name in ("gemm", "gemm_rowmajor", "conv", "attention", "attention_causal", "conv_transpose"):
+        for name in ("gemm", "gemm_rowmajor", "conv", "attention", "attention_causal", "conv_transpose", "resnet18_b1",
+                     "resnet18_b32"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)
