@@ -257,8 +257,8 @@ TraceaStatus tracea_conv_transpose2d_ex(TraceaTensorView x, TraceaTensorView w, 
 
 /* Split-K.  A gemm / conv2d launch with few output tiles and a long K (tiles * 2 <= 256 CUs,
  * at least 8 K tiles) is split along K over more workgroups; fp32 partial products go to a
- * scratch buffer the library keeps per (device, stream) (at most 64 MiB, allocated on first
- * need, never while the stream is being captured) and a second kernel sums them and applies
+ * scratch buffer the library keeps per (device, stream) (grown on demand up to 64 MiB, never
+ * while the stream is being captured, never freed) and a second kernel sums them and applies
  * the operator chain.  On by default; tracea_set_split_k(0) turns it off.
  * tracea_last_split_k: K ranges of the calling thread's latest gemm / conv2d launch (1: not split). */
 void tracea_set_split_k(int32_t enabled);

@@ -417,7 +417,8 @@ void fill_grid(ContractionArgs *a, const ContractionVariant &v) {
 // channels: 8 tiles, 72 K tiles each).  Such a launch is split along K over blockIdx.y;
 // the fp32 partial products go to a scratch buffer and a second kernel sums them and runs
 // the operator chain.  The scratch buffer is kept per (device, stream), grows on demand up
-// to 64 MiB and is never allocated while the stream is being captured into a graph.
+// to 64 MiB, is never allocated while the stream is being captured into a graph and is
+// never freed.
 constexpr size_t kSplitScratchCap = 64u << 20;
 std::mutex g_scratch_mu;
 std::map<std::pair<int, void *>, std::pair<void *, size_t>> g_scratch;
@@ -432,12 +433,9 @@ void *splitk_scratch(int device, hipStream_t stream, size_t bytes) {
     (void)hipGetLastError();
     return nullptr;
   }
-  if (slot.first != nullptr) {
-    // launches queued on this stream may still write the old buffer
-    if (hipStreamSynchronize(stream) != hipSuccess) return nullptr;
-    (void)hipFree(slot.first);
-    slot = {nullptr, 0};
-  }
+  // A buffer that is outgrown is not freed: launches queued on the stream, and HIP graphs
+  // captured from it, may still hold its address.  Sizes double, so everything ever
+  // allocated for one stream stays below twice the cap.
   size_t want = 1u << 20;
   while (want < bytes) want <<= 1;
   void *p = nullptr;

@@ -405,6 +405,19 @@ TraceaStatus ExecutionPlan::run(void *arena, int device, void *stream) const {
     if ((st.kind == "Conv2d" || st.kind == "Gemm" || st.kind == "Linear") && st.weight == nullptr)
       return fail(TRACEA_INVALID_PARAMS, "tracea_plan_run: '%s' has no weight bound", st.name.c_str());
   }
+  // the node kernels below launch on the current device; the caller's choice is put back
+  struct DeviceGuard {
+    int prev = -1;
+    ~DeviceGuard() { if (prev >= 0) (void)hipSetDevice(prev); }
+  } guard;
+  {
+    int cur = -1;
+    if (hipGetDevice(&cur) == hipSuccess && cur != device) {
+      hipError_t e = hipSetDevice(device);
+      if (e != hipSuccess) return fail(TRACEA_CUDA_ERROR, "tracea_plan_run: %s", hipGetErrorString(e));
+      guard.prev = cur;
+    }
+  }
   auto view = [&](void *ptr, int rank, const uint64_t *shape, const int64_t *stride, TraceaDType d) {
     TraceaTensorView v{};
     v.ptr = ptr; v.rank = (uint32_t)rank; v.shape = shape; v.stride = stride; v.dtype = d; v.device_id = device;
@@ -465,8 +478,6 @@ TraceaStatus ExecutionPlan::run(void *arena, int device, void *stream) const {
                                   view(address(st.inputs[1], arena), 4, sh, nullptr, dt),
                                   view(address(st.inputs[2], arena), 4, sh, nullptr, dt), &o, p);
     } else {
-      hipError_t cur = hipSetDevice(device);
-      if (cur != hipSuccess) return fail(TRACEA_CUDA_ERROR, "tracea_plan_run: %s", hipGetErrorString(cur));
       int e = 0;
       if (st.kind == "GlobalAveragePool") {
         e = launch_global_avg_pool(address(st.inputs[0], arena), out, dt, dt, (int)st.g[0], (int)(st.g[2] * st.g[3]),
