@@ -115,3 +115,18 @@ def test_large_problems_are_not_split(tracea_gpu, split_switch):
     a = torch.randn(64, 256, device="cuda").half()          # few tiles but a short K
     tracea_gpu.gemm(a, torch.randn(256, 64, device="cuda").half())
     assert capi.lib().tracea_last_split_k() == 1
+
+
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (256, 256, 4096), (100, 36, 2052)])
+def test_fp32_gemm_split_matches_float64(tracea_gpu, split_switch, shape):
+    capi = split_switch
+    m, n, k = shape
+    rng = np.random.default_rng(m + k)
+    a = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64) + bias
+    got = tracea_gpu.gemm(_dev(a), _dev(b), bias=_dev(bias), epilogue="bias")
+    assert capi.lib().tracea_last_split_k() >= 2
+    assert got.dtype == torch.float32
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=0, atol=1e-4 * np.sqrt(k))

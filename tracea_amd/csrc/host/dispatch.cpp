@@ -537,8 +537,27 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     args.M = (int)M; args.N = (int)N; args.K = (int)K;
     args.lda = a.stride[0]; args.ldb = b.stride[0]; args.ldc = c.stride[0];
     args.out_dtype = DT_F32;
-    args.epi = chain;
-    return hip_status("gemm_f32 launch", launch_gemm_f32(args, stream));
+    // the fp32 kernel has one tile shape, 128x128x16; it splits along K by the same rule
+    static const ContractionVariant f32_tile = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr};
+    int k_split = 0;
+    const int splits = g_split_k_enabled.load() ? choose_split(f32_tile, (int)M, (int)N, (int)K, &k_split) : 1;
+    void *scratch = splits > 1 ? splitk_scratch(c.device, stream, (size_t)splits * M * N * 4) : nullptr;
+    t_last_splits = scratch != nullptr ? splits : 1;
+    if (scratch == nullptr) {
+      args.epi = chain;
+      return hip_status("gemm_f32 launch", launch_gemm_f32(args, stream));
+    }
+    SplitKReduceArgs r{};
+    r.partial = (const float *)scratch;
+    r.out = c.ptr; r.out_dtype = DT_F32;
+    r.splits = splits; r.M = (int)M; r.N = (int)N; r.ldc = c.stride[0];
+    r.epi = chain;
+    args.C = scratch;
+    args.ldc = N;
+    args.k_split = k_split;
+    TraceaStatus st = hip_status("gemm_f32 launch", launch_gemm_f32(args, stream));
+    if (st != TRACEA_SUCCESS) return st;
+    return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
   }
   GenericGemmArgs g{};
   g.A = a.ptr; g.B = b.ptr; g.C = c.ptr;

@@ -25,7 +25,12 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
   int tile_m, tile_n;
   tile_coordinates(args, tile_m, tile_n);
   const int m0 = tile_m * F32_BM, n0 = tile_n * F32_BN;
-  const int M = args.M, N = args.N, K = args.K;
+  const int M = args.M, N = args.N;
+  // split-K as in the half-precision kernels: K range [kb, K) of this workgroup, partial
+  // product to rows zrow.. of the workspace
+  const int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
+  const int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
+  const long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
   const float *A = (const float *)args.A;
   const float *B = (const float *)args.B;
 
@@ -33,6 +38,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
   // B tile: 16 k x 128 n   = 512 float4 pieces, 2 per thread (k = q/32, nq = q%32)
   f32x4 ra[2], rb[2];
   auto fetch = [&](int k0) {
+    k0 += kb;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int q = tid + i * 256;
@@ -43,10 +49,10 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
       const f32x4 v = *(const f32x4 *)(A + (long long)m * args.lda + (ok ? k : 0));
       const f32x4 z = {0.f, 0.f, 0.f, 0.f};
       ra[i] = ok ? v : z;
-      const int kb = k0 + q / 32;
+      const int krow = k0 + q / 32;
       const int n = n0 + (q % 32) * 4;
-      const bool okb = kb < K && n < N;
-      const f32x4 w = *(const f32x4 *)(B + (okb ? (long long)kb * args.ldb + n : 0ll));
+      const bool okb = krow < K && n < N;
+      const f32x4 w = *(const f32x4 *)(B + (okb ? (long long)krow * args.ldb + n : 0ll));
       rb[i] = okb ? w : z;
     }
   };
@@ -70,7 +76,7 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   const int lrow = lane & 31, lhalf = lane >> 5;
-  const int nk = (K + F32_BK - 1) / F32_BK;
+  const int nk = (K - kb + F32_BK - 1) / F32_BK;
   fetch(0);
   for (int kt = 0; kt < nk; ++kt) {
     stash();
@@ -105,8 +111,8 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
         if (m < M && n < N) {
           float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
                         acc[i][j][g * 4 + 3]};
-          apply_epilogue<4>(v, m, n, N - n, args.epi);
-          store_from_float<4>(args.C, args.out_dtype, (long long)m * args.ldc + n, N - n, v);
+          apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
+          store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
         }
       }
   }
@@ -117,7 +123,8 @@ int launch_gemm_f32(const ContractionArgs &a, hipStream_t stream) {
   args.grid_m = (a.M + F32_BM - 1) / F32_BM;
   args.grid_n = (a.N + F32_BN - 1) / F32_BN;
   args.group_m = 4;
-  hipLaunchKernelGGL(gemm_f32_kernel, dim3((unsigned)(args.grid_m * args.grid_n)), dim3(256), 0,
+  const unsigned splits = a.k_split > 0 ? (unsigned)((a.K + a.k_split - 1) / a.k_split) : 1u;
+  hipLaunchKernelGGL(gemm_f32_kernel, dim3((unsigned)(args.grid_m * args.grid_n), splits), dim3(256), 0,
                      stream, args);
   return (int)hipGetLastError();
 }
