@@ -6,7 +6,7 @@ fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
 FlashAttention-2 forward named by the metric are timed in the same run and
 reported under "also".  Prints one JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_rowmajor|conv|attention|attention_causal|conv_transpose|resnet18_b1|resnet18_b32|copy]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_rowmajor|gemm_f32|gemm_f32_4096|conv|attention|attention_causal|conv_transpose|resnet18_b1|resnet18_b32|copy]
 """
 import argparse
 import json
@@ -19,6 +19,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
+PEAKS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}  # dense MFMA peak of the type a workload computes in
 # HBM-side bytes per launch of the dominant kernel of each workload, from the rocprofv3
 # FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
 # (profiles/bench_kernels_mi355x.md); None where no counter run exists.
@@ -46,6 +47,14 @@ def make_workload(name, torch, ops):
         c = torch.empty(m, n, device=dev, dtype=torch.float16)
         return ("fp16 GEMM 4096x4096x4096, A and B row-major, fp32 acc, fp16 out",
                 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n), "f16", lambda: ops.gemm(a, b, out=c))
+    if name in ("gemm_f32", "gemm_f32_4096"):
+        # the reference's CPU-runnable case on the device: fp32, row-major, uniform[-1,1] (fp32 MFMA peak 157.3 TFLOP/s)
+        m = n = k = 1024 if name == "gemm_f32" else 4096
+        a = torch.rand(m, k, device=dev, generator=g) * 2 - 1
+        b = torch.rand(k, n, device=dev, generator=g) * 2 - 1
+        c = torch.empty(m, n, device=dev)
+        return ("fp32 GEMM %dx%dx%d, row-major, uniform[-1,1]" % (m, n, k), 2.0 * m * n * k,
+                4.0 * (m * k + k * n + m * n), "f32", lambda: ops.gemm(a, b, out=c))
     if name == "conv":
         n, h, w, cin, cout = 32, 56, 56, 64, 64
         x = torch.randn(n, h, w, cin, device=dev, generator=g).half()
@@ -179,22 +188,22 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
         "data": "synthetic", "config": {"workload": label},
-        "pct_of_peak": round(100.0 * tflops / PEAK_TFLOPS, 2),
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_TFLOPS, 4),
+        "pct_of_peak": round(100.0 * tflops / PEAKS.get(dtype, PEAK_TFLOPS), 2),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAKS.get(dtype, PEAK_TFLOPS),
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAKS.get(dtype, PEAK_TFLOPS), 4),
                      "traffic": TRAFFIC_BYTES.get(args.workload),
                      "hbm_GBps_algorithmic": round(bytes_ / dev_s / 1e9, 1)},
     }
     if not args.no_extras:
         also = {}
-        for name in ("gemm", "gemm_rowmajor", "conv", "attention", "attention_causal", "conv_transpose", "resnet18_b1",
+        for name in ("gemm", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "attention", "attention_causal", "conv_transpose", "resnet18_b1",
                      "resnet18_b32"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)
             _, d = time_steps(torch, st, max(5, args.steps // 2), max(2, args.warmup // 2))
             also[name] = {"workload": lab, "tflops": round(fl / d / 1e12, 2),
-                          "pct_of_peak": round(100.0 * fl / d / 1e12 / PEAK_TFLOPS, 2),
+                          "pct_of_peak": round(100.0 * fl / d / 1e12 / PEAKS.get(dt, PEAK_TFLOPS), 2),
                           "us_per_launch": round(d * 1e6, 2), "dtype": dt}
         line["also"] = also
         line["cpu_baseline"] = cpu_baseline()

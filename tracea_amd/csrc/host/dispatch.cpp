@@ -537,6 +537,12 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     args.M = (int)M; args.N = (int)N; args.K = (int)K;
     args.lda = a.stride[0]; args.ldb = b.stride[0]; args.ldc = c.stride[0];
     args.out_dtype = DT_F32;
+    // the direct-to-LDS form addresses operands with 32-bit byte offsets
+    const long long a_extent = ((M - 1) * a.stride[0] + K) * 4, b_extent = ((K - 1) * b.stride[0] + N) * 4;
+    if (a_extent < (1ll << 31) && b_extent < (1ll << 31)) {
+      args.a_bytes = (unsigned)a_extent;
+      args.b_bytes = (unsigned)b_extent;
+    }
     // the fp32 kernel has one tile shape, 128x128x16; it splits along K by the same rule
     static const ContractionVariant f32_tile = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr};
     int k_split = 0;

@@ -100,22 +100,157 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
   }
 
   // operands were swapped: lane owns row (lane&31), channels 8g + 4*(lane>>5) + 0..3
+  // (compile-time indices: the body is large enough for the compiler to leave a plain loop
+  // rolled, and a run-time index into the accumulators moves them to scratch memory)
+  static_for<0, 16>([&](auto idx) {
+    constexpr int i = decltype(idx)::value >> 3, j = (decltype(idx)::value >> 2) & 1, g = decltype(idx)::value & 3;
+    const int m = m0 + wm * 64 + i * 32 + lrow;
+    const int n = n0 + wn * 64 + j * 32 + g * 8 + lhalf * 4;
+    if (m < M && n < N) {
+      float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+      apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
+      store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
+    }
+  });
+}
+
+
+// ---------------------------------------------------------------------------
+// fp32 GEMM, direct-to-LDS form.  Same product as gemm_f32_kernel, for operands
+// below 2 GiB (32-bit buffer offsets).  Tile 128x128x16, 4 waves (2x2), wave
+// tile 64x64 = 2x2 blocks of v_mfma_f32_32x32x2_f32.  Both operand tiles are
+// requested with buffer loads that write LDS directly into one of two stages
+// while the other is multiplied: one barrier per K tile, no staging registers,
+// no LDS write instructions.
+//   A tile [128 rows][16 k], 64-byte rows; piece q (16 bytes at LDS byte 16q) is
+//     row q/4, column q%4, and holds global column (q%4) ^ ((row/4)&3): the
+//     16-byte operand reads of 16 consecutive rows then fall in 16 different
+//     bank groups.
+//   B tile [16 k][128 n], 512-byte rows; piece q is k row q/32, column q%32, and
+//     holds global column (q%32) ^ (8*(row/8)): lanes 0-31 read k rows 0-7, lanes
+//     32-63 rows 8-15 of the same 32 channels, which the XOR moves to the other
+//     half of the banks.
+// An MFMA sums over two k; lane half h supplies k = 8h + t to the t-th MFMA of a
+// K tile for A and B alike, so A's operands are two 16-byte reads per row block
+// and B's are eight 4-byte reads per channel block.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs args) {
+  constexpr int BM = F32_BM, BN = F32_BN, BK = F32_BK;
+  constexpr int A_STAGE = BM * BK * 4, B_STAGE = BK * BN * 4, STAGE = A_STAGE + B_STAGE;
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int wm = wave & 1, wn = wave >> 1;
+  int tile_m, tile_n;
+  tile_coordinates(args, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int M = args.M, N = args.N;
+  const int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
+  const int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
+  const long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
+
+  constexpr unsigned OOB = 0x80000000u;
+  __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)args.A, 0, (int)args.a_bytes, 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)args.B, 0, (int)args.b_bytes, 0x00020000);
+  // two pieces of A and two of B per thread and K tile
+  unsigned a_voff[2], b_voff[2];
+  int a_kcol[2], b_krow[2];
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
-    const int m = m0 + wm * 64 + i * 32 + lrow;
+    const int q = tid + i * 256;
+    const int row = q >> 2;
+    int m = m0 + row;
+    m = m < M ? m : M - 1;  // rows past the end re-read the last row; their results are never stored
+    a_kcol[i] = ((q & 3) ^ ((row >> 2) & 3)) * 4;
+    a_voff[i] = (unsigned)(((long long)m * args.lda + a_kcol[i]) * 4);
+    b_krow[i] = q >> 5;
+    const int n = n0 + (((q & 31) ^ ((b_krow[i] >> 3) << 3)) << 2);
+    b_voff[i] = n < N ? (unsigned)(((long long)b_krow[i] * args.ldb + n) * 4) : OOB;
+  }
+  auto dma = [&](unsigned char *stage, int k0) {
+    k0 += kb;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      unsigned char *dst = stage + (i * 256 + wave_u * 64) * 16;
+      const unsigned va = k0 + a_kcol[i] < K ? a_voff[i] : OOB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void *)dst, 16, (int)va,
+                                               k0 * 4, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      unsigned char *dst = stage + A_STAGE + (i * 256 + wave_u * 64) * 16;
+      const unsigned vb = k0 + b_krow[i] < K ? b_voff[i] : OOB;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16, (int)vb,
+                                               (int)((long long)k0 * args.ldb * 4), 0, 0);
+    }
+  };
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * 64 + j * 32 + g * 8 + lhalf * 4;
-        if (m < M && n < N) {
-          float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
-                        acc[i][j][g * 4 + 3]};
-          apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
-          store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
-        }
-      }
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  // A: row wm*64 + i*32 + lrow, 16-byte columns 2h and 2h+1 (k = 8h .. 8h+7)
+  int a_off[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int row = wm * 64 + i * 32 + lrow;
+#pragma unroll
+    for (int c = 0; c < 2; ++c) a_off[i][c] = row * 64 + (((2 * lhalf + c) ^ ((row >> 2) & 3)) << 4);
   }
+  // B: k row 8h + t, channel wn*64 + j*32 + lrow
+  int b_off[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int n = wn * 64 + j * 32 + lrow;
+    b_off[j] = A_STAGE + (8 * lhalf) * 512 + ((((n >> 2) ^ (lhalf << 3)) << 2) + (n & 3)) * 4;
+  }
+
+  const int nk = (K - kb + BK - 1) / BK;
+  dma(smem, 0);
+  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const unsigned char *cur = smem + (kt & 1) * STAGE;
+    if (kt + 1 < nk) dma(smem + ((kt + 1) & 1) * STAGE, (kt + 1) * BK);
+    f32x4 af[2][2];
+    float bf[2][8];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) af[i][c] = *(const f32x4 *)(cur + a_off[i][c]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) bf[j][t] = *(const float *)(cur + b_off[j] + t * 512);
+#pragma unroll
+    for (int t = 0; t < 8; ++t)
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][t], af[i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // the next tile has landed (this wave's share)
+    __syncthreads();                     // ... everyone's, and nobody still reads `cur`
+  }
+
+  // operands were swapped: lane owns row (lane&31), channels 8g + 4*(lane>>5) + 0..3
+  // (compile-time indices: the body is large enough for the compiler to leave a plain loop
+  // rolled, and a run-time index into the accumulators moves them to scratch memory)
+  static_for<0, 16>([&](auto idx) {
+    constexpr int i = decltype(idx)::value >> 3, j = (decltype(idx)::value >> 2) & 1, g = decltype(idx)::value & 3;
+    const int m = m0 + wm * 64 + i * 32 + lrow;
+    const int n = n0 + wn * 64 + j * 32 + g * 8 + lhalf * 4;
+    if (m < M && n < N) {
+      float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+      apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
+      store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
+    }
+  });
 }
 
 int launch_gemm_f32(const ContractionArgs &a, hipStream_t stream) {
@@ -124,8 +259,10 @@ int launch_gemm_f32(const ContractionArgs &a, hipStream_t stream) {
   args.grid_n = (a.N + F32_BN - 1) / F32_BN;
   args.group_m = 4;
   const unsigned splits = a.k_split > 0 ? (unsigned)((a.K + a.k_split - 1) / a.k_split) : 1u;
-  hipLaunchKernelGGL(gemm_f32_kernel, dim3((unsigned)(args.grid_m * args.grid_n), splits), dim3(256), 0,
-                     stream, args);
+  const dim3 grid((unsigned)(args.grid_m * args.grid_n), splits);
+  // a_bytes / b_bytes are set by the dispatcher when both operands are below 2 GiB
+  if (a.a_bytes != 0 && a.b_bytes != 0) hipLaunchKernelGGL(gemm_f32_dma_kernel, grid, dim3(256), 0, stream, args);
+  else hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, args);
   return (int)hipGetLastError();
 }
 
