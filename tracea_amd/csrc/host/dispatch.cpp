@@ -332,26 +332,52 @@ TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s,
 // (operand re-use of the tile shape x measured gain of its pipeline).  Partial
 // tiles at the edges are paid in full through the tile count.  A tuning-cache
 // entry, when present, wins over this.
+namespace {
+// Number of K ranges for a launch of variant v (1: no split) and the extent of one range.
+int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split) {
+  const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
+  const int nk = (K + v.bk - 1) / v.bk;
+  if (v.pipeline == 4 || tiles * 2 > 256 || nk < 8) return 1;
+  long long splits = 256 / tiles;
+  if (splits > nk / 4) splits = nk / 4;  // at least 4 K tiles per range
+  if (splits < 2) return 1;
+  const int per = (int)((nk + splits - 1) / splits);
+  *k_split = per * v.bk;
+  return (nk + per - 1) / per;
+}
+
+}  // namespace
+
+// Estimated time in microseconds of each variant on the problem, smallest wins:
+//   rounds of workgroups over the 256 CUs x multiply-accumulates of one workgroup
+//   / (rate of a workgroup slot x the variant's efficiency), plus, for a launch that
+//   would be split along K, the reduction pass (launch and fp32 partials at ~3 TB/s).
+// The slot rate is calibrated on the 4096^3 GEMM (256x256 tiles, one round, 120 us);
+// the estimate then reads 52.8 / 25.9 us for a 3x3 convolution on N32 7x7x512 with
+// unsplit 64x64 tiles / 128x128 tiles split four ways, where 53.7 / 29.6 us were measured.
 int select_contraction_variant(int m, int n, int k, bool conv) {
-  (void)k;
   (void)conv;
-  const double cus = 256.0;
+  const double cus = 256.0, slot_rate = 1.43e6;  // multiply-accumulates per microsecond at efficiency 1
   int best = -1;
   double best_cost = 0.0;
   for (int i = 0; i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
     if (v.pipeline == 4) continue;  // needs the convolution geometry: see plan_conv_patch
     const double gm = (double)((m + v.bm - 1) / v.bm), gn = (double)((n + v.bn - 1) / v.bn);
-    const double tiles = gm * gn;
-    const double exact = tiles / cus > 1.0 ? tiles / cus : 1.0;
-    const double rounds = 0.5 * std::ceil(tiles / cus) + 0.5 * exact;  // co-resident workgroups soften the step
+    int k_split = 0;
+    const int splits = g_split_k_enabled.load() ? choose_split(v, m, n, k, &k_split) : 1;
+    const double units = gm * gn * splits;
+    const double k_per = splits > 1 ? (double)k_split : (double)(k > 0 ? k : 1);
+    const double exact = units / cus > 1.0 ? units / cus : 1.0;
+    const double rounds = 0.5 * std::ceil(units / cus) + 0.5 * exact;  // co-resident workgroups soften the step
     const double reuse = (double)(v.bm * v.bn) / (double)(v.bm + v.bn) / 128.0;
     double prior = reuse > 1.0 ? 1.0 : reuse;
     // measured on MI355X at 4096^3: the pipelined loops gain ~35 % over the plain
     // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
-    const double cost = rounds * (double)v.bm * (double)v.bn / prior;
+    double cost = rounds * (double)v.bm * (double)v.bn * k_per / (slot_rate * prior);
+    if (splits > 1) cost += 4.0 + (double)splits * m * n * 4.0 / 3.0e6;
     if (best < 0 || cost < best_cost) {
       best_cost = cost;
       best = i;
@@ -445,19 +471,6 @@ void *splitk_scratch(int device, hipStream_t stream, size_t bytes) {
   }
   slot = {p, want};
   return p;
-}
-
-// Number of K ranges for a launch of variant v (1: no split) and the extent of one range.
-int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split) {
-  const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
-  const int nk = (K + v.bk - 1) / v.bk;
-  if (v.pipeline == 4 || tiles * 2 > 256 || nk < 8) return 1;
-  long long splits = 256 / tiles;
-  if (splits > nk / 4) splits = nk / 4;  // at least 4 K tiles per range
-  if (splits < 2) return 1;
-  const int per = (int)((nk + splits - 1) / splits);
-  *k_split = per * v.bk;
-  return (nk + per - 1) / per;
 }
 
 // Launches `args` on variant v, split along K when that pays; `chain` is the operator chain
