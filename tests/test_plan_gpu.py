@@ -199,3 +199,31 @@ def test_unbound_inputs_are_reported_before_any_launch(tracea_gpu):
     plan.bind(0, torch.zeros(1, 8, 8, 16, device="cuda", dtype=torch.float16))
     with pytest.raises(RuntimeError, match="not bound|no weight bound"):
         plan.run()
+
+
+def test_attention_and_gemm_nodes_bf16(tracea_gpu):
+    from tracea_amd import graph as G, plan as P
+    b, h, s, d = 1, 2, 256, 64
+    g = {"operators": [G.input_node(1, "q"), G.input_node(2, "k"), G.input_node(3, "v"),
+                       {"Attention": dict(op_id=4, name="attn", b=b, s=s, h=h, d=d)},
+                       G.gemm_node(5, "proj", b * h * s, 48, d), G.relu_node(6, "act", b * h * s * 48)],
+         "dependencies": [[1, 4], [2, 4], [3, 4], [4, 5], [5, 6]]}
+    fused = G.fuse(g)
+    assert [list(n)[0] for n in fused["operators"]].count("Relu") == 0        # merged into the projection
+    gen = torch.Generator(device="cuda").manual_seed(21)
+    q, k, v = [torch.randn(b, h, s, d, device="cuda", generator=gen).bfloat16() for _ in range(3)]
+    w = (torch.randn(d, 48, device="cuda", generator=gen) * d ** -0.5).bfloat16()
+    plan = P.Plan(fused, dtype=torch.bfloat16)
+    plan.bind(1, q).bind(2, k).bind(3, v)
+    plan.bind(5, w.t().contiguous(), "weight_t")                              # stored [N,K]
+    plan.run()
+    attn = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    want = torch.relu(attn.bfloat16().float().reshape(-1, d) @ w.float())
+    got = plan.output(5, (b * h * s, 48)).float()
+    assert float((got - want).abs().max()) <= 3e-2 * max(1.0, float(want.abs().max()))
+    # the same plan again after rebinding one input gives the new answer (nothing is cached)
+    q2 = torch.randn(b, h, s, d, device="cuda", generator=gen).bfloat16()
+    plan.bind(1, q2).run()
+    attn2 = torch.nn.functional.scaled_dot_product_attention(q2.float(), k.float(), v.float())
+    want2 = torch.relu(attn2.bfloat16().float().reshape(-1, d) @ w.float())
+    assert float((plan.output(5, (b * h * s, 48)).float() - want2).abs().max()) <= 3e-2 * max(1.0, float(want2.abs().max()))
