@@ -23,7 +23,7 @@
 
 namespace tracea_amd {
 
-template <int DT, int TM, int BN, int WM, int WN, int NSB>
+template <int DT, int TM, int BN, int WM, int WN, int NSB, bool FULL>
 __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const ContractionArgs args) {
   constexpr int NT = WM * WN * 64;
   constexpr int BK = 64, CH = 8, ROW_BYTES = 128, RP = 2;  // filter tile: BN rows x 64 k, XOR-swizzled
@@ -161,16 +161,15 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
   // Tap state of the next k-step to be read: filter row r, column s, first channel c0.
   int tap_q = 0, tap_s = 0, tap_c = 0;  // q offset of (r, s=0); s; c0
   auto tap_offset = [&]() { return (tap_q + tap_s * args.dil_w) * pitch + tap_c * 2; };
+  // (selects, not branches: the main loop must stay one basic block, see below)
   auto tap_advance = [&]() {
     tap_c += 16;
-    if (tap_c == C) {
-      tap_c = 0;
-      tap_s += 1;
-      if (tap_s == s_sz) {
-        tap_s = 0;
-        tap_q += tap_h;
-      }
-    }
+    const bool wrap_c = tap_c == C;
+    tap_c = wrap_c ? 0 : tap_c;
+    tap_s += wrap_c ? 1 : 0;
+    const bool wrap_s = tap_s == s_sz;
+    tap_s = wrap_s ? 0 : tap_s;
+    tap_q += wrap_s ? tap_h : 0;
   };
 
   u32x4 fa[2][FM], fb[2][FN];
@@ -193,6 +192,41 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
   __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // patch and filter tile 0 of this wave have landed
   __syncthreads();
   read_operands(0, ring, 0);
+  if constexpr (FULL) {
+    // K is a multiple of BK: every tile has KS k-steps.  The loop body is then free of
+    // branches (the last tile is peeled off), which matters beyond the branches themselves:
+    // with the k-steps of a partial tile behind conditions the accumulators are live across
+    // several paths and the compiler reconciles its register choices at the loop head with
+    // a copy of all of them -- 64 v_accvgpr_mov per K tile and wave, as long as the 16 MFMAs
+    // of the tile.
+    int cur_i = 0, fill_i = NSB - 1;
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+      const unsigned char *cur = ring + cur_i * B_STAGE;
+      const int nxt_i = cur_i + 1 == NSB ? 0 : cur_i + 1;
+      const int tf = kt + NSB - 1 < nk ? kt + NSB - 1 : nk - 1;
+      dma_b(fill_i, tf * BK);
+#pragma unroll
+      for (int ks = 0; ks + 1 < KS; ++ks) {
+        read_operands((ks + 1) & 1, cur, ks + 1);
+        mma(ks & 1);
+      }
+      __builtin_amdgcn_s_waitcnt(WAIT_TILE);
+      __syncthreads();
+      read_operands(0, ring + nxt_i * B_STAGE, 0);
+      mma((KS - 1) & 1);
+      fill_i = cur_i;
+      cur_i = nxt_i;
+    }
+    {
+      const unsigned char *cur = ring + cur_i * B_STAGE;
+#pragma unroll
+      for (int ks = 0; ks + 1 < KS; ++ks) {
+        read_operands((ks + 1) & 1, cur, ks + 1);
+        mma(ks & 1);
+      }
+      mma((KS - 1) & 1);
+    }
+  } else
   for (int kt = 0; kt < nk; ++kt) {
     const unsigned char *cur = ring + (kt % NSB) * B_STAGE;
     const int nsteps = min(KS, ksteps - kt * KS);  // < KS only in the last tile
@@ -285,9 +319,9 @@ int launch_conv_patch(const ContractionArgs &a, bool conv, int dtype, bool b_nco
   size_t lds = (size_t)a.p_np_bytes + (size_t)NSB * BN * 128;
   if (lds < staging) lds = staging;
   const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(WM * WN * 64);
-#define TRACEA_LAUNCH_PATCH(DTV)                                                                    \
+#define TRACEA_LAUNCH_PATCH(DTV, FULLV)                                                             \
   do {                                                                                              \
-    auto kfn = conv_patch_kernel<DTV, TM, BN, WM, WN, NSB>;                                         \
+    auto kfn = conv_patch_kernel<DTV, TM, BN, WM, WN, NSB, FULLV>;                                  \
     static bool attr_done = false;                                                                  \
     if (!attr_done) {                                                                               \
       hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
@@ -298,8 +332,9 @@ int launch_conv_patch(const ContractionArgs &a, bool conv, int dtype, bool b_nco
     hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                           \
     return (int)hipGetLastError();                                                                  \
   } while (0)
-  if (dtype == DT_F16) TRACEA_LAUNCH_PATCH(DT_F16);
-  else TRACEA_LAUNCH_PATCH(DT_BF16);
+  const bool full = a.K % 64 == 0;  // every filter tile holds all of its k-steps
+  if (dtype == DT_F16) { if (full) TRACEA_LAUNCH_PATCH(DT_F16, true); else TRACEA_LAUNCH_PATCH(DT_F16, false); }
+  else { if (full) TRACEA_LAUNCH_PATCH(DT_BF16, true); else TRACEA_LAUNCH_PATCH(DT_BF16, false); }
 #undef TRACEA_LAUNCH_PATCH
   return (int)hipErrorInvalidValue;
 }

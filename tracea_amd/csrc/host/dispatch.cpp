@@ -797,22 +797,25 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
            g.pad_h, tuning_device_name());
   int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
   if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
-  // Default choice of a patch-resident variant.  Measured on MI355X it beats the
-  // streamed tiles only where the filter bank is narrow and an image holds
-  // several full tiles (N32 56x56x64 -> 64, 3x3: 21.9 us against 23.1 us); with
-  // 128 filters, stride 2 or 14x14 images the streamed 128x64 tiles are faster.
-  // One shape is thin evidence: a tuning-cache entry or a forced variant wins
-  // over this rule, and tracea_autotune_conv2d measures every variant.  Below 256
-  // tiles of 256 pixels the kernel cannot fill the device (it has no split along
-  // K): a single 56x56 image is 13 workgroups.
-  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && a.N <= 64 &&
-      g.stride_h == 1 && g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 &&
-      (long long)g.block.h_out * g.block.w_out >= 4 * 256 && (long long)a.M >= 256ll * 256) {
+  // Default choice of a patch-resident variant: stride-1 convolutions with a real filter
+  // window whose launch has enough workgroups to occupy the device (the kernel has no
+  // split along K: one 56x56 image is 13 workgroups) -- 256x64 tiles for up to 64 filters,
+  // 128x128 beyond.  Measured on MI355X, N = 32, 3x3, against the best streamed variant:
+  // 56x56x64->64 18.0 / 20.8 us, 28x28x128->128 17.9 / 21.1 us, 14x14x256->256 26.1 / 30.3 us.
+  // A tuning-cache entry or a forced variant wins over this rule, and
+  // tracea_autotune_conv2d measures every variant.
+  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && g.stride_h == 1 &&
+      g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 && a.K % 64 == 0) {
+    const int want_bm = a.N <= 64 ? 256 : 128, want_bn = a.N <= 64 ? 64 : 128;
     for (int i = 0; i < contraction_variant_count(); ++i) {
       const ContractionVariant &cv = contraction_variant(i);
-      if (cv.pipeline == 4 && cv.bm == 256 && cv.bn == 64) {
+      if (cv.pipeline == 4 && cv.bm == want_bm && cv.bn == want_bn) {
         ContractionArgs probe = a;
-        if (plan_conv_patch(g, cv, plan.w_ncontig, &probe)) vi = i;
+        // ... and whose tiles are mostly pixels: a 7x7 image fills 49 rows of a 128-row tile
+        const long long hw = (long long)g.block.h_out * g.block.w_out;
+        if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= 96 &&
+            hw * 4 >= (long long)probe.p_tiles * cv.bm * 3)
+          vi = i;
         break;
       }
     }
