@@ -108,15 +108,19 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
   }
   auto dma_b = [&](int stage, int k0) {
     unsigned char *sB = ring + stage * B_STAGE;
+    // columns of the last tile past K read as zero (and are not fetched: the scalar offset
+    // takes no part in the hardware's range check, so they would lie past the row's end)
+    const bool inside = FULL || k0 + gpc * 8 < K;
 #pragma unroll
     for (int i = 0; i < NB; ++i) {
       unsigned char *dst = sB + (i * PR_STEP + wave_u * (64 / CH)) * ROW_BYTES;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void *)dst, 16,
-                                               (int)b_voff[i], k0 * 2, 0, 0);
+                                               (int)(inside ? b_voff[i] : OOB), k0 * 2, 0, 0);
     }
   };
-  // K is a multiple of 16 (C is); the last filter tile may hold fewer than KS
-  // k-steps, the columns past K it carries are never multiplied
+  // K is a multiple of 16 (C is); when it is not a multiple of BK (FULL false) the last
+  // filter tile holds fewer than KS k-steps: its missing k-steps are multiplied all the same,
+  // with zero operands, so that the loop below has no conditions
   const int nk = (K + BK - 1) / BK;
   const int ksteps = K >> 4;
 #pragma unroll
@@ -173,12 +177,19 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
   };
 
   u32x4 fa[2][FM], fb[2][FN];
+  int next_step = 0;  // k-steps read so far (FULL false only)
   auto read_operands = [&](int set, const unsigned char *sB, int ks) {
-    const int toff = tap_offset();
+    const bool live = FULL || next_step < ksteps;
+    next_step += 1;
+    const int toff = live ? tap_offset() : 0;  // past the last tap the patch is not addressed
     tap_advance();
     const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
 #pragma unroll
-    for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(patch + a_base[i] + toff);
+    for (int i = 0; i < FM; ++i) {
+      const u32x4 v = *(const u32x4 *)(patch + a_base[i] + toff);
+      fa[set][i] = live ? v : zero4;
+    }
 #pragma unroll
     for (int j = 0; j < FN; ++j) fb[set][j] = *(const u32x4 *)(sB + b_row + j * 32 * ROW_BYTES + coff);
   };
@@ -192,17 +203,18 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
   __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // patch and filter tile 0 of this wave have landed
   __syncthreads();
   read_operands(0, ring, 0);
-  if constexpr (FULL) {
-    // K is a multiple of BK: every tile has KS k-steps.  The loop body is then free of
-    // branches (the last tile is peeled off), which matters beyond the branches themselves:
-    // with the k-steps of a partial tile behind conditions the accumulators are live across
-    // several paths and the compiler reconciles its register choices at the loop head with
-    // a copy of all of them -- 64 v_accvgpr_mov per K tile and wave, as long as the 16 MFMAs
-    // of the tile.
+  {
+    // The loop body is free of branches (the last tile is peeled off, a partial last tile is
+    // padded with zero operands), which matters beyond the branches themselves: with the
+    // k-steps of a partial tile behind conditions the accumulators were live across several
+    // paths and the compiler reconciled its register choices at the loop head with a copy of
+    // all of them -- 64 v_accvgpr_mov per K tile and wave, as long as the 16 MFMAs of the tile.
     int cur_i = 0, fill_i = NSB - 1;
     for (int kt = 0; kt + 1 < nk; ++kt) {
       const unsigned char *cur = ring + cur_i * B_STAGE;
       const int nxt_i = cur_i + 1 == NSB ? 0 : cur_i + 1;
+      // the stage released by the previous barrier receives tile kt+NSB-1 (clamped:
+      // a repeat of the last tile lands in a stage that is not read again)
       const int tf = kt + NSB - 1 < nk ? kt + NSB - 1 : nk - 1;
       dma_b(fill_i, tf * BK);
 #pragma unroll
@@ -210,8 +222,10 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
         read_operands((ks + 1) & 1, cur, ks + 1);
         mma(ks & 1);
       }
-      __builtin_amdgcn_s_waitcnt(WAIT_TILE);
+      __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // tile kt+1 has landed; newer requests stay in flight
       __syncthreads();
+      // the last k-step of the tile runs behind the barrier, together with the first
+      // operand reads of the next tile
       read_operands(0, ring + nxt_i * B_STAGE, 0);
       mma((KS - 1) & 1);
       fill_i = cur_i;
@@ -226,30 +240,6 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
       }
       mma((KS - 1) & 1);
     }
-  } else
-  for (int kt = 0; kt < nk; ++kt) {
-    const unsigned char *cur = ring + (kt % NSB) * B_STAGE;
-    const int nsteps = min(KS, ksteps - kt * KS);  // < KS only in the last tile
-    // the stage released by the previous barrier receives tile kt+NSB-1 (clamped:
-    // a repeat of the last tile lands in a stage that is not read again)
-    {
-      const int tf = kt + NSB - 1 < nk ? kt + NSB - 1 : nk - 1;
-      dma_b((kt + NSB - 1) % NSB, tf * BK);
-    }
-#pragma unroll
-    for (int ks = 0; ks + 1 < KS; ++ks) {
-      if (ks + 1 < nsteps) {
-        read_operands((ks + 1) & 1, cur, ks + 1);
-        mma(ks & 1);
-      }
-    }
-    __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // tile kt+1 has landed; newer requests stay in flight
-    __syncthreads();
-    // the last k-step of the tile runs behind the barrier, together with the first
-    // operand reads of the next tile (a full tile ends on set 1, so set 0 is free)
-    if (kt + 1 < nk) read_operands(0, ring + ((kt + 1) % NSB) * B_STAGE, 0);
-    if (nsteps & 1) mma(0);
-    else mma(1);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // no request may still land on the epilogue staging
   __syncthreads();
