@@ -69,17 +69,14 @@ struct Mfma32<DT_BF16> {
 // q = n / d, r = n % d through a precomputed reciprocal: m = ceil(2^(32+s)/d),
 // or m == 0 for a power-of-two d with s = log2(d).  Same arithmetic as the
 // reference's device fast_divmod (src/emitter/cuda/conv.rs:144-151).
+// One expression for all cases (n >= 0), because a branch on the kind of divisor, uniform as
+// it is, splits the tile loaders of the convolution into basic blocks that the MFMAs cannot
+// be interleaved with: umulhi(n, m) is the scaled quotient for a real reciprocal and 0 for
+// m == 0, where n itself takes its place (d == 1 is the power of two with s == 0).
 __device__ __forceinline__ void fast_divmod(int n, unsigned m, unsigned s, int d, int &q, int &r) {
-  if (d == 1) {
-    q = n;
-    r = 0;
-  } else if (m == 0) {
-    q = n >> s;
-    r = n & (d - 1);
-  } else {
-    q = (int)(__umulhi((unsigned)n, m) >> s);
-    r = n - q * d;
-  }
+  const unsigned scaled = __umulhi((unsigned)n, m) + (m == 0 ? (unsigned)n : 0u);
+  q = (int)(scaled >> s);
+  r = n - q * d;
 }
 
 // ---- epilogue helpers -------------------------------------------------------
@@ -660,7 +657,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
       for (int i = 0; i < NA; ++i) {
         const int hi = a_hb[i] + dh, wi = a_wb[i] + dw;
-        const bool ok = kvalid && hi >= 0 && hi < args.h_in && wi >= 0 && wi < args.w_in;
+        // (unsigned compares and bitwise &: no short-circuit control flow around the address)
+        const bool ok = kvalid & ((unsigned)hi < (unsigned)args.h_in) & ((unsigned)wi < (unsigned)args.w_in);
         const long long off = a_off[i] + ((long long)hi * args.w_in + wi) * args.c_in + ci;
         ra[i] = *(const u32x4 *)(Ag + (ok ? off : 0ll));
         a_ok |= ok ? (1u << i) : 0u;
@@ -745,8 +743,13 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       int soff;
       if constexpr (CONV) {
         const int hi_ = a_hb[i] + dh, wi = a_wb[i] + dw;
-        const bool ok = kvalid && hi_ >= 0 && hi_ < args.h_in && wi >= 0 && wi < args.w_in;
-        voff = ok ? a_voff[i] + (unsigned)(((hi_ * args.w_in + wi) * args.c_in + ci) * 2) : OOB;
+        // The offset is formed unconditionally and selected afterwards, with unsigned compares
+        // joined by bitwise &: written with && and inside the conditional, each piece became a
+        // predicated block of its own and the post-barrier share of the requests a chain of
+        // branches that no MFMA could be scheduled into.
+        const bool ok = kvalid & ((unsigned)hi_ < (unsigned)args.h_in) & ((unsigned)wi < (unsigned)args.w_in);
+        const unsigned in_range = a_voff[i] + (unsigned)(((hi_ * args.w_in + wi) * args.c_in + ci) * 2);
+        voff = ok ? in_range : OOB;
         soff = 0;
       } else {
         voff = kvalid ? a_voff[i] : OOB;

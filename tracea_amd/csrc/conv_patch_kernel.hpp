@@ -88,8 +88,10 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
     fast_divmod(chunk, args.p_cpp_m, args.p_cpp_s, cpp, qrel, part);
     fast_divmod(qmin + qrel, args.p_pw_m, args.p_pw_s, PW, hp, wp);
     const int hi = hp - args.pad_h, wi = wp - args.pad_w;
-    const bool ok = qrel < np && part < cdata && hi >= 0 && hi < args.h_in && wi >= 0 && wi < args.w_in;
-    const unsigned voff = ok ? (unsigned)(((hi * args.w_in + wi) * C + part * 8) * 2) : OOB;
+    const bool ok = (qrel < np) & (part < cdata) & ((unsigned)hi < (unsigned)args.h_in) &
+                    ((unsigned)wi < (unsigned)args.w_in);  // bitwise: no control flow around the address
+    const unsigned in_range = (unsigned)(((hi * args.w_in + wi) * C + part * 8) * 2);
+    const unsigned voff = ok ? in_range : OOB;
     unsigned char *dst = patch + (it * NT + wave_u * 64) * 16;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void *)dst, 16, (int)voff,
                                              0, 0, 0);

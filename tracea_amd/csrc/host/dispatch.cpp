@@ -370,8 +370,11 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
     const double k_per = splits > 1 ? (double)k_split : (double)(k > 0 ? k : 1);
     const double exact = units / cus > 1.0 ? units / cus : 1.0;
     const double rounds = 0.5 * std::ceil(units / cus) + 0.5 * exact;  // co-resident workgroups soften the step
+    // operand reuse of the tile relative to 256x256; its square root matches the measured
+    // ranking of the tile shapes better than the ratio itself, which overrates large tiles
+    // (smaller tiles put more waves on a CU and hide more latency)
     const double reuse = (double)(v.bm * v.bn) / (double)(v.bm + v.bn) / 128.0;
-    double prior = reuse > 1.0 ? 1.0 : reuse;
+    double prior = reuse > 1.0 ? 1.0 : std::sqrt(reuse);
     // measured on MI355X at 4096^3: the pipelined loops gain ~35 % over the plain
     // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
@@ -798,15 +801,15 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
   if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
   // Default choice of a patch-resident variant: stride-1 convolutions with a real filter
-  // window whose launch has enough workgroups to occupy the device (the kernel has no
-  // split along K: one 56x56 image is 13 workgroups) -- 256x64 tiles for up to 64 filters,
-  // 128x128 beyond.  Measured on MI355X, N = 32, 3x3, against the best streamed variant:
-  // 56x56x64->64 18.0 / 20.8 us, 28x28x128->128 17.9 / 21.1 us, 14x14x256->256 26.1 / 30.3 us.
-  // A tuning-cache entry or a forced variant wins over this rule, and
-  // tracea_autotune_conv2d measures every variant.
-  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && g.stride_h == 1 &&
+  // window and at most 64 filters, whose launch has enough workgroups to occupy the device
+  // (the kernel has no split along K: one 56x56 image is 13 workgroups).  Measured on
+  // MI355X, N = 32, 3x3, against the best streamed variant: 56x56x64->64 17.9 / 18.4 us.
+  // With 128 and 256 filters (28x28, 14x14) the streamed 128x64 tiles are faster
+  // (17.6 / 18.5 us, 20.9 / 23.5 us).  A tuning-cache entry or a forced variant wins over
+  // this rule, and tracea_autotune_conv2d measures every variant.
+  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && a.N <= 64 && g.stride_h == 1 &&
       g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 && a.K % 64 == 0) {
-    const int want_bm = a.N <= 64 ? 256 : 128, want_bn = a.N <= 64 ? 64 : 128;
+    const int want_bm = 256, want_bn = 64;
     for (int i = 0; i < contraction_variant_count(); ++i) {
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline == 4 && cv.bm == want_bm && cv.bn == want_bn) {
