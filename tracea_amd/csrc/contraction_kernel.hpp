@@ -523,6 +523,27 @@ struct Interleave {
   }
 };
 
+// The same for two classes that must keep their order (every instruction of the
+// first class ahead of every instruction of the second): the kFirst + kSecond
+// instructions are spread evenly over the MFMAs in that order.  Used where LDS
+// reads precede direct-to-LDS loads in program order: the compiler cannot tell
+// that the two touch different buffers and will not move one across the other,
+// so a pipeline that alternates the classes cannot be satisfied and is dropped.
+template <int kStep, int kMfmas, int kClassFirst, int kFirst, int kClassSecond, int kSecond>
+struct Sequenced {
+  static __device__ __forceinline__ void run() {
+    constexpr int total = kFirst + kSecond;
+    constexpr int lo = (kStep * total) / kMfmas, hi = ((kStep + 1) * total) / kMfmas;  // items [lo, hi) go here
+    constexpr int nf = (hi < kFirst ? hi : kFirst) - (lo < kFirst ? lo : kFirst);
+    constexpr int ns = (hi - lo) - nf;
+    if constexpr (nf > 0) __builtin_amdgcn_sched_group_barrier(kClassFirst, nf, 0);
+    if constexpr (ns > 0) __builtin_amdgcn_sched_group_barrier(kClassSecond, ns, 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (kStep + 1 < kMfmas)
+      Sequenced<kStep + 1, kMfmas, kClassFirst, kFirst, kClassSecond, kSecond>::run();
+  }
+};
+
 // ---- the kernel -----------------------------------------------------------------
 template <int DT, int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, bool CONV, bool B_NCONTIG>
 __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const ContractionArgs args) {
@@ -1007,7 +1028,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // The L requests of a tile are issued in SPREAD consecutive k-step regions,
     // the first of which is the one right after the barrier that freed the
     // destination buffer; the rest follow at the start of the next tile.
-    constexpr int SPREAD = 2;  // three shares measured no better than two
+    constexpr int SPREAD = 2;  // three shares measured no better than two, one share worse
     constexpr int CUT1 = L / SPREAD, CUT2 = SPREAD == 3 ? 2 * L / SPREAD : L;
     dma(smem, smem + A_STAGE, 0, 0, L);
     dma(smem + STAGE, smem + STAGE + A_STAGE, nk > 1 ? BK : 0, 0, CUT1);  // first share of tile 1
@@ -1019,10 +1040,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       unsigned char *nxt = smem + ((kt + 1) & 1) * STAGE;
       // k-step 0 carries the second share of tile kt+1 (its first share was
       // requested right after the previous barrier, or in the prologue)
-      dma(nxt, nxt + A_STAGE, (kt + 1) * BK, CUT1, CUT2);
       read_operands(1, cur, cur + A_STAGE, 1);
+      dma(nxt, nxt + A_STAGE, (kt + 1) * BK, CUT1, CUT2);
       mma(0);
-      Interleave<0, R, 0x020, CUT2 - CUT1, 0x100, D>::run();
+      Sequenced<0, R, 0x100, D, 0x020, CUT2 - CUT1>::run();
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int ks = 1; ks + 1 < KS; ++ks) {
@@ -1038,10 +1059,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       // every wave has finished reading `cur`: request the first share of tile
       // kt+2 into it (clamped to the last tile, whose second copy is never read)
       // while the last k-step of tile kt runs from registers
-      dma(cur, cur + A_STAGE, (kt + 2 < nk ? kt + 2 : nk - 1) * BK, 0, CUT1);
       read_operands(0, nxt, nxt + A_STAGE, 0);
+      dma(cur, cur + A_STAGE, (kt + 2 < nk ? kt + 2 : nk - 1) * BK, 0, CUT1);
       mma((KS - 1) & 1);
-      Interleave<0, R, 0x020, CUT1, 0x100, D>::run();
+      Sequenced<0, R, 0x100, D, 0x020, CUT1>::run();
       __builtin_amdgcn_sched_barrier(0);
     }
     {
