@@ -184,6 +184,18 @@ TraceaStatus tracea_gemm(TraceaTensorView a, TraceaTensorView b, const TraceaTen
                          const TraceaTensorView *residual, TraceaTensorView *c,
                          TraceaGemmParams params);
 
+/* ---- Low-rank MLP: the reference's UnifiedOpType::LowRankMlp {m, n, k, r}
+ * (src/emitter/traits.rs:95-100; kernel sketch src/emitter/cuda/low_rank.rs:4-150, whose
+ * matrix steps are left empty; expected value k*r for all-ones operands in
+ * examples/low_rank_mlp_test.rs:96-98).  c[M,N] = epilogue((x[M,K] a[K,R]) b[R,N]);
+ * the rank-r product is rounded to the operands' type before the second product,
+ * as the reference keeps it in a half-precision tile.  x, a, b share one floating
+ * type; strides and epilogue as for tracea_gemm.  The intermediate lives in a
+ * stream-ordered allocation: the call must not be captured into a HIP graph. */
+TraceaStatus tracea_low_rank_mlp(TraceaTensorView x, TraceaTensorView a, TraceaTensorView b,
+                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                 TraceaTensorView *c, TraceaGemmParams params);
+
 /* ---- FlashAttention-2 forward: reference include/tracea.hpp:147-149,
  * src/interface/c_bindings.rs:443-495.  q,k,v,o [B,H,S,D]. */
 TraceaStatus tracea_attention(TraceaTensorView q, TraceaTensorView k, TraceaTensorView v,

@@ -17,7 +17,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def _declared_functions():
     names = set()
-    for header in ("tracea.h", "tracea_tuner.h", "tracea_graph.h", "tracea_plan.h"):
+    for header in ("tracea.h", "tracea_tuner.h", "tracea_graph.h", "tracea_plan.h", "tracea_ttg.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names.update(re.findall(r"\b(tracea_[a-z0-9_]+)\s*\(", text))

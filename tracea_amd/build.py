@@ -31,7 +31,7 @@ INCLUDE = os.path.normpath(os.path.join(HERE, "..", "include"))
 COMMON = ["-I" + INCLUDE, "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-command-line-argument",
           "-Wno-pass-failed"]
 
-HOST_SOURCES = ["abi.cpp", "tuner_abi.cpp", "graph_abi.cpp", "plan_abi.cpp", "host/execution_plan.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
+HOST_SOURCES = ["abi.cpp", "tuner_abi.cpp", "graph_abi.cpp", "plan_abi.cpp", "ttg_abi.cpp", "host/tile_graph.cpp", "host/execution_plan.cpp", "contraction_registry.cpp", "host/dispatch.cpp", "host/tuning.cpp",
                 "host/pipeline_config.cpp", "host/gaussian_process.cpp", "host/autotuner.cpp",
                 "host/graph_fusion.cpp"]
 DEVICE_SOURCES = ["support_kernels.hip", "conv_transpose_kernels.hip", "graph_kernels.hip", "attention_kernels.hip"]

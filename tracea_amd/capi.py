@@ -104,6 +104,32 @@ SIGNATURES = {
     "tracea_plan_output": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "tracea_plan_bind": (C.c_int, [C.c_void_p, C.c_uint64, C.c_char_p, C.c_void_p]),
     "tracea_plan_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "tracea_low_rank_mlp": (C.c_int, [TensorView, TensorView, TensorView, C.POINTER(TensorView),
+                                      C.POINTER(TensorView), C.POINTER(TensorView), GemmParams]),
+    "tracea_ttg_from_dense": (C.c_void_p, [C.c_uint32] * 6),
+    "tracea_ttg_from_dense_k_split": (C.c_void_p, [C.c_uint32] * 7),
+    "tracea_ttg_from_mask": (C.c_void_p, [C.c_uint32] * 6 + [C.c_void_p]),
+    "tracea_ttg_from_diagonal": (C.c_void_p, [C.c_uint32] * 6),
+    "tracea_ttg_from_random": (C.c_void_p, [C.c_uint32] * 6 + [C.c_double, C.c_uint64]),
+    "tracea_ttg_from_low_rank": (C.c_void_p, [C.c_uint32] * 7),
+    "tracea_ttg_from_tables": (C.c_void_p, [C.c_uint32] * 6 + [C.c_void_p, C.c_uint32, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_destroy": (None, [C.c_void_p]),
+    "tracea_ttg_num_active_tiles": (C.c_uint32, [C.c_void_p]),
+    "tracea_ttg_num_records": (C.c_uint32, [C.c_void_p]),
+    "tracea_ttg_num_edges": (C.c_uint32, [C.c_void_p]),
+    "tracea_ttg_l1_map": (C.c_uint32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_l1_map_ordered": (C.c_uint32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_l2_table": (C.c_uint32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_execution_order": (C.c_uint32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_edges": (C.c_uint32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_reuse_hints": (C.c_uint32, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_validate_order": (C.c_int32, [C.c_void_p, C.c_void_p, C.c_uint32]),
+    "tracea_ttg_device_size": (C.c_int, [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "tracea_ttg_upload_to": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]),
+    "tracea_gemm_ttg": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), C.POINTER(TensorView),
+                                  C.POINTER(TensorView), GemmParams, C.c_void_p]),
+    "tracea_gemm_ttg_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), GemmParams,
+                                     C.POINTER(EpilogueOp), C.c_uint32, C.c_void_p]),
     "tracea_set_split_k": (None, [C.c_int32]),
     "tracea_last_split_k": (C.c_int32, []),
     "tracea_variant_count": (C.c_int32, [C.c_char_p]),

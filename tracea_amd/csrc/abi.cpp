@@ -96,6 +96,12 @@ TraceaStatus tracea_gemm_ex(TraceaTensorView a, TraceaTensorView b, TraceaTensor
   TRACEA_GUARDED(dispatch_gemm_ops(a, b, c, params, ops, n_ops))
 }
 
+TraceaStatus tracea_low_rank_mlp(TraceaTensorView x, TraceaTensorView a, TraceaTensorView b,
+                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                 TraceaTensorView *c, TraceaGemmParams params) {
+  TRACEA_GUARDED(dispatch_low_rank_mlp(x, a, b, bias, residual, c, params))
+}
+
 TraceaStatus tracea_conv2d(TraceaTensorView x, TraceaTensorView w, const TraceaTensorView *b,
                            const TraceaTensorView *residual, TraceaTensorView *out,
                            TraceaConv2dParams params) {

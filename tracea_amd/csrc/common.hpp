@@ -41,6 +41,14 @@ struct ContractionArgs {
   int k_split;         // 0: one workgroup per tile runs all of K; else the K extent of one split (a multiple
                        // of the variant's BK): grid.y = ceil(K / k_split), C is the [splits][M][ldc] workspace
   int group_m;         // tile-order group height
+  // GEMM over a tile list (null: the dense grid_m x grid_n grid): workgroup p of the
+  // launch (grid.x = list length) runs record tile_list[p]; a record is 5 words
+  // {tile row, tile column, first k, end k, role}; tile_slice[p], if given, is the row
+  // block of the fp32 workspace C = [slices][M][ldc] its partial product goes to
+  const unsigned *tile_list;
+  const unsigned *tile_records;
+  const unsigned *tile_slice;
+  int tile_count;
   // convolution geometry (ConvParams of the reference, h/w split)
   int h_in, w_in, c_in, h_out, w_out, s_sz;
   int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;

@@ -568,16 +568,30 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   const int wave = tid >> 6;
   const int wm = wave % WM, wn = wave / WM;
 
-  int tile_m, tile_n;
-  tile_coordinates(args, tile_m, tile_n);
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int M = args.M, N = args.N;
   // Split-K: workgroups with blockIdx.y = z multiply the K range [z*k_split, (z+1)*k_split)
   // and write their fp32 partial product to rows z*M.. of C, which is then a workspace that
   // a reduction kernel sums.  kb is added to every K offset below; K is the end of the range.
-  const int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
-  const int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
-  const long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
+  int tile_m, tile_n;
+  int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
+  int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
+  long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
+  if (!CONV && args.tile_list != nullptr) {
+    // Tile list (the reference's two-level tile table, src/core/ttg.rs:3-11 and
+    // src/emitter/cuda/low_rank.rs:69-76): workgroup p runs record tile_list[p] =
+    // {tile row, tile column, first k, end k, role}; tiles without a record are not
+    // touched.  tile_slice, if given, names the row block of the fp32 workspace that
+    // receives this record's partial product (records that share a tile).
+    const unsigned *rec = args.tile_records + 5u * args.tile_list[blockIdx.x];
+    tile_m = (int)rec[0];
+    tile_n = (int)rec[1];
+    kb = (int)rec[2];
+    K = min(args.K, (int)rec[3]);
+    zrow = args.tile_slice != nullptr ? (long long)args.tile_slice[blockIdx.x] * M : 0ll;
+  } else {
+    tile_coordinates(args, tile_m, tile_n);
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   // ---- per-thread source coordinates of the pieces this thread moves ----
   const int pc = tid % CH;      // 16-byte column of every A piece of this thread
@@ -1236,7 +1250,9 @@ template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE>
 int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
                        hipStream_t stream) {
   constexpr size_t lds = (size_t)NS * (BM + BN) * BK * 2;
-  const dim3 grid((unsigned)(a.grid_m * a.grid_n), (unsigned)(a.k_split > 0 ? (a.K + a.k_split - 1) / a.k_split : 1)),
+  const bool listed = !conv && a.tile_list != nullptr;  // one workgroup per record, no split grid
+  const dim3 grid((unsigned)(listed ? a.tile_count : a.grid_m * a.grid_n),
+                  (unsigned)(!listed && a.k_split > 0 ? (a.K + a.k_split - 1) / a.k_split : 1)),
       block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \

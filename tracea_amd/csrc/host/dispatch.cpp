@@ -5,6 +5,7 @@
 // INVALID_PARAMS; groups/dtype/layout the kernels do not cover ->
 // UNSUPPORTED_CONFIG; host pointers -> CPU_ERROR; HIP failures -> CUDA_ERROR.
 #include "dispatch.hpp"
+#include "tile_graph.hpp"
 
 #include <algorithm>
 #include <atomic>
@@ -644,6 +645,179 @@ TraceaStatus dispatch_gemm_ops(const TraceaTensorView &ta, const TraceaTensorVie
   st = lower_chain("tracea_gemm_ex", ops, n_ops, c.shape[1], c.shape[1], &chain);
   if (st != TRACEA_SUCCESS) return st;
   return run_gemm(a, b, c, chain, (hipStream_t)params.stream);
+}
+
+// ---- GEMM over a tile list ---------------------------------------------------------
+// The tile extents of the layout name the kernel: a compiled variant with that macro-tile
+// runs one workgroup per listed record.  Output tiles without a record are not written.
+// When several records share a tile (a K split written out as records), every tile must
+// have the same number of them: their partial products go to the split-K workspace and
+// the reduction kernel sums them and applies the operator chain.
+TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &ta, const TraceaTensorView &tb,
+                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                 TraceaTensorView *tc, const TraceaGemmParams &params,
+                                 const TraceaEpilogueOp *ops_in, uint32_t n_ops, const TileLayout &layout,
+                                 const DeviceTileTables &tables) {
+  const char *what = "tracea_gemm_ttg";
+  View a, b, c;
+  TraceaStatus st = gemm_common(ta, tb, tc, &a, &b, &c);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  if (ops_in == nullptr) {
+    TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
+    const int n = kind_to_ops((int)params.epilogue, bias, residual, ops);
+    if (n < 0) return fail(TRACEA_INVALID_PARAMS, "%s: unknown epilogue kind %d", what, (int)params.epilogue);
+    st = check_bias_residual(what, bias, residual, c.shape[1], c, c.device, ops, n);
+    if (st != TRACEA_SUCCESS) return st;
+    st = lower_chain(what, ops, (uint32_t)n, c.shape[1], c.shape[1], &chain);
+  } else {
+    st = lower_chain(what, ops_in, n_ops, c.shape[1], c.shape[1], &chain);
+  }
+  if (st != TRACEA_SUCCESS) return st;
+
+  const long long M = a.shape[0], K = a.shape[1], N = b.shape[1];
+  if (M != layout.m || N != layout.n || K != layout.k)
+    return fail(TRACEA_INVALID_PARAMS, "%s: operands are %lldx%lldx%lld, the layout was built for %ux%ux%u", what, M,
+                N, K, layout.m, layout.n, layout.k);
+  t_last_contraction = -1;
+  t_last_splits = 1;
+  if (tables.count == 0) return TRACEA_SUCCESS;  // nothing listed: nothing written
+  if (tables.l1 == nullptr || tables.l2 == nullptr || (tables.slices > 1 && tables.slice == nullptr))
+    return fail(TRACEA_INVALID_PARAMS, "%s: the layout has no tables on device %d", what, c.device);
+
+  const bool a_ok = a.stride[1] == 1 && a.stride[0] % 8 == 0 && K % 8 == 0 && aligned(a.ptr, 16);
+  const bool b_kcontig = b.stride[0] == 1 && b.stride[1] % 8 == 0 && aligned(b.ptr, 16);
+  const bool b_ncontig = b.stride[1] == 1 && b.stride[0] % 8 == 0 && N % 8 == 0 && aligned(b.ptr, 16);
+  if (!(is_half(a.dtype) && b.dtype == a.dtype && a_ok && (b_kcontig || b_ncontig) && c.stride[1] == 1))
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "%s: needs fp16 or bf16 operands of one type, 16-byte aligned, K-contiguous A with K and the row "
+                "stride multiples of 8, B contiguous along K or N, unit column stride of C", what);
+  if (tables.k_gcd % 8 != 0 || tables.start_gcd % 8 != 0)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: every k_start and k range length must be a multiple of 8", what);
+
+  const long long a_extent = ((M - 1) * a.stride[0] + K) * 2;
+  const long long b_extent = b_kcontig ? ((N - 1) * b.stride[1] + K) * 2 : ((K - 1) * b.stride[0] + N) * 2;
+  const bool small = a_extent < (1ll << 31) && b_extent < (1ll << 31);
+  // the variant: forced if its tile fits, else the most pipelined one with this macro-tile
+  int vi = -1;
+  const int forced = forced_variant("gemm");
+  if (forced >= 0 && contraction_variant(forced).pipeline != 4 && contraction_variant(forced).bm == (int)layout.mt &&
+      contraction_variant(forced).bn == (int)layout.nt)
+    vi = forced;
+  static const int rank_of_pipeline[5] = {0, 1, 3, 2, -1};
+  const bool use_forced = vi >= 0;
+  for (int i = 0; !use_forced && i < contraction_variant_count(); ++i) {
+    const ContractionVariant &v = contraction_variant(i);
+    if (v.pipeline == 4 || v.bm != (int)layout.mt || v.bn != (int)layout.nt) continue;
+    if (vi < 0) { vi = i; continue; }
+    const ContractionVariant &best = contraction_variant(vi);
+    const int r = rank_of_pipeline[v.pipeline], rb = rank_of_pipeline[best.pipeline];
+    if (r > rb || (r == rb && v.waves_m * v.waves_n > best.waves_m * best.waves_n)) vi = i;
+  }
+  if (vi < 0)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: no kernel with a %ux%u macro-tile (compiled: 64x64, 128x64, 128x128, "
+                "256x64, 256x128, 256x256)", what, layout.mt, layout.nt);
+  vi = resolve_variant(vi, false, !small, tables.k_gcd % contraction_variant(vi).bk == 0);
+  const ContractionVariant &v = contraction_variant(vi);
+
+  DeviceScope scope(c.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  hipStream_t stream = (hipStream_t)params.stream;
+  ContractionArgs args{};
+  args.A = a.ptr; args.B = b.ptr; args.C = c.ptr;
+  args.M = (int)M; args.N = (int)N; args.K = (int)K;
+  args.lda = a.stride[0];
+  args.ldb = b_kcontig ? b.stride[1] : b.stride[0];
+  args.ldc = c.stride[0];
+  args.out_dtype = c.dtype;
+  args.a_bytes = (unsigned)(small ? a_extent : 0);
+  args.b_bytes = (unsigned)(small ? b_extent : 0);
+  fill_grid(&args, v);
+  args.tile_list = tables.l1;
+  args.tile_records = tables.l2;
+  args.tile_count = (int)tables.count;
+  t_last_contraction = vi;
+  if (tables.slices <= 1) {
+    args.epi = chain;
+    return hip_status("gemm tile-list launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
+  }
+  if ((long long)tables.count != (long long)tables.slices * args.grid_m * args.grid_n)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: records that share a tile are summed only when every tile of the "
+                "grid has the same number of them", what);
+  void *scratch = splitk_scratch(c.device, stream, (size_t)tables.slices * M * N * 4);
+  if (scratch == nullptr)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: %u partial products of %lldx%lld exceed the 64 MiB workspace", what,
+                tables.slices, M, N);
+  t_last_splits = (int)tables.slices;
+  SplitKReduceArgs r{};
+  r.partial = (const float *)scratch;
+  r.out = c.ptr; r.out_dtype = c.dtype;
+  r.splits = (int)tables.slices; r.M = (int)M; r.N = (int)N; r.ldc = c.stride[0];
+  r.epi = chain;
+  args.C = scratch;
+  args.ldc = N;
+  args.out_dtype = DT_F32;
+  args.tile_slice = tables.slice;
+  st = hip_status("gemm tile-list launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
+  if (st != TRACEA_SUCCESS) return st;
+  return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
+}
+
+// ---- low-rank MLP ------------------------------------------------------------------
+// C = chain((X A) B): the rank-r product T = X A is rounded to the operands' type, as the
+// reference's kernel keeps it (half sT, src/emitter/cuda/low_rank.rs:28-31, 86-94), and
+// lives in a stream-ordered allocation for the duration of the call; both products run
+// on the GEMM kernels.
+TraceaStatus dispatch_low_rank_mlp(const TraceaTensorView &tx, const TraceaTensorView &ta,
+                                   const TraceaTensorView &tb, const TraceaTensorView *bias,
+                                   const TraceaTensorView *residual, TraceaTensorView *tc,
+                                   const TraceaGemmParams &params) {
+  const char *what = "tracea_low_rank_mlp";
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "%s: tracea_init has not been called", what);
+  if (tc == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: output view is NULL", what);
+  View x, a, b, c;
+  TraceaStatus st;
+  if ((st = read_view("tracea_low_rank_mlp: x", tx, 2, &x)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_low_rank_mlp: a", ta, 2, &a)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_low_rank_mlp: b", tb, 2, &b)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_low_rank_mlp: c", *tc, 2, &c)) != TRACEA_SUCCESS) return st;
+  if (!is_float_type(x.dtype) || a.dtype != x.dtype || b.dtype != x.dtype || !is_float_type(c.dtype))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: x, a and b must share one floating type (%s, %s, %s)", what,
+                dtype_name(x.dtype), dtype_name(a.dtype), dtype_name(b.dtype));
+  const long long M = x.shape[0], K = x.shape[1], R = a.shape[1], N = b.shape[1];
+  if (a.shape[0] != K || b.shape[0] != R || c.shape[0] != M || c.shape[1] != N)
+    return fail(TRACEA_INVALID_PARAMS, "%s: shapes x[%lld,%lld] a[%lld,%lld] b[%lld,%lld] c[%lld,%lld] do not agree",
+                what, M, K, a.shape[0], R, b.shape[0], N, c.shape[0], c.shape[1]);
+  if ((st = check_device(what, c.device)) != TRACEA_SUCCESS) return st;
+  if (x.device != c.device || a.device != c.device || b.device != c.device)
+    return fail(TRACEA_INVALID_PARAMS, "%s: operands live on different devices", what);
+  if (M >= (1ll << 31) || K >= (1ll << 31) || N >= (1ll << 31) || R >= (1ll << 31))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dimension exceeds 2^31-1", what);
+  TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
+  const int n = kind_to_ops((int)params.epilogue, bias, residual, ops);
+  if (n < 0) return fail(TRACEA_INVALID_PARAMS, "%s: unknown epilogue kind %d", what, (int)params.epilogue);
+  st = check_bias_residual(what, bias, residual, N, c, c.device, ops, n);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain(what, ops, (uint32_t)n, N, N, &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  if (M == 0 || N == 0) return TRACEA_SUCCESS;
+
+  hipStream_t stream = (hipStream_t)params.stream;
+  DeviceScope scope(c.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  const long long ldt = (R + 7) / 8 * 8;  // rows of T start 16-byte aligned
+  void *t_mem = nullptr;
+  hipError_t e = hipMallocAsync(&t_mem, (size_t)std::max(1ll, M * ldt) * elem_size(x.dtype), stream);
+  if (e != hipSuccess) return hip_status("tracea_low_rank_mlp: workspace allocation", (int)e);
+  View t{};
+  t.ptr = t_mem; t.dtype = x.dtype; t.device = c.device; t.rank = 2;
+  t.shape[0] = M; t.shape[1] = R; t.stride[0] = ldt; t.stride[1] = 1;
+  st = run_gemm(x, a, t, EpilogueChain{}, stream);
+  if (st == TRACEA_SUCCESS) st = run_gemm(t, b, c, chain, stream);
+  e = hipFreeAsync(t_mem, stream);
+  if (st == TRACEA_SUCCESS && e != hipSuccess) st = hip_status("tracea_low_rank_mlp: workspace release", (int)e);
+  return st;
 }
 
 // ---- Conv2d ----------------------------------------------------------------------

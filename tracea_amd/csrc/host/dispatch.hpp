@@ -44,6 +44,29 @@ TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorVie
 TraceaStatus dispatch_gemm_ops(const TraceaTensorView &a, const TraceaTensorView &b,
                                TraceaTensorView *c, const TraceaGemmParams &params,
                                const TraceaEpilogueOp *ops, uint32_t n_ops);
+// GEMM over a tile list.  `tables` are the device copies of a TileLayout's tables on the
+// device of c: level-1 map in launch order, records, and (slices > 1 only) the workspace
+// row block of every workgroup.  Exactly one of (ops, n_ops) and the kind in params is used:
+// ops == nullptr selects the kind.
+struct TileLayout;
+struct DeviceTileTables {
+  const unsigned *l1 = nullptr;
+  const unsigned *l2 = nullptr;
+  const unsigned *slice = nullptr;
+  uint32_t count = 0;   // workgroups
+  uint32_t slices = 1;  // records per tile (all tiles alike when > 1)
+  uint32_t k_gcd = 0;      // gcd of the k range lengths (k_end clipped to K) of all listed records
+  uint32_t start_gcd = 0;  // gcd of their k_start (0: all start at 0)
+};
+TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &a, const TraceaTensorView &b,
+                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
+                                 TraceaTensorView *c, const TraceaGemmParams &params,
+                                 const TraceaEpilogueOp *ops, uint32_t n_ops, const TileLayout &layout,
+                                 const DeviceTileTables &tables);
+TraceaStatus dispatch_low_rank_mlp(const TraceaTensorView &x, const TraceaTensorView &a,
+                                   const TraceaTensorView &b, const TraceaTensorView *bias,
+                                   const TraceaTensorView *residual, TraceaTensorView *c,
+                                   const TraceaGemmParams &params);
 TraceaStatus dispatch_conv2d_kind(const TraceaTensorView &x, const TraceaTensorView &w,
                                   const TraceaTensorView *bias, const TraceaTensorView *residual,
                                   TraceaTensorView *out, const TraceaConv2dParams &params);

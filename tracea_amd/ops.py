@@ -66,6 +66,23 @@ def gemm(a, b, out=None, bias=None, residual=None, epilogue="none", out_dtype=No
     return out
 
 
+def low_rank_mlp(x, a, b, out=None, bias=None, residual=None, epilogue="none", out_dtype=None):
+    """out[M,N] = epilogue((x[M,K] @ a[K,R]) @ b[R,N]); the rank-R product is rounded to the
+    operands' type in between (the reference's LowRankMlp operator)."""
+    m, _ = x.shape
+    _, n = b.shape
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype or x.dtype, device=x.device)
+    vx, va, vb, vc = _view(x), _view(a), _view(b), _view(out)
+    vbias = _view(bias) if bias is not None else None
+    vres = _view(residual) if residual is not None else None
+    params = capi.GemmParams(parse_epilogue(epilogue), _stream(x))
+    st = capi.lib().tracea_low_rank_mlp(vx.c, va.c, vb.c, C.byref(vbias.c) if vbias else None,
+                                        C.byref(vres.c) if vres else None, C.byref(vc.c), params)
+    capi.check("tracea_low_rank_mlp", st)
+    return out
+
+
 def _ops_array(ops):
     """[(kind, tensors..., [eps])] -> (EpilogueOp array, keep-alive list)."""
     arr = (capi.EpilogueOp * max(1, len(ops)))()
