@@ -112,6 +112,21 @@ def make_workload(name, torch, ops):
         plan.capture()
         return ("fp16 ResNet-18 forward, batch %d, 224x224, %d fused launches replayed as one HIP graph"
                 % (batch, len(plan.describe()["steps"])), flops, 0.0, "f16", plan.replay)
+    if name == "gemm_tiles_half":
+        # the headline product restricted to a random half of its 128x128 output tiles through a tile
+        # list (the reference's examples/ttg_sparse_experiment.rs at full size); FLOPs count listed tiles
+        # only.  (With 256x256 tiles half of the list is 124 workgroups for 256 CUs and takes as long as one
+        # tile's walk over K, 96 us.)
+        from tracea_amd.ttg import TileLayout, gemm_ttg
+        m = n = k = 4096
+        a = (torch.randn(m, k, device=dev, generator=g) / k ** 0.5).half()
+        bt = (torch.randn(n, k, device=dev, generator=g) / k ** 0.5).half()
+        c = torch.zeros(m, n, device=dev, dtype=torch.float16)
+        lay = TileLayout.from_random(m, n, k, 128, 128, 64, 0.5, seed=11)
+        tiles = lay.num_active_tiles
+        return ("fp16 GEMM 4096x4096x4096 over a tile list: %d of 1024 tiles of 128x128" % tiles,
+                2.0 * tiles * 128 * 128 * k, 2.0 * (m * k + k * n + tiles * 128 * 128), "f16",
+                lambda: gemm_ttg(a, bt.t(), lay, c))
     if name == "copy":
         # calibration workload for the HBM traffic counters: a plain device copy of known size
         n = 256 << 20
@@ -197,7 +212,7 @@ def main():
     if not args.no_extras:
         also = {}
         for name in ("gemm", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "attention", "attention_causal", "conv_transpose", "resnet18_b1",
-                     "resnet18_b32"):
+                     "resnet18_b32", "gemm_tiles_half"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)
