@@ -267,6 +267,30 @@ TraceaStatus tracea_conv_transpose2d_ex(TraceaTensorView x, TraceaTensorView w, 
                                         TraceaConvTranspose2dParams params,
                                         const TraceaEpilogueOp *ops, uint32_t n_ops);
 
+/* ---- Operators that are not contractions: the reference's Softmax, BatchNorm,
+ * GlobalAveragePool and Linear kernels (src/emitter/cuda/nn.rs:3-135) and its
+ * element-wise ReLU / Add nodes.  Activations are contiguous with the channel
+ * axis last (NHWC), the layout of every other entry point here; the reference's
+ * BatchNorm and pooling kernels index NCHW, and a tensor strided that way is
+ * TRACEA_UNSUPPORTED_CONFIG.  Storage may be f32, f16 or bf16 (in and out
+ * independently); arithmetic is fp32.  `stream` is a hipStream_t (NULL: default).
+ *
+ * tracea_apply_epilogue: out = chain(x) in one pass; x and out of equal shape, rank 1-4.
+ *   Standalone BatchNorm is {TRACEA_EPI_OP_BATCHNORM, p0..p3 = gamma, beta, mean, var (f32), epsilon}:
+ *   (x - mean) * rsqrt(var + eps) * gamma + beta (nn.rs:56-66); ReLU and a residual Add likewise.
+ * tracea_softmax: over the last axis, max-subtracted (nn.rs:14-32).
+ * tracea_global_avg_pool: x [N,H,W,C] -> out [N,C], the mean over H*W (nn.rs:84-97).
+ * tracea_linear: c[b] = epilogue(a[b] w[b]) with a [B,M,K], c [B,M,N] and w [B,K,N] (nn.rs:113-131)
+ *   or a shared w [K,N]; any strides within a batch as for tracea_gemm; epilogue kinds without a
+ *   residual. */
+TraceaStatus tracea_apply_epilogue(TraceaTensorView x, TraceaTensorView *out, const TraceaEpilogueOp *ops,
+                                   uint32_t n_ops, void *stream);
+TraceaStatus tracea_softmax(TraceaTensorView x, TraceaTensorView *out, void *stream);
+TraceaStatus tracea_global_avg_pool(TraceaTensorView x, TraceaTensorView *out, void *stream);
+TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaTensorView *bias, TraceaTensorView *c,
+                           TraceaGemmParams params);
+
+
 /* Split-K.  A gemm / conv2d launch with few output tiles and a long K (tiles * 2 <= 256 CUs,
  * at least 8 K tiles) is split along K over more workgroups; fp32 partial products go to a
  * scratch buffer the library keeps per (device, stream) (grown on demand up to 64 MiB, never

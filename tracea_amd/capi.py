@@ -104,6 +104,11 @@ SIGNATURES = {
     "tracea_plan_output": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "tracea_plan_bind": (C.c_int, [C.c_void_p, C.c_uint64, C.c_char_p, C.c_void_p]),
     "tracea_plan_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
+    "tracea_apply_epilogue": (C.c_int, [TensorView, C.POINTER(TensorView), C.POINTER(EpilogueOp), C.c_uint32,
+                                        C.c_void_p]),
+    "tracea_softmax": (C.c_int, [TensorView, C.POINTER(TensorView), C.c_void_p]),
+    "tracea_global_avg_pool": (C.c_int, [TensorView, C.POINTER(TensorView), C.c_void_p]),
+    "tracea_linear": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), C.POINTER(TensorView), GemmParams]),
     "tracea_low_rank_mlp": (C.c_int, [TensorView, TensorView, TensorView, C.POINTER(TensorView),
                                       C.POINTER(TensorView), C.POINTER(TensorView), GemmParams]),
     "tracea_ttg_from_dense": (C.c_void_p, [C.c_uint32] * 6),

@@ -96,6 +96,24 @@ TraceaStatus tracea_gemm_ex(TraceaTensorView a, TraceaTensorView b, TraceaTensor
   TRACEA_GUARDED(dispatch_gemm_ops(a, b, c, params, ops, n_ops))
 }
 
+TraceaStatus tracea_apply_epilogue(TraceaTensorView x, TraceaTensorView *out, const TraceaEpilogueOp *ops,
+                                   uint32_t n_ops, void *stream) {
+  TRACEA_GUARDED(dispatch_apply_epilogue(x, out, ops, n_ops, stream))
+}
+
+TraceaStatus tracea_softmax(TraceaTensorView x, TraceaTensorView *out, void *stream) {
+  TRACEA_GUARDED(dispatch_softmax(x, out, stream))
+}
+
+TraceaStatus tracea_global_avg_pool(TraceaTensorView x, TraceaTensorView *out, void *stream) {
+  TRACEA_GUARDED(dispatch_global_avg_pool(x, out, stream))
+}
+
+TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaTensorView *bias, TraceaTensorView *c,
+                           TraceaGemmParams params) {
+  TRACEA_GUARDED(dispatch_linear(a, w, bias, c, params))
+}
+
 TraceaStatus tracea_low_rank_mlp(TraceaTensorView x, TraceaTensorView a, TraceaTensorView b,
                                  const TraceaTensorView *bias, const TraceaTensorView *residual,
                                  TraceaTensorView *c, TraceaGemmParams params) {

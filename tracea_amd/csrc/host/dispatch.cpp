@@ -820,6 +820,173 @@ TraceaStatus dispatch_low_rank_mlp(const TraceaTensorView &tx, const TraceaTenso
   return st;
 }
 
+// ---- operators that are not contractions (src/emitter/cuda/nn.rs:3-135) -------------
+namespace {
+
+// A contiguous tensor whose last axis is the channel axis: rows x channels.
+TraceaStatus rows_by_channels(const char *what, const TraceaTensorView &t, long long *rows, long long *channels,
+                              View *v) {
+  if (t.rank < 1 || t.rank > 4) return fail(TRACEA_INVALID_PARAMS, "%s: rank %u, expected 1 to 4", what, t.rank);
+  TraceaStatus st = read_view(what, t, (int)t.rank, v);
+  if (st != TRACEA_SUCCESS) return st;
+  if (!is_float_type(v->dtype)) return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dtype %s unsupported", what, dtype_name(v->dtype));
+  long long expect = 1, r = 1;
+  for (int i = v->rank - 1; i >= 0; --i) {
+    if (v->shape[i] > 1 && v->stride[i] != expect)
+      return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: the tensor must be contiguous with the channel axis last "
+                  "(NHWC); axis %d has stride %lld, expected %lld", what, i, v->stride[i], expect);
+    expect *= v->shape[i];
+    if (i < v->rank - 1) r *= v->shape[i];
+  }
+  *rows = r;
+  *channels = v->shape[v->rank - 1];
+  if (*channels >= (1ll << 31)) return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: more than 2^31-1 channels", what);
+  return TRACEA_SUCCESS;
+}
+
+bool same_shape(const View &a, const View &b) {
+  if (a.rank != b.rank) return false;
+  for (int i = 0; i < a.rank; ++i)
+    if (a.shape[i] != b.shape[i]) return false;
+  return true;
+}
+
+}  // namespace
+
+// out = chain(x), element by element with per-channel operands: standalone BatchNorm
+// (nn.rs:37-70, channel axis last here), ReLU, bias, residual Add as one pass over the tensor.
+TraceaStatus dispatch_apply_epilogue(const TraceaTensorView &tx, TraceaTensorView *tout, const TraceaEpilogueOp *ops,
+                                     uint32_t n_ops, void *stream) {
+  const char *what = "tracea_apply_epilogue";
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "%s: tracea_init has not been called", what);
+  if (tout == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: output view is NULL", what);
+  View x, out;
+  long long rows, channels, orows, ochannels;
+  TraceaStatus st;
+  if ((st = rows_by_channels("tracea_apply_epilogue: x", tx, &rows, &channels, &x)) != TRACEA_SUCCESS) return st;
+  if ((st = rows_by_channels("tracea_apply_epilogue: out", *tout, &orows, &ochannels, &out)) != TRACEA_SUCCESS) return st;
+  if (!same_shape(x, out)) return fail(TRACEA_INVALID_PARAMS, "%s: x and out differ in shape", what);
+  if ((st = check_device(what, out.device)) != TRACEA_SUCCESS) return st;
+  if (x.device != out.device) return fail(TRACEA_INVALID_PARAMS, "%s: operands live on different devices", what);
+  ChainApplyArgs a{};
+  st = lower_chain(what, ops, n_ops, channels, channels, &a.epi);
+  if (st != TRACEA_SUCCESS) return st;
+  a.x = x.ptr; a.out = out.ptr;
+  a.x_dtype = x.dtype; a.out_dtype = out.dtype;
+  a.rows = rows; a.channels = (int)channels;
+  DeviceScope scope(out.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  return hip_status("operator chain launch", launch_chain_apply(a, (hipStream_t)stream));
+}
+
+// Softmax over the last axis (nn.rs:3-35), fp32 arithmetic whatever the storage type.
+TraceaStatus dispatch_softmax(const TraceaTensorView &tx, TraceaTensorView *tout, void *stream) {
+  const char *what = "tracea_softmax";
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "%s: tracea_init has not been called", what);
+  if (tout == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: output view is NULL", what);
+  View x, out;
+  long long rows, cols, orows, ocols;
+  TraceaStatus st;
+  if ((st = rows_by_channels("tracea_softmax: x", tx, &rows, &cols, &x)) != TRACEA_SUCCESS) return st;
+  if ((st = rows_by_channels("tracea_softmax: out", *tout, &orows, &ocols, &out)) != TRACEA_SUCCESS) return st;
+  if (!same_shape(x, out)) return fail(TRACEA_INVALID_PARAMS, "%s: x and out differ in shape", what);
+  if ((st = check_device(what, out.device)) != TRACEA_SUCCESS) return st;
+  if (x.device != out.device) return fail(TRACEA_INVALID_PARAMS, "%s: operands live on different devices", what);
+  DeviceScope scope(out.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  return hip_status("softmax launch",
+                    launch_softmax_rows(x.ptr, out.ptr, x.dtype, out.dtype, rows, (int)cols, (hipStream_t)stream));
+}
+
+// out[n, c] = mean over (h, w) of x[n, h, w, c] (nn.rs:72-100; the reference indexes NCHW).
+TraceaStatus dispatch_global_avg_pool(const TraceaTensorView &tx, TraceaTensorView *tout, void *stream) {
+  const char *what = "tracea_global_avg_pool";
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "%s: tracea_init has not been called", what);
+  if (tout == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: output view is NULL", what);
+  if (tx.rank != 4 || tout->rank != 2)
+    return fail(TRACEA_INVALID_PARAMS, "%s: x must be [N,H,W,C] and out [N,C]", what);
+  View x, out;
+  long long rows, channels, orows, ochannels;
+  TraceaStatus st;
+  if ((st = rows_by_channels("tracea_global_avg_pool: x", tx, &rows, &channels, &x)) != TRACEA_SUCCESS) return st;
+  if ((st = rows_by_channels("tracea_global_avg_pool: out", *tout, &orows, &ochannels, &out)) != TRACEA_SUCCESS) return st;
+  if (out.shape[0] != x.shape[0] || ochannels != channels)
+    return fail(TRACEA_INVALID_PARAMS, "%s: out is [%lld,%lld], expected [%lld,%lld]", what, out.shape[0], ochannels,
+                x.shape[0], channels);
+  if ((st = check_device(what, out.device)) != TRACEA_SUCCESS) return st;
+  if (x.device != out.device) return fail(TRACEA_INVALID_PARAMS, "%s: operands live on different devices", what);
+  const long long hw = x.shape[1] * x.shape[2];
+  if (x.shape[0] > 65535 || hw >= (1ll << 31))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: batch above 65535 or more than 2^31-1 pixels", what);
+  if (hw == 0) return fail(TRACEA_INVALID_PARAMS, "%s: empty spatial extent", what);
+  DeviceScope scope(out.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  return hip_status("global average pool launch",
+                    launch_global_avg_pool(x.ptr, out.ptr, x.dtype, out.dtype, (int)x.shape[0], (int)hw, (int)channels,
+                                           (hipStream_t)stream));
+}
+
+// c[b] = epilogue(a[b] w[b]) for every batch b (nn.rs:102-135: A [B,M,K], B [B,K,N], C [B,M,N]);
+// a weight of rank 2 is shared by all batches, and the batch then folds into the rows.
+TraceaStatus dispatch_linear(const TraceaTensorView &ta, const TraceaTensorView &tw, const TraceaTensorView *bias,
+                             TraceaTensorView *tc, const TraceaGemmParams &params) {
+  const char *what = "tracea_linear";
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "%s: tracea_init has not been called", what);
+  if (tc == nullptr) return fail(TRACEA_INVALID_PARAMS, "%s: output view is NULL", what);
+  if (ta.rank != 3 || tc->rank != 3 || (tw.rank != 2 && tw.rank != 3))
+    return fail(TRACEA_INVALID_PARAMS, "%s: a and c must have rank 3 ([B,M,K], [B,M,N]), w rank 2 or 3", what);
+  View a, w, c;
+  TraceaStatus st;
+  if ((st = read_view("tracea_linear: a", ta, 3, &a)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_linear: w", tw, (int)tw.rank, &w)) != TRACEA_SUCCESS) return st;
+  if ((st = read_view("tracea_linear: c", *tc, 3, &c)) != TRACEA_SUCCESS) return st;
+  const long long B = a.shape[0], M = a.shape[1], K = a.shape[2];
+  const bool shared = w.rank == 2;
+  const long long wk = w.shape[w.rank - 2], N = w.shape[w.rank - 1];
+  if (wk != K || c.shape[0] != B || c.shape[1] != M || c.shape[2] != N || (!shared && w.shape[0] != B))
+    return fail(TRACEA_INVALID_PARAMS, "%s: shapes a[%lld,%lld,%lld], w[..,%lld,%lld], c[%lld,%lld,%lld] do not agree",
+                what, B, M, K, wk, N, c.shape[0], c.shape[1], c.shape[2]);
+  if (!is_float_type(a.dtype) || !is_float_type(w.dtype) || !is_float_type(c.dtype))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dtypes %s x %s -> %s unsupported", what, dtype_name(a.dtype),
+                dtype_name(w.dtype), dtype_name(c.dtype));
+  if ((st = check_device(what, c.device)) != TRACEA_SUCCESS) return st;
+  if (a.device != c.device || w.device != c.device)
+    return fail(TRACEA_INVALID_PARAMS, "%s: operands live on different devices", what);
+  if (M >= (1ll << 31) || K >= (1ll << 31) || N >= (1ll << 31) || B * M >= (1ll << 31))
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: dimension exceeds 2^31-1", what);
+  if (params.epilogue == TRACEA_EPILOGUE_RESIDUAL || params.epilogue == TRACEA_EPILOGUE_RESIDUAL_RELU)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: residual epilogues are not defined for a batched product", what);
+  TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
+  const int n = kind_to_ops((int)params.epilogue, bias, nullptr, ops);
+  if (n < 0) return fail(TRACEA_INVALID_PARAMS, "%s: unknown epilogue kind %d", what, (int)params.epilogue);
+  View c2{};
+  c2.ptr = c.ptr; c2.rank = 2; c2.dtype = c.dtype; c2.device = c.device;
+  c2.shape[0] = M; c2.shape[1] = N; c2.stride[0] = c.stride[1]; c2.stride[1] = c.stride[2];
+  st = check_bias_residual(what, bias, nullptr, N, c2, c.device, ops, n);
+  if (st != TRACEA_SUCCESS) return st;
+  EpilogueChain chain{};
+  st = lower_chain(what, ops, (uint32_t)n, N, N, &chain);
+  if (st != TRACEA_SUCCESS) return st;
+  hipStream_t stream = (hipStream_t)params.stream;
+  View a2 = c2, w2 = c2;
+  a2.ptr = a.ptr; a2.dtype = a.dtype; a2.shape[0] = M; a2.shape[1] = K; a2.stride[0] = a.stride[1]; a2.stride[1] = a.stride[2];
+  w2.ptr = w.ptr; w2.dtype = w.dtype; w2.shape[0] = K; w2.shape[1] = N;
+  w2.stride[0] = w.stride[w.rank - 2]; w2.stride[1] = w.stride[w.rank - 1];
+  // one launch when the weight is shared and the batches of a and c are evenly spaced rows
+  if (shared && (B <= 1 || (a.stride[0] == M * a.stride[1] && c.stride[0] == M * c.stride[1]))) {
+    a2.shape[0] = c2.shape[0] = B * M;
+    return run_gemm(a2, w2, c2, chain, stream);
+  }
+  for (long long b = 0; b < B; ++b) {
+    View ab = a2, wb = w2, cb = c2;
+    ab.ptr = (char *)a.ptr + b * a.stride[0] * elem_size(a.dtype);
+    cb.ptr = (char *)c.ptr + b * c.stride[0] * elem_size(c.dtype);
+    if (!shared) wb.ptr = (char *)w.ptr + b * w.stride[0] * elem_size(w.dtype);
+    if ((st = run_gemm(ab, wb, cb, chain, stream)) != TRACEA_SUCCESS) return st;
+  }
+  return TRACEA_SUCCESS;
+}
+
 // ---- Conv2d ----------------------------------------------------------------------
 namespace {
 

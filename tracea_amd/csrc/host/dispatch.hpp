@@ -63,6 +63,12 @@ TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &a, const TraceaTensorVi
                                  TraceaTensorView *c, const TraceaGemmParams &params,
                                  const TraceaEpilogueOp *ops, uint32_t n_ops, const TileLayout &layout,
                                  const DeviceTileTables &tables);
+TraceaStatus dispatch_apply_epilogue(const TraceaTensorView &x, TraceaTensorView *out, const TraceaEpilogueOp *ops,
+                                     uint32_t n_ops, void *stream);
+TraceaStatus dispatch_softmax(const TraceaTensorView &x, TraceaTensorView *out, void *stream);
+TraceaStatus dispatch_global_avg_pool(const TraceaTensorView &x, TraceaTensorView *out, void *stream);
+TraceaStatus dispatch_linear(const TraceaTensorView &a, const TraceaTensorView &w, const TraceaTensorView *bias,
+                             TraceaTensorView *c, const TraceaGemmParams &params);
 TraceaStatus dispatch_low_rank_mlp(const TraceaTensorView &x, const TraceaTensorView &a,
                                    const TraceaTensorView &b, const TraceaTensorView *bias,
                                    const TraceaTensorView *residual, TraceaTensorView *c,

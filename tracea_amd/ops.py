@@ -83,6 +83,55 @@ def low_rank_mlp(x, a, b, out=None, bias=None, residual=None, epilogue="none", o
     return out
 
 
+def apply_epilogue(x, ops, out=None, out_dtype=None):
+    """out = chain(x) in one pass over a channels-last tensor, e.g. standalone BatchNorm
+    [(OP_BATCHNORM, gamma, beta, mean, var, eps)], ReLU [(OP_RELU,)], Add [(OP_RESIDUAL_ADD, other)]."""
+    if out is None:
+        out = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    arr, _keep = _ops_array(ops)
+    vx, vo = _view(x), _view(out)
+    st = capi.lib().tracea_apply_epilogue(vx.c, C.byref(vo.c), arr, len(ops), _stream(x))
+    capi.check("tracea_apply_epilogue", st)
+    return out
+
+
+def batchnorm(x, gamma, beta, mean, var, eps=1e-5, out=None):
+    """Inference BatchNorm over the last (channel) axis."""
+    return apply_epilogue(x, [(capi.OP_BATCHNORM, gamma, beta, mean, var, eps)], out=out)
+
+
+def softmax(x, out=None, out_dtype=None):
+    """Softmax over the last axis."""
+    if out is None:
+        out = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    vx, vo = _view(x), _view(out)
+    capi.check("tracea_softmax", capi.lib().tracea_softmax(vx.c, C.byref(vo.c), _stream(x)))
+    return out
+
+
+def global_avg_pool(x, out=None, out_dtype=None):
+    """x [N,H,W,C] -> [N,C]."""
+    if out is None:
+        out = torch.empty((x.shape[0], x.shape[3]), dtype=out_dtype or x.dtype, device=x.device)
+    vx, vo = _view(x), _view(out)
+    capi.check("tracea_global_avg_pool", capi.lib().tracea_global_avg_pool(vx.c, C.byref(vo.c), _stream(x)))
+    return out
+
+
+def linear(a, w, bias=None, epilogue=None, out=None, out_dtype=None):
+    """c[b] = epilogue(a[b] @ w[b]); a [B,M,K], w [B,K,N] or [K,N]."""
+    if out is None:
+        out = torch.empty((a.shape[0], a.shape[1], w.shape[-1]), dtype=out_dtype or a.dtype, device=a.device)
+    if epilogue is None:
+        epilogue = "bias" if bias is not None else "none"
+    va, vw, vc = _view(a), _view(w), _view(out)
+    vbias = _view(bias) if bias is not None else None
+    params = capi.GemmParams(parse_epilogue(epilogue), _stream(a))
+    st = capi.lib().tracea_linear(va.c, vw.c, C.byref(vbias.c) if vbias else None, C.byref(vc.c), params)
+    capi.check("tracea_linear", st)
+    return out
+
+
 def _ops_array(ops):
     """[(kind, tensors..., [eps])] -> (EpilogueOp array, keep-alive list)."""
     arr = (capi.EpilogueOp * max(1, len(ops)))()
