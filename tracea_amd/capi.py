@@ -238,14 +238,19 @@ def init():
         raise RuntimeError("tracea_init failed: " + last_error())
 
 
+_SHAPE_TYPES = [C.c_uint64 * n for n in range(9)]
+_STRIDE_TYPES = [C.c_int64 * n for n in range(9)]
+
+
 class View:
     """Owns the shape/stride arrays a TraceaTensorView borrows."""
+    __slots__ = ("_shape", "_stride", "c")
 
     def __init__(self, ptr, shape, stride, dtype, device_id):
-        self._shape = (C.c_uint64 * len(shape))(*shape)
-        self._stride = (C.c_int64 * len(stride))(*stride) if stride is not None else None
-        self.c = TensorView(ptr, len(shape), self._shape,
-                            self._stride if stride is not None else None, dtype, device_id)
+        n = len(shape)
+        self._shape = _SHAPE_TYPES[n](*shape)
+        self._stride = _STRIDE_TYPES[n](*stride) if stride is not None else None
+        self.c = TensorView(ptr, n, self._shape, self._stride, dtype, device_id)
 
 
 def take_result(res):

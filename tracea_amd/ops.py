@@ -17,14 +17,29 @@ _DTYPES = {torch.float32: capi.F32, torch.float16: capi.F16, torch.bfloat16: cap
            torch.int32: capi.I32, torch.int8: capi.I8}
 
 
+_VIEW_CACHE = {}
+
+
 def _view(t, shape=None, stride=None):
-    if t.dtype not in _DTYPES:
-        raise TypeError("unsupported dtype %s" % t.dtype)
-    dev = t.device.index if t.is_cuda else -1
-    if t.is_cuda and dev is None:
-        dev = torch.cuda.current_device()
-    return capi.View(t.data_ptr(), list(shape if shape is not None else t.shape),
-                     list(stride if stride is not None else t.stride()), _DTYPES[t.dtype], dev)
+    """TraceaTensorView of a tensor.  Building the ctypes structure costs 2-3 us, four or five
+    times per call, more than the library's own dispatch: views are kept by (address, extents,
+    strides, type, device), which a loop over the same tensors hits every time.  A view holds no
+    reference to the tensor, so a stale entry is only a few hundred bytes."""
+    if shape is None:
+        shape = t.shape
+    if stride is None:
+        stride = t.stride()
+    key = (t.data_ptr(), shape, stride, t.dtype, t.get_device())
+    v = _VIEW_CACHE.get(key)
+    if v is None:
+        dtype = _DTYPES.get(t.dtype)
+        if dtype is None:
+            raise TypeError("unsupported dtype %s" % t.dtype)
+        if len(_VIEW_CACHE) >= 1024:
+            _VIEW_CACHE.clear()
+        # get_device(): the device index of a GPU tensor, -1 for a host tensor (which the library rejects)
+        v = _VIEW_CACHE[key] = capi.View(key[0], shape, stride, dtype, key[4])
+    return v
 
 
 def _stream(t):
@@ -194,8 +209,8 @@ def conv2d(x, w, bias=None, residual=None, stride=1, padding=0, dilation=1, epil
     """x [N,H,W,C] (NHWC); w [K,R,S,C] ('krsc') or [R,S,C,K] ('rsck'); out [N,Ho,Wo,K]."""
     stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
     vw = _weight_view(w, weight_layout)
-    wshape = tuple(vw.c.shape[i] for i in range(4))
     if out is None:
+        wshape = tuple(vw.c.shape[i] for i in range(4))
         out = torch.empty(conv_out_shape(x.shape, wshape, stride, padding, dilation),
                           dtype=out_dtype or x.dtype, device=x.device)
     vx, vo = _view(x), _view(out)
@@ -214,8 +229,8 @@ def conv2d_ex(x, w, ops, stride=1, padding=0, dilation=1, out=None, weight_layou
     """Convolution with an explicit operator chain (BatchNorm, scale/shift, ...)."""
     stride, padding, dilation = _pair(stride), _pair(padding), _pair(dilation)
     vw = _weight_view(w, weight_layout)
-    wshape = tuple(vw.c.shape[i] for i in range(4))
     if out is None:
+        wshape = tuple(vw.c.shape[i] for i in range(4))
         out = torch.empty(conv_out_shape(x.shape, wshape, stride, padding, dilation),
                           dtype=out_dtype or x.dtype, device=x.device)
     vx, vo = _view(x), _view(out)
