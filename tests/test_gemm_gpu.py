@@ -182,3 +182,35 @@ def test_error_paths(tracea_gpu):
     tv = capi.TensorView(None, 2, shape, None, capi.F16, 0)
     st = capi.lib().tracea_gemm(tv, tv, None, None, C.byref(tv), capi.GemmParams(0, None))
     assert st == capi.INVALID_PARAMS
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+def test_operand_beyond_2gib_takes_the_register_staged_kernels(tracea_gpu, dtype):
+    # the direct-to-LDS kernels address operands with 32-bit byte offsets; an A whose rows are spread
+    # over more than 2 GiB must run on the kernels that form 64-bit addresses, with the same results
+    from tracea_amd import capi
+    m, n, k = 130, 200, 192
+    tdt = torch.float32 if dtype == "f32" else torch.float16
+    lda = (2 ** 31 // (m - 1)) // tdt.itemsize + 64          # (m-1)*lda*itemsize just above 2 GiB
+    lda -= lda % 8
+    buf = torch.empty((m - 1) * lda + k, dtype=tdt, device="cuda")
+    a_view = buf.as_strided((m, k), (lda, 1))
+    assert ((m - 1) * lda + k) * tdt.itemsize >= 2 ** 31
+    rng = np.random.default_rng(77)
+    a = (rng.standard_normal((m, k)) / np.sqrt(k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    if dtype == "f16":
+        a, b = round_f16(a), round_f16(b)
+    a_view.copy_(_dev(a, tdt))
+    bias = rng.standard_normal(n).astype(np.float32)
+    got = tracea_gpu.gemm(a_view, _dev(b, tdt), bias=_dev(bias), epilogue="bias+relu").float().cpu().numpy()
+    ref = np.maximum(oracle.gemm_f64(a, b) + bias[None, :], 0.0)
+    if dtype == "f32":
+        assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+    else:
+        name = capi.last_variant("gemm")
+        assert "_p2" not in name and "_p3" not in name, name
+        assert_close_scaled(got, ref, tol_half(k, "f16"), "A beyond 2 GiB")
+    # the same product from a compact copy of A runs the direct-to-LDS kernels and agrees
+    compact = tracea_gpu.gemm(a_view.contiguous(), _dev(b, tdt), bias=_dev(bias), epilogue="bias+relu").float().cpu().numpy()
+    np.testing.assert_allclose(got, compact, rtol=0, atol=2e-3 if dtype == "f16" else 1e-5)

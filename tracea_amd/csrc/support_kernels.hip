@@ -17,6 +17,52 @@ namespace tracea_amd {
 // ---------------------------------------------------------------------------
 constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16, F32_PITCH = 132;
 
+// Epilogue of the 128x128 fp32 tile kernels.  Operands were swapped in the MFMAs: a lane owns
+// row (lane&31), channels 8g + 4*(lane>>5) + 0..3 of each 32x32 block of its wave's 64x64 tile.
+// The accumulators go through LDS, ROWS rows at a time (`stage` is ROWS x 64 floats private to
+// the wave), and a rolled loop takes them from there row by row.  Applying the operator chain
+// to the accumulators in place needs compile-time indices, i.e. sixteen copies of the chain
+// code, and with them the compiler copied the chain description from the kernel arguments to
+// scratch memory (488 bytes per lane) and kept 192 registers: 1024^3 took 46.6 us that way and
+// takes 32.9 us this way, 4096^3 1194 -> 979 us.
+template <int ROWS>
+__device__ __forceinline__ void f32_tile_epilogue(const f32x16 (&acc)[2][2], float *stage, const ContractionArgs &args,
+                                                  int m_wave, int n_wave, long long zrow, int lane) {
+  static_assert(ROWS == 32 || ROWS == 16, "a 32-row block is staged whole or in two halves");
+  const int lrow = lane & 31, lhalf = lane >> 5;
+  const int er = lane >> 4, lc = lane & 15;  // reader: 4 rows per step, 16 lanes x 4 channels per row
+  const int M = args.M, N = args.N;
+  static_for<0, 2 * (32 / ROWS)>([&](auto blk) {
+    constexpr int i = decltype(blk)::value / (32 / ROWS), part = decltype(blk)::value % (32 / ROWS);
+    if (ROWS == 32 || (lrow / ROWS) == part) {
+      const int srow = lrow % ROWS;
+#pragma unroll
+      for (int jj = 0; jj < 2; ++jj)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = {acc[i][jj][g * 4 + 0], acc[i][jj][g * 4 + 1], acc[i][jj][g * 4 + 2], acc[i][jj][g * 4 + 3]};
+          const int chunk = jj * 8 + g * 2 + lhalf;  // 16-byte chunk of the row, XOR-ed with the row against bank conflicts
+          *(f32x4 *)(stage + srow * 64 + ((chunk ^ (srow & 15)) << 2)) = v;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+#pragma nounroll
+    for (int r = er; r < ROWS; r += 4) {
+      const int m = m_wave + i * 32 + part * ROWS + r;
+      const int n = n_wave + lc * 4;
+      if (m < M && n < N) {
+        const f32x4 t = *(const f32x4 *)(stage + r * 64 + ((lc ^ (r & 15)) << 2));
+        float v[4] = {t[0], t[1], t[2], t[3]};
+        apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
+        store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  });
+}
+
 __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs args) {
   __shared__ float As[F32_BK][F32_PITCH];
   __shared__ float Bs[F32_BK][F32_PITCH];
@@ -99,19 +145,9 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
     __syncthreads();
   }
 
-  // operands were swapped: lane owns row (lane&31), channels 8g + 4*(lane>>5) + 0..3
-  // (compile-time indices: the body is large enough for the compiler to leave a plain loop
-  // rolled, and a run-time index into the accumulators moves them to scratch memory)
-  static_for<0, 16>([&](auto idx) {
-    constexpr int i = decltype(idx)::value >> 3, j = (decltype(idx)::value >> 2) & 1, g = decltype(idx)::value & 3;
-    const int m = m0 + wm * 64 + i * 32 + lrow;
-    const int n = n0 + wn * 64 + j * 32 + g * 8 + lhalf * 4;
-    if (m < M && n < N) {
-      float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-      apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
-      store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
-    }
-  });
+  // the tile buffers are too small to stage 32 rows per wave: 16 rows at a time in a buffer of their own
+  __shared__ __attribute__((aligned(16))) float stage_mem[4 * 16 * 64];
+  f32_tile_epilogue<16>(acc, stage_mem + (tid >> 6) * (16 * 64), args, m0 + wm * 64, n0 + wn * 64, zrow, lane);
 }
 
 
@@ -238,19 +274,7 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
     __syncthreads();                     // ... everyone's, and nobody still reads `cur`
   }
 
-  // operands were swapped: lane owns row (lane&31), channels 8g + 4*(lane>>5) + 0..3
-  // (compile-time indices: the body is large enough for the compiler to leave a plain loop
-  // rolled, and a run-time index into the accumulators moves them to scratch memory)
-  static_for<0, 16>([&](auto idx) {
-    constexpr int i = decltype(idx)::value >> 3, j = (decltype(idx)::value >> 2) & 1, g = decltype(idx)::value & 3;
-    const int m = m0 + wm * 64 + i * 32 + lrow;
-    const int n = n0 + wn * 64 + j * 32 + g * 8 + lhalf * 4;
-    if (m < M && n < N) {
-      float v[4] = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-      apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
-      store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
-    }
-  });
+  f32_tile_epilogue<32>(acc, (float *)smem + wave_u * (32 * 64), args, m0 + wm * 64, n0 + wn * 64, zrow, lane);
 }
 
 int launch_gemm_f32(const ContractionArgs &a, hipStream_t stream) {
