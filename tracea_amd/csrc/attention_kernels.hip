@@ -606,6 +606,11 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           lsum += x;
           if ((idx & 7) == 7) pf[idx >> 3] = pack8<DT>(p);
         }
+        // The row sum is not needed before the next iteration, and the compiler would sink
+        // its 32 additions, one dependent chain, out of the chunks into the tail of the loop
+        // body, behind every MFMA: pinning the partial sum at the end of each chunk keeps
+        // the additions where the matrix pipe hides them.
+        asm volatile("" : "+v"(lsum));
         kf0 = kn0;
         kf1 = kn1;
         __builtin_amdgcn_sched_barrier(0);
