@@ -67,6 +67,68 @@ __global__ void __launch_bounds__(256) mfma_loop(const half8 *src, float *sink, 
   if (s == 12345.678f) sink[tid] = s;  // keeps the accumulators alive; practically never true
 }
 
+// The same 8 MFMAs per iteration with the data movement of a GEMM main loop around them: R operand
+// fragments read from LDS (ds_read_b128 per lane) and G direct-to-LDS tile requests of 16 bytes per
+// lane.  The 256x256x64 tile with 128x64 wave tiles has R = 6, G = 2 per 8 MFMAs; 128x128 wave tiles R = 4.
+template <int R, int G>
+__global__ void __launch_bounds__(256) mfma_mix_loop(const half8 *src, float *sink, int iters) {
+  __shared__ half8 lds[4096];  // 64 KB
+  const int tid = blockIdx.x * 256 + threadIdx.x, t = threadIdx.x;
+  for (int i = t; i < 4096; i += 256) lds[i] = src[(blockIdx.x * 4096 + i) & 0xfffff];
+  __syncthreads();
+  half8 f[6];
+  for (int i = 0; i < 6; ++i) f[i] = src[(tid * 6 + i) & 0xfffff];
+  float16v acc[4][2];
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 2; ++j)
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)src, 0, 1 << 24, 0x00020000);
+  int off = t;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) f[r % 6] = lds[(off + r * 256) & 4095];
+    off += 67;
+    if constexpr (G > 0) {
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (__attribute__((address_space(3))) void *)(lds + ((g * 256 + (t & ~63)) & 4095)), 16,
+            ((it * 8 + g) * 4096 + tid * 16) & 0xffffff, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(f[4 + j], f[i], acc[i][j], 0, 0, 0);
+    if constexpr (G > 0) {
+      if ((it & 7) == 7) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): bounds the requests in flight
+    }
+  }
+  float s = 0.f;
+  for (int i = 0; i < 4; ++i)
+    for (int j = 0; j < 2; ++j)
+      for (int e = 0; e < 16; ++e) s += acc[i][j][e];
+  if (s == 12345.678f) sink[tid] = s;
+}
+
+template <int R, int G>
+static int run_mix(const half8 *src, float *sink, int blocks, int iters, int launches, const char *what) {
+  hipEvent_t e0, e1;
+  CHECK(hipEventCreate(&e0));
+  CHECK(hipEventCreate(&e1));
+  float ms = 0.f;
+  for (int rep = 0; rep < 2; ++rep) {
+    CHECK(hipEventRecord(e0));
+    for (int q = 0; q < launches; ++q) hipLaunchKernelGGL((mfma_mix_loop<R, G>), dim3(blocks), dim3(256), 0, 0, src, sink, iters);
+    CHECK(hipGetLastError());
+    CHECK(hipEventRecord(e1));
+    CHECK(hipEventSynchronize(e1));
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+  }
+  std::printf("N(0,1)/64, 32x32x16, %-44s %7.2f ms, %6.0f TFLOP/s\n", what, ms,
+              (double)launches * blocks * 4.0 * iters * 8.0 * 32768.0 / ms / 1e9);
+  return 0;
+}
+
 int main() {
   const int iters = 4000, launches = 5;
   const size_t n = 1 << 20;
@@ -110,5 +172,12 @@ int main() {
                   shape == 32 ? "32x32x16" : "16x16x32", ms, flop / ms / 1e9);
     }
   }
+  // operands are the N(0,1)/64 set from here on
+  if (run_mix<0, 0>(src, sink, blocks, iters, launches, "no data movement")) return 1;
+  if (run_mix<4, 0>(src, sink, blocks, iters, launches, "4 LDS reads per 8 MFMAs")) return 1;
+  if (run_mix<6, 0>(src, sink, blocks, iters, launches, "6 LDS reads per 8 MFMAs")) return 1;
+  if (run_mix<0, 2>(src, sink, blocks, iters, launches, "2 tile requests per 8 MFMAs")) return 1;
+  if (run_mix<4, 2>(src, sink, blocks, iters, launches, "4 LDS reads + 2 tile requests per 8 MFMAs")) return 1;
+  if (run_mix<6, 2>(src, sink, blocks, iters, launches, "6 LDS reads + 2 tile requests per 8 MFMAs")) return 1;
   return 0;
 }
