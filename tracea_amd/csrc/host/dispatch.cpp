@@ -1156,11 +1156,12 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // window whose K fits 40 filter tiles (the kernel has no split along K).  Fitted on the
   // ResNet-18/50 layer shapes at batch 1, 8 and 32, every variant timed inside a replayed
   // HIP graph (eager launches from a host loop cost 15 us apiece here and hide differences
-  // between kernels shorter than that): the 256-pixel tile wins only with at least 400
-  // workgroups of mostly real pixels (N32 56x56x64->64: 15.4 us against 19.0 for the
-  // 128-pixel tile and 17.5 for the best streamed variant); otherwise the 128-pixel tile,
+  // between kernels shorter than that): the 256-pixel tile (eight waves of 32 pixels) wins
+  // with at least 256 workgroups of mostly real pixels (N32 56x56x64->64: 15.4 us against
+  // 19.6 for the 128-pixel tile and 17.5 for the best streamed variant; N32 28x28
+  // 128->128: 14.3 against 16.0); otherwise the 128-pixel tile,
   // provided the launch has 100 workgroups or K is at most 9 filter tiles (N32 14x14
-  // 256->256: 18.2 us against 21.3 streamed; N32 28x28 128->128: 15.0 against 15.9; one
+  // 256->256: 18.2 us against 21.3 streamed; one
   // 56x56x64->64 image: 7.9 against 9.3).  With fewer workgroups and a long K the streamed
   // variants, which split along K, are faster.  A tuning-cache entry or a forced variant
   // wins over this rule, and tracea_autotune_conv2d measures every variant.
@@ -1172,7 +1173,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline != 4 || cv.bm != 256 || cv.bn != 64) continue;
       ContractionArgs probe = a;
-      if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= 400 &&
+      if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= 256 &&
           hw * 4 >= (long long)probe.p_tiles * cv.bm * 3)
         chosen = i;
     }
