@@ -357,6 +357,7 @@ int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split)
 // the estimate then reads 52.8 / 25.9 us for a 3x3 convolution on N32 7x7x512 with
 // unsplit 64x64 tiles / 128x128 tiles split four ways, where 53.7 / 29.6 us were measured.
 int select_contraction_variant(int m, int n, int k, bool conv) {
+  (void)conv;
   const double cus = 256.0, slot_rate = 1.43e6;  // multiply-accumulates per microsecond at efficiency 1
   int best = -1;
   double best_cost = 0.0;
@@ -379,12 +380,13 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
     // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
-    if (conv) {
+    {
       // A CU with fewer than 8 resident waves (one 4-wave workgroup, the launch too small or
-      // the tile's LDS too large for a second) hides less of the gather's latency.  The
-      // fourth root is fitted on 48 convolution shapes (ResNet-18/50 layers at batch 1, 8, 32,
-      // every variant timed inside a replayed HIP graph): it moves the choice from 128x128 to
-      // 128x64 tiles where the former leave CUs idle, and leaves the other choices alone.
+      // the tile's LDS too large for a second) hides less latency.  The fourth root is fitted
+      // on 48 convolution shapes (ResNet-18/50 layers at batch 1, 8, 32) and 17 GEMM shapes,
+      // every variant timed inside a replayed HIP graph: it moves the choice from 128x128 to
+      // 128x64 tiles where the former leave CUs idle, and leaves the other choices alone
+      // (defaults within 1.4 % / 1.6 % of the per-shape best in total on the two sets).
       const double lds = (double)v.stages * (v.bm + v.bn) * v.bk * 2.0;
       const double fit = std::floor(160.0 * 1024.0 / lds) < 1.0 ? 1.0 : std::floor(160.0 * 1024.0 / lds);
       const double per_cu = units / cus < 1.0 ? 1.0 : (units / cus > fit ? fit : units / cus);
@@ -1155,16 +1157,14 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // Default choice of a patch-resident variant: stride-1 convolutions with a real filter
   // window whose K fits 40 filter tiles (the kernel has no split along K).  Fitted on the
   // ResNet-18/50 layer shapes at batch 1, 8 and 32, every variant timed inside a replayed
-  // HIP graph (eager launches from a host loop cost 15 us apiece here and hide differences
+  // HIP graph (eager launches from a host loop cost 9-15 us apiece here and hide differences
   // between kernels shorter than that): the 256-pixel tile (eight waves of 32 pixels) wins
-  // with at least 256 workgroups of mostly real pixels (N32 56x56x64->64: 15.4 us against
-  // 19.6 for the 128-pixel tile and 17.5 for the best streamed variant; N32 28x28
-  // 128->128: 14.3 against 16.0); otherwise the 128-pixel tile,
-  // provided the launch has 100 workgroups or K is at most 9 filter tiles (N32 14x14
-  // 256->256: 18.2 us against 21.3 streamed; one
-  // 56x56x64->64 image: 7.9 against 9.3).  With fewer workgroups and a long K the streamed
-  // variants, which split along K, are faster.  A tuning-cache entry or a forced variant
-  // wins over this rule, and tracea_autotune_conv2d measures every variant.
+  // with at least 256 workgroups of mostly real pixels (N32 56x56x64->64: 15.0 us against
+  // 17.8 for the best streamed variant; N32 28x28 128->128: 14.0 against 15.3); the
+  // 128-pixel tile (eight waves of 32 pixels x 32 filters) wins on small launches with a
+  // short K (one 56x56x64->64 image: 7.4 us against 8.4).  Everywhere else the streamed
+  // 8-wave 128x64 and pipelined 64x64 tiles are as fast or faster.  A tuning-cache entry or
+  // a forced variant wins over this rule, and tracea_autotune_conv2d measures every variant.
   if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && g.stride_h == 1 &&
       g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 && a.K % 64 == 0 && a.K / 64 <= 40) {
     const long long hw = (long long)g.block.h_out * g.block.w_out;
@@ -1181,8 +1181,8 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline != 4 || cv.bm != 128 || cv.bn != 64) continue;
       ContractionArgs probe = a;
-      if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) &&
-          ((long long)probe.grid_m * probe.grid_n >= 100 || a.K / 64 <= 9))
+      if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n < 100 &&
+          a.K / 64 <= 9)
         chosen = i;
     }
     if (chosen >= 0) vi = chosen;
