@@ -112,6 +112,37 @@ def make_workload(name, torch, ops):
         plan.capture()
         return ("fp16 ResNet-18 forward, batch %d, 224x224, %d fused launches replayed as one HIP graph"
                 % (batch, len(plan.describe()["steps"])), flops, 0.0, "f16", plan.replay)
+    if name in ("basic_block", "downsample_block"):
+        # the reference's fused ResNet basic block, N=32: conv3x3+BN+ReLU -> conv3x3+BN+residual+ReLU on 128
+        # channels at 28x28, and the downsampling form (64ch 56x56 -> 128ch 28x28, stride-2 first convolution,
+        # 1x1 stride-2 shortcut convolution with BN); BN folded to scale/shift, every operator in an epilogue
+        from tracea_amd import capi
+        n = 32
+        down = name == "downsample_block"
+        cin, hin = (64, 56) if down else (128, 28)
+        ch, ho = 128, 28
+        x = torch.randn(n, hin, hin, cin, device=dev, generator=g).half()
+        w1 = (torch.randn(ch, 3, 3, cin, device=dev, generator=g) * (2.0 / (9 * cin)) ** 0.5).half()
+        w2 = (torch.randn(ch, 3, 3, ch, device=dev, generator=g) * (2.0 / (9 * ch)) ** 0.5).half()
+        ws = (torch.randn(ch, 1, 1, cin, device=dev, generator=g) * (2.0 / cin) ** 0.5).half()
+        bn = [(torch.rand(ch, device=dev, generator=g) + 0.5, torch.randn(ch, device=dev, generator=g) * 0.1) for _ in range(3)]
+        y1 = torch.empty(n, ho, ho, ch, device=dev, dtype=torch.float16)
+        sc = torch.empty_like(y1)
+        y2 = torch.empty_like(y1)
+
+        def block():
+            ops.conv2d_ex(x, w1, [(capi.OP_SCALE_SHIFT,) + bn[0], (capi.OP_RELU,)], stride=2 if down else 1, padding=1, out=y1)
+            skip = x
+            if down:
+                ops.conv2d_ex(x, ws, [(capi.OP_SCALE_SHIFT,) + bn[2]], stride=2, padding=0, out=sc)
+                skip = sc
+            ops.conv2d_ex(y1, w2, [(capi.OP_SCALE_SHIFT,) + bn[1], (capi.OP_RESIDUAL_ADD, skip), (capi.OP_RELU,)],
+                          stride=1, padding=1, out=y2)
+        m = n * ho * ho
+        flops = 2.0 * m * ch * 9 * cin + 2.0 * m * ch * 9 * ch + (2.0 * m * ch * cin if down else 0.0)
+        byts = 2.0 * (x.numel() * (2 if not down else 2) + w1.numel() + w2.numel() + 2 * y1.numel() + y2.numel())
+        return ("fp16 NHWC fused ResNet %s block N32 -> 128ch 28x28 (%d launches)" % ("downsampling" if down else "basic", 3 if down else 2),
+                flops, byts, "f16", block)
     if name == "gemm_tiles_half":
         # the headline product restricted to a random half of its 128x128 output tiles through a tile
         # list (the reference's examples/ttg_sparse_experiment.rs at full size); FLOPs count listed tiles
@@ -230,8 +261,8 @@ def main():
     if not args.no_extras:
         cpu = cpu_baseline()
         also = {}
-        for name in ("gemm", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "attention", "attention_causal", "conv_transpose", "resnet18_b1",
-                     "resnet18_b32", "gemm_tiles_half"):
+        for name in ("gemm", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "basic_block", "downsample_block", "attention", "attention_causal",
+                     "conv_transpose", "resnet18_b1", "resnet18_b32", "gemm_tiles_half"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)
@@ -239,7 +270,7 @@ def main():
             also[name] = {"workload": lab, "tflops": round(fl / d / 1e12, 2),
                           "pct_of_peak": round(100.0 * fl / d / 1e12 / PEAKS.get(dt, PEAK_TFLOPS), 2),
                           "us_per_launch": round(d * 1e6, 2), "dtype": dt}
-            if name in ("conv", "gemm_f32"):  # shorter than the host's per-call cost: also as a replayed graph
+            if name in ("conv", "gemm_f32", "basic_block", "downsample_block"):  # launches shorter than the host's per-call cost: also as a replayed graph
                 dg = time_steps_graph(torch, st, 40)
                 also[name]["us_per_launch_graph"] = round(dg * 1e6, 2)
                 also[name]["tflops_graph"] = round(fl / dg / 1e12, 2)
