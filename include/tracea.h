@@ -298,6 +298,13 @@ TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaT
  * the operator chain.  On by default; tracea_set_split_k(0) turns it off.
  * tracea_last_split_k: K ranges of the calling thread's latest gemm / conv2d launch (1: not split). */
 void tracea_set_split_k(int32_t enabled);
+/* tracea_conv_transpose2d runs as one stride-1 convolution per output phase (stride_h * stride_w
+ * launches on a regrouped copy of the filter bank, the outputs written in place) when every phase
+ * has taps and no negative padding and the input is dense half-precision NHWC with a multiple of 8
+ * channels; otherwise, and always after tracea_set_conv_transpose_by_phase(0), as a GEMM to fp32
+ * partial products followed by a gather.  The two formulations agree within the tolerance of the
+ * operator (fp32 accumulation in a different order). */
+void tracea_set_conv_transpose_by_phase(int32_t enabled);
 int32_t tracea_last_split_k(void);
 
 /* Kernel-variant control for tuners and benchmarks.  `op` is "gemm", "conv2d"

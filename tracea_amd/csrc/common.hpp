@@ -53,6 +53,17 @@ struct ContractionArgs {
   int h_in, w_in, c_in, h_out, w_out, s_sz;
   int stride_h, stride_w, pad_h, pad_w, dil_h, dil_w;
   unsigned hw_m, hw_s, w_m, w_s, sc_m, sc_s, c_m, c_s;
+  // streamed convolution only (out_map != 0): output pixel (q, p) of image b is written to row
+  // b*o_img + (o_a + o_sh*q)*o_wo + o_b + o_sw*p of C instead of row m (one phase of a transposed
+  // convolution); residual operands are indexed by the same row.  Not combined with a K split.
+  int out_map, o_sh, o_sw, o_a, o_b, o_wo;
+  long long o_img;
+  // phases > 1: grid.z = phases = o_sh*o_sw launches all phases at once; workgroups with
+  // blockIdx.z = z work on phase (o_a, o_b) = (z / o_sw, z % o_sw) with the filter bank at
+  // B + z*phase_b_stride elements and the padding phase_pad_h[o_a], phase_pad_w[o_b] (strides up to 4)
+  int phases;
+  long long phase_b_stride;
+  int phase_pad_h[4], phase_pad_w[4];
   // patch-resident convolution (pipeline 4) only: filter rows, M tiles per image,
   // padded row width W + 2 pad_w, 16-byte chunks per patch pixel (odd), patch
   // load iterations per thread, LDS bytes reserved for the patch, and the
@@ -136,6 +147,19 @@ int launch_col2im_epilogue(const Col2imArgs &args, hipStream_t stream);
 // the B operand of the transposed convolution's GEMM, columns ordered (r, s, k):
 // [R][S][K][C] (K-contiguous B, for the half-precision kernels) when c_inner,
 // else [C][R][S][K] (row-major B, for the fp32 kernel).
+// Filters of a transposed convolution regrouped by output phase: tap (r, s) of the filter bank
+// goes to out + tap_base[r*S + s] + k * tap_kstride[r*S + s] + c (half precision only), which
+// makes every phase a [K, taps_r, taps_s, C] filter bank for the convolution kernels.
+struct PhaseFilterArgs {
+  const void *w;
+  void *out;
+  int C, K, R, S;
+  long long sc, sk, sr, ss;  // element strides of c, k, r, s in w
+  long long tap_base[64];
+  int tap_kstride[64];
+};
+int launch_phase_filters(const PhaseFilterArgs &args, hipStream_t stream);
+
 struct FilterRepackArgs {
   const void *w;
   void *out;

@@ -608,6 +608,19 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 
   const unsigned short *Ag = (const unsigned short *)args.A;
   const unsigned short *Bg = (const unsigned short *)args.B;
+  // all phases of a transposed convolution in one launch: blockIdx.z names the phase
+  int pad_h = args.pad_h, pad_w = args.pad_w, o_a = args.o_a, o_b = args.o_b;
+  if constexpr (CONV) {
+    if (args.phases > 1) {
+      const int z = (int)blockIdx.z;
+      o_a = z / args.o_sw;
+      o_b = z - o_a * args.o_sw;
+      // selects, not an index: a run-time index into the kernel arguments can move them to scratch memory
+      pad_h = o_a == 0 ? args.phase_pad_h[0] : o_a == 1 ? args.phase_pad_h[1] : o_a == 2 ? args.phase_pad_h[2] : args.phase_pad_h[3];
+      pad_w = o_b == 0 ? args.phase_pad_w[0] : o_b == 1 ? args.phase_pad_w[1] : o_b == 2 ? args.phase_pad_w[2] : args.phase_pad_w[3];
+      Bg += (long long)z * args.phase_b_stride;
+    }
+  }
 
   long long a_off[NA];              // GEMM: element offset of the row start (+ piece column)
   int a_hb[CONV ? NA : 1], a_wb[CONV ? NA : 1];  // conv: ho*stride-pad, wo*stride-pad
@@ -620,8 +633,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       fast_divmod(m, args.hw_m, args.hw_s, args.h_out * args.w_out, bn, rem);
       fast_divmod(rem, args.w_m, args.w_s, args.w_out, ho, wo);
       a_off[i] = (long long)bn * args.h_in * args.w_in * args.c_in;
-      a_hb[i] = ho * args.stride_h - args.pad_h;
-      a_wb[i] = wo * args.stride_w - args.pad_w;
+      a_hb[i] = ho * args.stride_h - pad_h;
+      a_wb[i] = wo * args.stride_w - pad_w;
     } else {
       a_off[i] = (long long)m * args.lda;
     }
@@ -733,7 +746,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       (void *)args.A, 0, (int)args.a_bytes, 0x00020000);
   __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      (void *)args.B, 0, (int)args.b_bytes, 0x00020000);
+      (void *)Bg, 0, (int)args.b_bytes, 0x00020000);
   unsigned a_voff[NA], b_voff[NB];
   if constexpr (PIPE >= 2) {
 #pragma unroll
@@ -1213,9 +1226,23 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // overwrites what this one reads).
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
+    // Output row of GEMM row m.  A convolution may scatter its pixels into a larger image: pixel
+    // (q, p) of image b goes to row b*o_img + (o_a + o_sh*q)*o_wo + o_b + o_sw*p (one phase of a
+    // transposed convolution writing its share of the full output).
+    auto out_row = [&](int m) -> long long {
+      if constexpr (CONV) {
+        if (args.out_map != 0) {
+          int img, rem, q, pcol;
+          fast_divmod(m, args.hw_m, args.hw_s, args.h_out * args.w_out, img, rem);
+          fast_divmod(rem, args.w_m, args.w_s, args.w_out, q, pcol);
+          return (long long)img * args.o_img + (long long)(o_a + args.o_sh * q) * args.o_wo + o_b + args.o_sw * pcol;
+        }
+      }
+      return zrow + m;
+    };
     if (simple) {
       const int mb = m0 + wm * TM + i * 32;
-      auto row_of = [&](int r) -> long long { return mb + r < M ? zrow + (mb + r) : -1ll; };
+      auto row_of = [&](int r) -> long long { return mb + r < M ? out_row(mb + r) : -1ll; };
       if constexpr (F32_SIMPLE) {
         if (out_f32) simple_rows<DT, TN, true>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
         else simple_rows<DT, TN, false>(stage, lane, n0 + wn * TN + ec, args, plan, tab, BN, row_of);
@@ -1236,8 +1263,9 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
             v[4 + e] = hi[e];
           }
           const int nvalid = N - n;
-          apply_epilogue_tab(v, zrow + m, n, nvalid, args.epi, plan, tab, BN);
-          store_from_float<8>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, nvalid, v);
+          const long long row = out_row(m);
+          apply_epilogue_tab(v, row, n, nvalid, args.epi, plan, tab, BN);
+          store_from_float<8>(args.C, args.out_dtype, row * args.ldc + n, nvalid, v);
         }
       }
     }
@@ -1252,7 +1280,8 @@ int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_nc
   constexpr size_t lds = (size_t)NS * (BM + BN) * BK * 2;
   const bool listed = !conv && a.tile_list != nullptr;  // one workgroup per record, no split grid
   const dim3 grid((unsigned)(listed ? a.tile_count : a.grid_m * a.grid_n),
-                  (unsigned)(!listed && a.k_split > 0 ? (a.K + a.k_split - 1) / a.k_split : 1)),
+                  (unsigned)(!listed && a.k_split > 0 ? (a.K + a.k_split - 1) / a.k_split : 1),
+                  (unsigned)(conv && a.phases > 1 ? a.phases : 1)),
       block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \

@@ -113,4 +113,48 @@ int launch_filter_repack(const FilterRepackArgs &a, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
+// One workgroup per (64 input channels, 64 filters, tap): a 64x64 tile goes through LDS so that
+// both the reads (whichever of c and k is the faster axis of w) and the writes (c fastest) are
+// coalesced.
+__global__ void __launch_bounds__(256) phase_filter_kernel(const PhaseFilterArgs a) {
+  __shared__ unsigned short tile[64][65];
+  const int c0 = blockIdx.x * 64, k0 = blockIdx.y * 64;
+  const int z = blockIdx.z, r = z / a.S, s = z % a.S;
+  const int fast = threadIdx.x & 63, slow = threadIdx.x >> 6;
+  const bool k_fast = a.sk <= a.sc;
+  const unsigned short *src = (const unsigned short *)a.w + (long long)r * a.sr + (long long)s * a.ss;
+  // all sixteen loads in flight before the first LDS write (a rolled loop waits for each in turn)
+  unsigned short v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int kk = k_fast ? fast : slow + i * 4, cc = k_fast ? slow + i * 4 : fast;
+    const int k = k0 + kk, c = c0 + cc;
+    v[i] = (k < a.K && c < a.C) ? src[(long long)k * a.sk + (long long)c * a.sc] : (unsigned short)0;
+  }
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int kk = k_fast ? fast : slow + i * 4, cc = k_fast ? slow + i * 4 : fast;
+    tile[cc][kk] = v[i];
+  }
+  __syncthreads();
+  // two channels per store (C is a multiple of 8 on this path, every destination 4-byte aligned)
+  unsigned short *dst = (unsigned short *)a.out + a.tap_base[z];
+  const long long kstride = a.tap_kstride[z];
+  const int pair = threadIdx.x & 31, krow = threadIdx.x >> 5;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int kk = krow + i * 8, k = k0 + kk, c = c0 + pair * 2;
+    if (k < a.K && c < a.C)
+      *(unsigned *)(dst + k * kstride + c) = (unsigned)tile[pair * 2][kk] | ((unsigned)tile[pair * 2 + 1][kk] << 16);
+  }
+}
+
+int launch_phase_filters(const PhaseFilterArgs &a, hipStream_t stream) {
+  if (a.R * a.S > 64 || a.R * a.S <= 0) return (int)hipErrorInvalidValue;
+  const dim3 grid((unsigned)((a.C + 63) / 64), (unsigned)((a.K + 63) / 64), (unsigned)(a.R * a.S));
+  if (grid.y > 65535) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(phase_filter_kernel, grid, dim3(256), 0, stream, a);
+  return (int)hipGetLastError();
+}
+
 }  // namespace tracea_amd

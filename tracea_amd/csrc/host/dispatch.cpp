@@ -241,6 +241,7 @@ std::atomic<int> g_forced_contraction{-1};
 std::atomic<int> g_forced_conv{-1};
 std::atomic<int> g_forced_attention{-1};
 std::atomic<bool> g_split_k_enabled{true};
+std::atomic<bool> g_conv_transpose_by_phase{true};
 // variant the calling thread's latest launch of each operator used (-1: none,
 // or a kernel outside the variant tables)
 thread_local int t_last_contraction = -1, t_last_conv = -1, t_last_attention = -1;
@@ -254,6 +255,7 @@ TraceaStatus hip_status(const char *what, int e) {
 }  // namespace
 
 void set_split_k_enabled(bool on) { g_split_k_enabled.store(on); }
+void set_conv_transpose_by_phase(bool on) { g_conv_transpose_by_phase.store(on); }
 int last_split_k() { return t_last_splits; }
 
 void set_forced_variant(const char *op, int index) {
@@ -1360,6 +1362,142 @@ TraceaStatus conv_transpose_common(const TraceaTensorView &tx, const TraceaTenso
   return TRACEA_SUCCESS;
 }
 
+// ---- transposed convolution by output phase ----------------------------------------
+// Output pixels whose row is congruent to a modulo stride_h (and column to b modulo stride_w)
+// are reached by the taps r = r0 + stride_h*t, r0 = (a + pad_h) mod stride_h, only, from input
+// rows q + d - t with oh = a + stride_h*q, d = (a + pad_h - r0) / stride_h: each of the
+// stride_h*stride_w phases is an ordinary stride-1 convolution of the input with the flipped
+// sub-filter (taps_r x taps_s taps), top padding taps_r - 1 - d, whose output pixels are
+// written into their places of the full output by the kernel's row map.  Against the
+// formulation through partial products (a GEMM to [pixels, R*S*K] fp32 and a gather) nothing
+// but the input, the filters and the output touches memory.
+struct PhaseAxis {
+  int taps, pad, out;  // taps of the sub-filter, top/left padding, output extent of the phase
+  int first_tap;       // r0
+};
+
+PhaseAxis phase_axis(int a, int stride, int pad, int filter, long long out_extent) {
+  PhaseAxis p{};
+  p.first_tap = (a + pad) % stride;
+  p.taps = p.first_tap < filter ? (filter - p.first_tap + stride - 1) / stride : 0;
+  const int d = (a + pad - p.first_tap) / stride;
+  p.pad = p.taps - 1 - d;
+  p.out = a < out_extent ? (int)((out_extent - a + stride - 1) / stride) : 0;
+  return p;
+}
+
+// True when every phase is a convolution the streamed kernels take: taps in every phase, no
+// negative padding, half-precision dense NHWC input with channels in 16-byte groups.
+bool conv_transpose_by_phase_ok(const ConvTransposePlan &plan) {
+  const View &x = plan.x, &w = plan.w, &out = plan.out;
+  const long long C = x.shape[3], R = w.shape[1], S = w.shape[2];
+  if (!is_half(x.dtype) || C % 8 != 0 || plan.ldx != C || !aligned(x.ptr, 16) || R * S > 64) return false;
+  if (x.shape[0] * x.shape[1] * x.shape[2] * C * 2 >= (1ll << 40)) return false;
+  for (int a = 0; a < plan.stride_h; ++a) {
+    const PhaseAxis p = phase_axis(a, plan.stride_h, plan.pad_h, (int)R, out.shape[1]);
+    if (p.taps <= 0 || p.pad < 0 || p.out <= 0) return false;
+  }
+  for (int b = 0; b < plan.stride_w; ++b) {
+    const PhaseAxis p = phase_axis(b, plan.stride_w, plan.pad_w, (int)S, out.shape[2]);
+    if (p.taps <= 0 || p.pad < 0 || p.out <= 0) return false;
+  }
+  return (long long)plan.stride_h * plan.stride_w <= 16;
+}
+
+TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const EpilogueChain &chain,
+                                         hipStream_t stream) {
+  const View &x = plan.x, &w = plan.w, &out = plan.out;
+  const int N = (int)x.shape[0], H = (int)x.shape[1], W = (int)x.shape[2], C = (int)x.shape[3];
+  const int K = (int)w.shape[0], R = (int)w.shape[1], S = (int)w.shape[2];
+  const long long Ho = out.shape[1], Wo = out.shape[2];
+  const int sh = plan.stride_h, sw = plan.stride_w;
+  // the filter bank, regrouped: phase (a, b) holds [K][taps_r][taps_s][C], flipped
+  PhaseFilterArgs f{};
+  f.w = w.ptr; f.C = C; f.K = K; f.R = R; f.S = S;
+  f.sk = w.stride[0]; f.sr = w.stride[1]; f.ss = w.stride[2]; f.sc = w.stride[3];
+  std::vector<long long> phase_off((size_t)sh * sw);
+  long long total = 0;
+  for (int a = 0; a < sh; ++a)
+    for (int b = 0; b < sw; ++b) {
+      const PhaseAxis pr = phase_axis(a, sh, plan.pad_h, R, Ho), ps = phase_axis(b, sw, plan.pad_w, S, Wo);
+      phase_off[(size_t)a * sw + b] = total;
+      for (int t = 0; t < pr.taps; ++t)
+        for (int u = 0; u < ps.taps; ++u) {
+          const int r = pr.first_tap + sh * t, s_ = ps.first_tap + sw * u;
+          const int z = r * S + s_;
+          f.tap_base[z] = total + ((long long)(pr.taps - 1 - t) * ps.taps + (ps.taps - 1 - u)) * C;
+          f.tap_kstride[z] = pr.taps * ps.taps * C;
+        }
+      total += (long long)K * pr.taps * ps.taps * C;
+    }
+  void *filt = nullptr;
+  hipError_t e = hipMallocAsync(&filt, (size_t)total * 2 + 256, stream);
+  if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+  f.out = filt;
+  TraceaStatus st = hip_status("phase filter launch", launch_phase_filters(f, stream));
+  const long long x_extent = (long long)N * H * W * C * 2;
+  // Phases that are alike but for their padding (even filter extents divided by the stride: the 4x4
+  // stride-2 decoder layer) go out as one launch with the phase in blockIdx.z.
+  bool uniform = sh <= 4 && sw <= 4 && sh * sw > 1;
+  for (int a = 1; a < sh && uniform; ++a) {
+    const PhaseAxis p0 = phase_axis(0, sh, plan.pad_h, R, Ho), pa = phase_axis(a, sh, plan.pad_h, R, Ho);
+    uniform = p0.taps == pa.taps && p0.out == pa.out;
+  }
+  for (int b = 1; b < sw && uniform; ++b) {
+    const PhaseAxis p0 = phase_axis(0, sw, plan.pad_w, S, Wo), pb = phase_axis(b, sw, plan.pad_w, S, Wo);
+    uniform = p0.taps == pb.taps && p0.out == pb.out;
+  }
+  for (int a = 0; a < sh && st == TRACEA_SUCCESS; ++a)
+    for (int b = 0; b < sw && st == TRACEA_SUCCESS; ++b) {
+      if (uniform && (a > 0 || b > 0)) continue;  // phase (0, 0) launched all of them
+      const PhaseAxis pr = phase_axis(a, sh, plan.pad_h, R, Ho), ps = phase_axis(b, sw, plan.pad_w, S, Wo);
+      const long long m = (long long)N * pr.out * ps.out, kg = (long long)pr.taps * ps.taps * C;
+      if (m >= (1ll << 31) || kg >= (1ll << 31)) {
+        st = fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv_transpose2d: problem too large for 32-bit row indices");
+        break;
+      }
+      ContractionArgs c{};
+      c.A = x.ptr;
+      c.B = (const unsigned short *)filt + phase_off[(size_t)a * sw + b];
+      c.C = out.ptr;
+      c.M = (int)m; c.N = K; c.K = (int)kg;
+      c.ldb = kg; c.ldc = plan.ldc;
+      c.out_dtype = out.dtype;
+      c.h_in = H; c.w_in = W; c.c_in = C;
+      c.h_out = pr.out; c.w_out = ps.out; c.s_sz = ps.taps;
+      c.stride_h = c.stride_w = 1; c.dil_h = c.dil_w = 1;
+      c.pad_h = pr.pad; c.pad_w = ps.pad;
+      magic_for_divisor((uint32_t)(pr.out * ps.out), (uint64_t)m, &c.hw_m, &c.hw_s);
+      magic_for_divisor((uint32_t)ps.out, (uint64_t)pr.out * ps.out, &c.w_m, &c.w_s);
+      magic_for_divisor((uint32_t)(ps.taps * C), (uint64_t)kg + 1024, &c.sc_m, &c.sc_s);
+      magic_for_divisor((uint32_t)C, (uint64_t)ps.taps * C, &c.c_m, &c.c_s);
+      c.out_map = 1;
+      c.o_sh = sh; c.o_sw = sw; c.o_a = a; c.o_b = b; c.o_wo = (int)Wo;
+      c.o_img = Ho * Wo;
+      if (uniform) {
+        c.phases = sh * sw;
+        c.phase_b_stride = (long long)K * kg;
+        for (int i = 0; i < sh; ++i) c.phase_pad_h[i] = phase_axis(i, sh, plan.pad_h, R, Ho).pad;
+        for (int i = 0; i < sw; ++i) c.phase_pad_w[i] = phase_axis(i, sw, plan.pad_w, S, Wo).pad;
+      }
+      c.epi = chain;
+      int vi = select_contraction_variant(c.M, c.N, c.K, true);
+      if (vi < 0) { st = fail(TRACEA_UNKNOWN_ERROR, "tracea_conv_transpose2d: no kernel variant available"); break; }
+      const long long w_extent = (long long)K * kg * 2;
+      const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
+      vi = resolve_variant(vi, true, !small, true);
+      const ContractionVariant &v = contraction_variant(vi);
+      c.a_bytes = (unsigned)(small ? x_extent : 0);
+      c.b_bytes = (unsigned)(small ? w_extent : 0);
+      fill_grid(&c, v);
+      t_last_conv = vi;
+      st = hip_status("conv_transpose2d phase launch", v.launch(c, true, x.dtype, false, stream));
+    }
+  e = hipFreeAsync(filt, stream);
+  if (st == TRACEA_SUCCESS && e != hipSuccess) st = hip_status("tracea_conv_transpose2d: workspace release", (int)e);
+  return st;
+}
+
 TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueChain &chain, hipStream_t stream) {
   const View &x = plan.x, &w = plan.w, &out = plan.out;
   const long long N = x.shape[0], H = x.shape[1], W = x.shape[2], C = x.shape[3];
@@ -1367,6 +1505,8 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
   const long long J = plan.fm.columns;
   DeviceScope scope(out.device);
   if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  if (g_conv_transpose_by_phase.load() && conv_transpose_by_phase_ok(plan))
+    return run_conv_transpose_by_phase(plan, chain, stream);
   // Images per pass: the partial products of a pass stay below 512 MiB, the GEMM
   // rows and the gather kernel's thread count below 2^31.
   const long long per_image = H * W * J * 4;

@@ -36,6 +36,9 @@ int last_variant(const char *op);
 // Split-K of launches with few output tiles and a long K (on by default), and the number of
 // K ranges the calling thread's latest gemm / conv2d launch was split into (1: not split).
 void set_split_k_enabled(bool on);
+// Transposed convolutions as one stride-1 convolution per output phase where that applies (on by
+// default); off: always the GEMM to partial products followed by the gather.
+void set_conv_transpose_by_phase(bool on);
 int last_split_k();
 
 TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorView &b,
