@@ -184,3 +184,45 @@ def test_argument_errors(tracea_gpu):
     assert "dilation" in capi.last_error()
     p = capi.ConvTranspose2dParams(0, 2, 0, 0, 0, 0, 1, 1, 1, capi.EPI_IDENTITY, None)
     assert capi.lib().tracea_conv_transpose2d(vx.c, vw.c, None, None, C.byref(vo.c), p) == capi.INVALID_PARAMS
+
+
+PHASE_SHAPES = [  # n, h, w, c, k, r, s, stride, pad, output_padding: every phase has taps and no negative padding
+    (2, 8, 8, 16, 24, 4, 4, 2, 1, 0),            # uniform phases: one launch, phase in blockIdx.z
+    (2, 9, 7, 32, 40, 3, 3, 2, 1, 1),            # phases of 2x2, 2x1, 1x2 and 1x1 taps: four launches
+    (1, 6, 10, 8, 16, 5, 3, (3, 2), (2, 1), (2, 1)),
+    (3, 5, 5, 24, 8, 2, 2, 2, 0, 0),
+    (1, 12, 12, 64, 72, 6, 6, 3, 2, 0),
+    (2, 7, 6, 16, 16, 3, 4, (1, 2), (1, 1), (0, 0)),
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape", PHASE_SHAPES)
+def test_formulation_by_output_phase_against_the_oracle_and_the_other_formulation(tracea_gpu, shape, dtype):
+    """The phase path forced on and off on the same operands, with a chain that reads a residual
+    through the row map: both match the oracle within the operator's tolerance."""
+    from tracea_amd import capi
+    n, h, w, c, k, r, s, stride, pad, opad = shape
+    tdt, rnd = (torch.float16, round_f16) if dtype == "f16" else (torch.bfloat16, round_bf16)
+    rng = np.random.default_rng(h * 31 + c)
+    x = rnd(rng.uniform(-1, 1, (n, h, w, c)))
+    wt = rnd(rng.uniform(-0.5, 0.5, (c, r, s, k)))
+    bias = rng.standard_normal(k).astype(np.float32)
+    ho, wo = oracle.conv_transpose_out_shape(h, w, r, s, stride, pad, opad)
+    res = rnd(rng.standard_normal((n, ho, wo, k)))
+    ref = np.maximum(oracle.conv_transpose2d_nhwc(x, wt, stride, pad, opad) + bias + res, 0.0)
+    got = {}
+    try:
+        for mode in (1, 0):
+            capi.lib().tracea_set_conv_transpose_by_phase(mode)
+            y = tracea_gpu.conv_transpose2d_ex(
+                _dev(x, tdt), _dev(wt, tdt),
+                [(capi.OP_BIAS_ADD, _dev(bias)), (capi.OP_RESIDUAL_ADD, _dev(res, tdt)), (capi.OP_RELU,)],
+                stride=stride, padding=pad, output_padding=opad)
+            got[mode] = y.float().cpu().numpy()
+            assert_close_scaled(got[mode], ref, tol_half(c * r * s, dtype), "mode %d %s %s" % (mode, dtype, shape))
+    finally:
+        capi.lib().tracea_set_conv_transpose_by_phase(1)
+    # the two differ by the order of fp32 additions and one output rounding at most
+    ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
+    assert np.abs(got[1] - got[0]).max() <= ulp * max(1.0, np.abs(ref).max())
