@@ -1430,9 +1430,16 @@ TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const Ep
         }
       total += (long long)K * pr.taps * ps.taps * C;
     }
-  void *filt = nullptr;
-  hipError_t e = hipMallocAsync(&filt, (size_t)total * 2 + 256, stream);
-  if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+  // The regrouped filters live in the per-(device, stream) scratch buffer that split-K launches use
+  // (no launch of this path splits K, and work on one stream is ordered); a bank beyond its 64 MiB
+  // cap, or a first use while the stream is being captured, takes a stream-ordered allocation.
+  hipError_t e = hipSuccess;
+  void *filt = splitk_scratch(out.device, stream, (size_t)total * 2 + 256);
+  const bool pooled = filt != nullptr;
+  if (!pooled) {
+    e = hipMallocAsync(&filt, (size_t)total * 2 + 256, stream);
+    if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+  }
   f.out = filt;
   TraceaStatus st = hip_status("phase filter launch", launch_phase_filters(f, stream));
   const long long x_extent = (long long)N * H * W * C * 2;
@@ -1493,8 +1500,10 @@ TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const Ep
       t_last_conv = vi;
       st = hip_status("conv_transpose2d phase launch", v.launch(c, true, x.dtype, false, stream));
     }
-  e = hipFreeAsync(filt, stream);
-  if (st == TRACEA_SUCCESS && e != hipSuccess) st = hip_status("tracea_conv_transpose2d: workspace release", (int)e);
+  if (!pooled) {
+    e = hipFreeAsync(filt, stream);
+    if (st == TRACEA_SUCCESS && e != hipSuccess) st = hip_status("tracea_conv_transpose2d: workspace release", (int)e);
+  }
   return st;
 }
 
