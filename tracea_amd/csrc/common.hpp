@@ -103,7 +103,7 @@ int contraction_variant_count();
 const ContractionVariant &contraction_variant(int i);
 
 // fp32 MFMA GEMM (row-major A [M,K], row-major B [K,N]).
-int launch_gemm_f32(const ContractionArgs &args, hipStream_t stream);
+int launch_gemm_f32(const ContractionArgs &args, int tile, hipStream_t stream);  // tile: 128 or 64
 // Any dtype/stride combination, no alignment requirement (VALU, slow).
 struct GenericGemmArgs {
   const void *A, *B;

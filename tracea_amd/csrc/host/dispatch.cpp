@@ -337,12 +337,12 @@ TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s,
 // entry, when present, wins over this.
 namespace {
 // Number of K ranges for a launch of variant v (1: no split) and the extent of one range.
-int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split) {
+int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split, int min_tiles = 4) {
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
-  if (v.pipeline == 4 || tiles * 2 > 256 || nk < 8) return 1;
+  if (v.pipeline == 4 || tiles * 2 > 256 || nk < 2 * min_tiles) return 1;
   long long splits = 256 / tiles;
-  if (splits > nk / 4) splits = nk / 4;  // at least 4 K tiles per range
+  if (splits > nk / min_tiles) splits = nk / min_tiles;  // at least min_tiles K tiles per range
   if (splits < 2) return 1;
   const int per = (int)((nk + splits - 1) / splits);
   *k_split = per * v.bk;
@@ -575,15 +575,24 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.a_bytes = (unsigned)a_extent;
       args.b_bytes = (unsigned)b_extent;
     }
-    // the fp32 kernel has one tile shape, 128x128x16; it splits along K by the same rule
-    static const ContractionVariant f32_tile = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr};
+    // Two tile shapes, 128x128x16 and (direct-to-LDS form only) 64x64x16.  A CU works through its
+    // share of the tiles at one 128x128 tile per 4 units of time or one 64x64 tile per 1.06 units
+    // (the small tile reads its operands from LDS twice as often): the shape whose busiest CU
+    // finishes first is taken.  Measured, 128 / 64, in us: 1024^3 32.5 / 27.0, 1536^3 104 / 79,
+    // 2304x2048x512 70 / 49, 3072^3 539 / 454, 2048^3 138 / 135, 4096^3 972 / 1027.
+    // Both split along K by the rule of the half kernels.
+    static const ContractionVariant f32_tile128 = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr};
+    static const ContractionVariant f32_tile64 = {"f32_64x64x16", 64, 64, 16, 2, 2, 1, 0, 0, nullptr};
+    const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
+    const int tile = args.a_bytes != 0 && (double)((tiles64 + 255) / 256) * 1.06 < (double)((tiles128 + 255) / 256) * 4.0 ? 64 : 128;
+    const ContractionVariant &f32_tile = tile == 64 ? f32_tile64 : f32_tile128;
     int k_split = 0;
-    const int splits = g_split_k_enabled.load() ? choose_split(f32_tile, (int)M, (int)N, (int)K, &k_split) : 1;
+    const int splits = g_split_k_enabled.load() ? choose_split(f32_tile, (int)M, (int)N, (int)K, &k_split, tile == 64 ? 16 : 4) : 1;
     void *scratch = splits > 1 ? splitk_scratch(c.device, stream, (size_t)splits * M * N * 4) : nullptr;
     t_last_splits = scratch != nullptr ? splits : 1;
     if (scratch == nullptr) {
       args.epi = chain;
-      return hip_status("gemm_f32 launch", launch_gemm_f32(args, stream));
+      return hip_status("gemm_f32 launch", launch_gemm_f32(args, tile, stream));
     }
     SplitKReduceArgs r{};
     r.partial = (const float *)scratch;
@@ -593,7 +602,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     args.C = scratch;
     args.ldc = N;
     args.k_split = k_split;
-    TraceaStatus st = hip_status("gemm_f32 launch", launch_gemm_f32(args, stream));
+    TraceaStatus st = hip_status("gemm_f32 launch", launch_gemm_f32(args, tile, stream));
     if (st != TRACEA_SUCCESS) return st;
     return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
   }

@@ -17,42 +17,43 @@ namespace tracea_amd {
 // ---------------------------------------------------------------------------
 constexpr int F32_BM = 128, F32_BN = 128, F32_BK = 16, F32_PITCH = 132;
 
-// Epilogue of the 128x128 fp32 tile kernels.  Operands were swapped in the MFMAs: a lane owns
-// row (lane&31), channels 8g + 4*(lane>>5) + 0..3 of each 32x32 block of its wave's 64x64 tile.
-// The accumulators go through LDS, ROWS rows at a time (`stage` is ROWS x 64 floats private to
+// Epilogue of the fp32 tile kernels.  Operands were swapped in the MFMAs: a lane owns row
+// (lane&31), channels 8g + 4*(lane>>5) + 0..3 of each 32x32 block of its wave's 32FM x 32FN tile.
+// The accumulators go through LDS, ROWS rows at a time (`stage` is ROWS x 32FN floats private to
 // the wave), and a rolled loop takes them from there row by row.  Applying the operator chain
 // to the accumulators in place needs compile-time indices, i.e. sixteen copies of the chain
 // code, and with them the compiler copied the chain description from the kernel arguments to
 // scratch memory (488 bytes per lane) and kept 192 registers: 1024^3 took 46.6 us that way and
-// takes 32.9 us this way, 4096^3 1194 -> 979 us.
-template <int ROWS>
-__device__ __forceinline__ void f32_tile_epilogue(const f32x16 (&acc)[2][2], float *stage, const ContractionArgs &args,
+// 32.9 us this way (128x128 tiles), 4096^3 1194 -> 979 us.
+template <int ROWS, int FM, int FN>
+__device__ __forceinline__ void f32_tile_epilogue(const f32x16 (&acc)[FM][FN], float *stage, const ContractionArgs &args,
                                                   int m_wave, int n_wave, long long zrow, int lane) {
   static_assert(ROWS == 32 || ROWS == 16, "a 32-row block is staged whole or in two halves");
+  constexpr int W = 32 * FN, CH = 8 * FN;  // floats and 16-byte chunks per staged row
   const int lrow = lane & 31, lhalf = lane >> 5;
-  const int er = lane >> 4, lc = lane & 15;  // reader: 4 rows per step, 16 lanes x 4 channels per row
+  const int er = lane / CH, lc = lane % CH;  // reader: 64/CH rows per step, CH lanes x 4 channels per row
   const int M = args.M, N = args.N;
-  static_for<0, 2 * (32 / ROWS)>([&](auto blk) {
+  static_for<0, FM * (32 / ROWS)>([&](auto blk) {
     constexpr int i = decltype(blk)::value / (32 / ROWS), part = decltype(blk)::value % (32 / ROWS);
     if (ROWS == 32 || (lrow / ROWS) == part) {
       const int srow = lrow % ROWS;
 #pragma unroll
-      for (int jj = 0; jj < 2; ++jj)
+      for (int jj = 0; jj < FN; ++jj)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const f32x4 v = {acc[i][jj][g * 4 + 0], acc[i][jj][g * 4 + 1], acc[i][jj][g * 4 + 2], acc[i][jj][g * 4 + 3]};
           const int chunk = jj * 8 + g * 2 + lhalf;  // 16-byte chunk of the row, XOR-ed with the row against bank conflicts
-          *(f32x4 *)(stage + srow * 64 + ((chunk ^ (srow & 15)) << 2)) = v;
+          *(f32x4 *)(stage + srow * W + ((chunk ^ (srow & (CH - 1))) << 2)) = v;
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
 #pragma nounroll
-    for (int r = er; r < ROWS; r += 4) {
+    for (int r = er; r < ROWS; r += 64 / CH) {
       const int m = m_wave + i * 32 + part * ROWS + r;
       const int n = n_wave + lc * 4;
       if (m < M && n < N) {
-        const f32x4 t = *(const f32x4 *)(stage + r * 64 + ((lc ^ (r & 15)) << 2));
+        const f32x4 t = *(const f32x4 *)(stage + r * W + ((lc ^ (r & (CH - 1))) << 2));
         float v[4] = {t[0], t[1], t[2], t[3]};
         apply_epilogue<4>(v, zrow + m, n, N - n, args.epi);
         store_from_float<4>(args.C, args.out_dtype, (zrow + m) * args.ldc + n, N - n, v);
@@ -147,33 +148,45 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
 
   // the tile buffers are too small to stage 32 rows per wave: 16 rows at a time in a buffer of their own
   __shared__ __attribute__((aligned(16))) float stage_mem[4 * 16 * 64];
-  f32_tile_epilogue<16>(acc, stage_mem + (tid >> 6) * (16 * 64), args, m0 + wm * 64, n0 + wn * 64, zrow, lane);
+  f32_tile_epilogue<16, 2, 2>(acc, stage_mem + (tid >> 6) * (16 * 64), args, m0 + wm * 64, n0 + wn * 64, zrow, lane);
 }
 
 
 // ---------------------------------------------------------------------------
 // fp32 GEMM, direct-to-LDS form.  Same product as gemm_f32_kernel, for operands
-// below 2 GiB (32-bit buffer offsets).  Tile 128x128x16, 4 waves (2x2), wave
-// tile 64x64 = 2x2 blocks of v_mfma_f32_32x32x2_f32.  Both operand tiles are
-// requested with buffer loads that write LDS directly into one of two stages
-// while the other is multiplied: one barrier per K tile, no staging registers,
-// no LDS write instructions.
-//   A tile [128 rows][16 k], 64-byte rows; piece q (16 bytes at LDS byte 16q) is
+// below 2 GiB (32-bit buffer offsets).  Tile 64T x 64T x 16 (T = 2 or 1), 4 waves
+// (2x2), wave tile 32T x 32T = TxT blocks of v_mfma_f32_32x32x2_f32.  Both operand
+// tiles are requested with buffer loads that write LDS directly into one of
+// STAGES stages while an earlier one is multiplied: one barrier per K tile, no
+// staging registers, no LDS write instructions.
+//   A tile [64T rows][16 k], 64-byte rows; piece q (16 bytes at LDS byte 16q) is
 //     row q/4, column q%4, and holds global column (q%4) ^ ((row/4)&3): the
 //     16-byte operand reads of 16 consecutive rows then fall in 16 different
 //     bank groups.
-//   B tile [16 k][128 n], 512-byte rows; piece q is k row q/32, column q%32, and
-//     holds global column (q%32) ^ (8*(row/8)): lanes 0-31 read k rows 0-7, lanes
+//   B tile [16 k][64T n], 256T-byte rows; piece q is k row q/16T, column q%16T, and
+//     holds global column (q%16T) ^ (8*(row/8)): lanes 0-31 read k rows 0-7, lanes
 //     32-63 rows 8-15 of the same 32 channels, which the XOR moves to the other
 //     half of the banks.
 // An MFMA sums over two k; lane half h supplies k = 8h + t to the t-th MFMA of a
 // K tile for A and B alike, so A's operands are two 16-byte reads per row block
 // and B's are eight 4-byte reads per channel block.
+// The 128x128 tile multiplies a K tile for 2048 cycles and runs two stages; the
+// 64x64 tile, for problems with fewer than a CU's worth of large tiles each, has
+// 512 cycles per K tile and keeps three tiles in flight (four stages) to cover
+// the latency of a request (two sub-tiles of 16 k per stage and barrier, KSUB = 2,
+// gained 3 % at 1024^3 and lost 7 % at 2048^3, where the 64 KB of LDS leave two
+// workgroups per CU instead of five).  Past the end of K the requests are still issued,
+// out of range (they write zeros to a stage nobody multiplies), so that the
+// count of outstanding requests a wave waits on is the same in every iteration.
 // ---------------------------------------------------------------------------
+template <int T, int STAGES, int KSUB>
 __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs args) {
-  constexpr int BM = F32_BM, BN = F32_BN, BK = F32_BK;
-  constexpr int A_STAGE = BM * BK * 4, B_STAGE = BK * BN * 4, STAGE = A_STAGE + B_STAGE;
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
+  constexpr int BM = 64 * T, BN = 64 * T, BK = F32_BK * KSUB;  // a stage holds KSUB sub-tiles of 16 k, each [A][B]
+  constexpr int A_STAGE = BM * F32_BK * 4, B_STAGE = F32_BK * BN * 4, SUB = A_STAGE + B_STAGE, STAGE = KSUB * SUB;
+  constexpr int B_PITCH = BN * 4, B_PIECES = BN / 4;  // bytes and 16-byte pieces per k row of B
+  static_assert(STAGES * STAGE >= 4 * 32 * 32 * T * 4, "the epilogue stages 32 rows per wave in the tile buffers");
+  static_assert((STAGES - 1) * 2 * T * KSUB < 16, "outstanding requests must fit the 4-bit wait count used here");
+  __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int wm = wave & 1, wn = wave >> 1;
@@ -188,105 +201,139 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   constexpr unsigned OOB = 0x80000000u;
   __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)args.A, 0, (int)args.a_bytes, 0x00020000);
   __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)args.B, 0, (int)args.b_bytes, 0x00020000);
-  // two pieces of A and two of B per thread and K tile
-  unsigned a_voff[2], b_voff[2];
-  int a_kcol[2], b_krow[2];
+  // T pieces of A and T of B per thread and K tile
+  unsigned a_voff[T], b_voff[T];
+  int a_kcol[T], b_krow[T];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < T; ++i) {
     const int q = tid + i * 256;
     const int row = q >> 2;
     int m = m0 + row;
     m = m < M ? m : M - 1;  // rows past the end re-read the last row; their results are never stored
     a_kcol[i] = ((q & 3) ^ ((row >> 2) & 3)) * 4;
     a_voff[i] = (unsigned)(((long long)m * args.lda + a_kcol[i]) * 4);
-    b_krow[i] = q >> 5;
-    const int n = n0 + (((q & 31) ^ ((b_krow[i] >> 3) << 3)) << 2);
+    b_krow[i] = q / B_PIECES;
+    const int n = n0 + (((q % B_PIECES) ^ ((b_krow[i] >> 3) << 3)) << 2);
     b_voff[i] = n < N ? (unsigned)(((long long)b_krow[i] * args.ldb + n) * 4) : OOB;
   }
-  auto dma = [&](unsigned char *stage, int k0) {
+  auto dma_sub = [&](unsigned char *stage, int k0) {
     k0 += kb;
+    const bool any = k0 < K;  // uniform: a tile wholly past K asks for nothing but zeros
+    const int so_a = any ? k0 * 4 : 0;
+    const int so_b = any ? (int)((long long)k0 * args.ldb * 4) : 0;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < T; ++i) {
       unsigned char *dst = stage + (i * 256 + wave_u * 64) * 16;
       const unsigned va = k0 + a_kcol[i] < K ? a_voff[i] : OOB;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void *)dst, 16, (int)va,
-                                               k0 * 4, 0, 0);
+                                               so_a, 0, 0);
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < T; ++i) {
       unsigned char *dst = stage + A_STAGE + (i * 256 + wave_u * 64) * 16;
       const unsigned vb = k0 + b_krow[i] < K ? b_voff[i] : OOB;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16, (int)vb,
-                                               (int)((long long)k0 * args.ldb * 4), 0, 0);
+                                               so_b, 0, 0);
     }
   };
+  auto dma = [&](unsigned char *stage, int k0) {
+#pragma unroll
+    for (int u = 0; u < KSUB; ++u) dma_sub(stage + u * SUB, k0 + u * F32_BK);
+  };
 
-  f32x16 acc[2][2];
+  f32x16 acc[T][T];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < T; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < T; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   const int lrow = lane & 31, lhalf = lane >> 5;
-  // A: row wm*64 + i*32 + lrow, 16-byte columns 2h and 2h+1 (k = 8h .. 8h+7)
-  int a_off[2][2];
+  // A: row wm*32T + i*32 + lrow, 16-byte columns 2h and 2h+1 (k = 8h .. 8h+7)
+  int a_off[T][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int row = wm * 64 + i * 32 + lrow;
+  for (int i = 0; i < T; ++i) {
+    const int row = wm * (32 * T) + i * 32 + lrow;
 #pragma unroll
     for (int c = 0; c < 2; ++c) a_off[i][c] = row * 64 + (((2 * lhalf + c) ^ ((row >> 2) & 3)) << 4);
   }
-  // B: k row 8h + t, channel wn*64 + j*32 + lrow
-  int b_off[2];
+  // B: k row 8h + t, channel wn*32T + j*32 + lrow
+  int b_off[T];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int n = wn * 64 + j * 32 + lrow;
-    b_off[j] = A_STAGE + (8 * lhalf) * 512 + ((((n >> 2) ^ (lhalf << 3)) << 2) + (n & 3)) * 4;
+  for (int j = 0; j < T; ++j) {
+    const int n = wn * (32 * T) + j * 32 + lrow;
+    b_off[j] = A_STAGE + (8 * lhalf) * B_PITCH + ((((n >> 2) ^ (lhalf << 3)) << 2) + (n & 3)) * 4;
   }
 
+  // Operands of tile kt+1 are read from LDS while tile kt is multiplied from registers (with one
+  // wave per SIMD nothing else would cover the latency of those reads).  Stage kt%STAGES is free
+  // once every wave has its operands of tile kt, so tile kt+STAGES is requested into it: after the
+  // prologue STAGES-1 tiles are in flight or landed beyond the one being read.
+  constexpr int PER = 2 * T * KSUB;  // requests per thread and tile; the wait count is bits 3:0 of the immediate
+  constexpr int WAIT_FIRST = 0x0f70 | ((STAGES - 1) * PER), WAIT_NEXT = 0x0f70 | ((STAGES - 2) * PER);
+  auto read_operands = [&](const unsigned char *cur, f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8]) {
+#pragma unroll
+    for (int u = 0; u < KSUB; ++u) {
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) af[u][i][c] = *(const f32x4 *)(cur + u * SUB + a_off[i][c]);
+#pragma unroll
+      for (int j = 0; j < T; ++j)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) bf[u][j][t] = *(const float *)(cur + u * SUB + b_off[j] + t * B_PITCH);
+    }
+  };
+  auto step = [&](int kt, const f32x4 (&af)[KSUB][T][2], const float (&bf)[KSUB][T][8], f32x4 (&af_next)[KSUB][T][2],
+                  float (&bf_next)[KSUB][T][8]) {
+    __builtin_amdgcn_s_waitcnt(WAIT_NEXT);  // tile kt+1 has landed (this wave's share)
+    __syncthreads();                        // ... everyone's, and everyone holds its operands of tile kt
+    dma(smem + (kt % STAGES) * STAGE, (kt + STAGES) * BK);
+    read_operands(smem + ((kt + 1) % STAGES) * STAGE, af_next, bf_next);
+#pragma unroll
+    for (int u = 0; u < KSUB; ++u)
+#pragma unroll
+      for (int t = 0; t < 8; ++t)
+#pragma unroll
+        for (int i = 0; i < T; ++i)
+#pragma unroll
+          for (int j = 0; j < T; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+  };
   const int nk = (K - kb + BK - 1) / BK;
-  dma(smem, 0);
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+#pragma unroll
+  for (int s = 0; s < STAGES; ++s) dma(smem + s * STAGE, s * BK);
+  __builtin_amdgcn_s_waitcnt(WAIT_FIRST);
   __syncthreads();
-  for (int kt = 0; kt < nk; ++kt) {
-    const unsigned char *cur = smem + (kt & 1) * STAGE;
-    if (kt + 1 < nk) dma(smem + ((kt + 1) & 1) * STAGE, (kt + 1) * BK);
-    f32x4 af[2][2];
-    float bf[2][8];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int c = 0; c < 2; ++c) af[i][c] = *(const f32x4 *)(cur + a_off[i][c]);
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int t = 0; t < 8; ++t) bf[j][t] = *(const float *)(cur + b_off[j] + t * 512);
-#pragma unroll
-    for (int t = 0; t < 8; ++t)
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[j][t], af[i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // the next tile has landed (this wave's share)
-    __syncthreads();                     // ... everyone's, and nobody still reads `cur`
+  f32x4 af0[KSUB][T][2], af1[KSUB][T][2];
+  float bf0[KSUB][T][8], bf1[KSUB][T][8];
+  read_operands(smem, af0, bf0);
+  for (int kt = 0; kt < nk; kt += 2) {
+    step(kt, af0, bf0, af1, bf1);
+    if (kt + 1 < nk) step(kt + 1, af1, bf1, af0, bf0);
   }
+  // requests past the end of K may still be writing zeros where the epilogue stages
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
 
-  f32_tile_epilogue<32>(acc, (float *)smem + wave_u * (32 * 64), args, m0 + wm * 64, n0 + wn * 64, zrow, lane);
+  f32_tile_epilogue<32, T, T>(acc, (float *)smem + wave_u * (32 * 32 * T), args, m0 + wm * (32 * T), n0 + wn * (32 * T),
+                              zrow, lane);
 }
 
-int launch_gemm_f32(const ContractionArgs &a, hipStream_t stream) {
+int launch_gemm_f32(const ContractionArgs &a, int tile, hipStream_t stream) {
   ContractionArgs args = a;
-  args.grid_m = (a.M + F32_BM - 1) / F32_BM;
-  args.grid_n = (a.N + F32_BN - 1) / F32_BN;
+  // the 64x64 tile exists in the direct-to-LDS form only (operands below 2 GiB, a_bytes / b_bytes set by the dispatcher)
+  const bool dma = a.a_bytes != 0 && a.b_bytes != 0;
+  if (tile != 64 || !dma) tile = 128;
+  args.grid_m = (a.M + tile - 1) / tile;
+  args.grid_n = (a.N + tile - 1) / tile;
   args.group_m = 4;
   const unsigned splits = a.k_split > 0 ? (unsigned)((a.K + a.k_split - 1) / a.k_split) : 1u;
   const dim3 grid((unsigned)(args.grid_m * args.grid_n), splits);
-  // a_bytes / b_bytes are set by the dispatcher when both operands are below 2 GiB
-  if (a.a_bytes != 0 && a.b_bytes != 0) hipLaunchKernelGGL(gemm_f32_dma_kernel, grid, dim3(256), 0, stream, args);
-  else hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, args);
+  if (!dma) hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, args);
+  else if (tile == 64) hipLaunchKernelGGL((gemm_f32_dma_kernel<1, 4, 1>), grid, dim3(256), 0, stream, args);
+  else hipLaunchKernelGGL((gemm_f32_dma_kernel<2, 2, 1>), grid, dim3(256), 0, stream, args);
   return (int)hipGetLastError();
 }
 
