@@ -117,7 +117,8 @@ def test_large_problems_are_not_split(tracea_gpu, split_switch):
     assert capi.lib().tracea_last_split_k() == 1
 
 
-@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (256, 256, 4096), (100, 36, 2052)])
+# shapes of few 64x64 tiles and a long K (1024^3 fills the device with 256 such tiles and is not split)
+@pytest.mark.parametrize("shape", [(512, 512, 1024), (256, 256, 4096), (100, 36, 2052)])
 def test_fp32_gemm_split_matches_float64(tracea_gpu, split_switch, shape):
     capi = split_switch
     m, n, k = shape

@@ -175,7 +175,8 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
 // 512 cycles per K tile and keeps three tiles in flight (four stages) to cover
 // the latency of a request (two sub-tiles of 16 k per stage and barrier, KSUB = 2,
 // gained 3 % at 1024^3 and lost 7 % at 2048^3, where the 64 KB of LDS leave two
-// workgroups per CU instead of five).  Past the end of K the requests are still issued,
+// workgroups per CU instead of five; a third stage for the 128x128 tile lost 2-6 %).
+// Past the end of K the requests are still issued,
 // out of range (they write zeros to a stage nobody multiplies), so that the
 // count of outstanding requests a wave waits on is the same in every iteration.
 // ---------------------------------------------------------------------------
@@ -287,6 +288,20 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   };
   auto step = [&](int kt, const f32x4 (&af)[KSUB][T][2], const float (&bf)[KSUB][T][8], f32x4 (&af_next)[KSUB][T][2],
                   float (&bf_next)[KSUB][T][8]) {
+    // first half of tile kt's MFMAs, then the barrier, the requests and the operand reads of tile
+    // kt+1 spread between the MFMAs of the second half: with one wave per SIMD whatever is issued
+    // between two barriers without an MFMA in flight is time the matrix pipe stands still
+    auto mfma = [&](int u, int t) {
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+    };
+#pragma unroll
+    for (int u = 0; u < KSUB; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) mfma(u, t);
     __builtin_amdgcn_s_waitcnt(WAIT_NEXT);  // tile kt+1 has landed (this wave's share)
     __syncthreads();                        // ... everyone's, and everyone holds its operands of tile kt
     dma(smem + (kt % STAGES) * STAGE, (kt + STAGES) * BK);
@@ -294,12 +309,13 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
 #pragma unroll
     for (int u = 0; u < KSUB; ++u)
 #pragma unroll
-      for (int t = 0; t < 8; ++t)
+      for (int t = 4; t < 8; ++t) mfma(u, t);
+    __builtin_amdgcn_sched_group_barrier(0x020, 2 * T * KSUB, 0);  // the requests first
 #pragma unroll
-        for (int i = 0; i < T; ++i)
-#pragma unroll
-          for (int j = 0; j < T; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+    for (int q = 0; q < 4 * T * T * KSUB; ++q) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, T == 1 ? 3 : 2, 0);
+    }
   };
   const int nk = (K - kb + BK - 1) / BK;
 #pragma unroll
