@@ -6,7 +6,7 @@ fp32 accumulate, fp16 output); the 3x3 implicit-GEMM convolution and the
 FlashAttention-2 forward named by the metric are timed in the same run and
 reported under "also".  Prints one JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_rowmajor|gemm_f32|gemm_f32_4096|conv|attention|attention_causal|conv_transpose|resnet18_b1|resnet18_b32|copy]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload gemm|gemm_nonsquare|gemm_rowmajor|gemm_f32|gemm_f32_4096|conv|attention|attention_causal|conv_transpose|resnet18_b1|resnet18_b32|copy]
 """
 import argparse
 import json
@@ -38,6 +38,15 @@ def make_workload(name, torch, ops):
         c = torch.empty(m, n, device=dev, dtype=torch.float16)
         b = bt.t()
         return ("fp16 GEMM 4096x4096x4096, A row-major, B column-major, fp32 acc, fp16 out",
+                2.0 * m * n * k, 2.0 * (m * k + k * n + m * n), "f16", lambda: ops.gemm(a, b, out=c))
+    if name == "gemm_nonsquare":
+        # the second shape of the fp16 GEMM configuration, there to exercise the choice of tile shape
+        m, n, k = 8192, 2048, 8192
+        a = (torch.randn(m, k, device=dev, generator=g) / k ** 0.5).half()
+        bt = (torch.randn(n, k, device=dev, generator=g) / k ** 0.5).half()
+        c = torch.empty(m, n, device=dev, dtype=torch.float16)
+        b = bt.t()
+        return ("fp16 GEMM 8192x2048x8192, A row-major, B column-major, fp32 acc, fp16 out",
                 2.0 * m * n * k, 2.0 * (m * k + k * n + m * n), "f16", lambda: ops.gemm(a, b, out=c))
     if name == "gemm_rowmajor":
         # the same product with B stored [K,N] row-major, the layout the reference's tracea_gemm documents
@@ -261,7 +270,7 @@ def main():
     if not args.no_extras:
         cpu = cpu_baseline()
         also = {}
-        for name in ("gemm", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "basic_block", "downsample_block", "attention", "attention_causal",
+        for name in ("gemm", "gemm_nonsquare", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "basic_block", "downsample_block", "attention", "attention_causal",
                      "conv_transpose", "resnet18_b1", "resnet18_b32", "gemm_tiles_half"):
             if name == args.workload:
                 continue

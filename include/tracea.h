@@ -292,7 +292,8 @@ TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaT
 
 
 /* Split-K.  A gemm / conv2d launch with few output tiles and a long K (tiles * 2 <= 256 CUs,
- * at least 8 K tiles) is split along K over more workgroups; fp32 partial products go to a
+ * at least 8 K tiles; 32 K tiles of 16 for the 64x64 tile of the fp32 GEMM) is split along K
+ * over more workgroups; fp32 partial products go to a
  * scratch buffer the library keeps per (device, stream) (grown on demand up to 64 MiB, never
  * while the stream is being captured, never freed) and a second kernel sums them and applies
  * the operator chain.  On by default; tracea_set_split_k(0) turns it off.
