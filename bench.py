@@ -193,6 +193,34 @@ def time_steps(torch, step, steps, warmup):
     return wall / steps, e0.elapsed_time(e1) * 1e-3 / steps
 
 
+def launch_stats(torch, step, launches=50, cold_trials=5):
+    """Per-launch figures of the timing protocol: median and minimum over `launches` back-to-back
+    launches (one event between each pair; caches are not flushed between them), and the median of
+    `cold_trials` single launches that each follow a 1 GiB fill, which leaves nothing of the
+    operands in the 32 MB of L2 or the 256 MB memory-side cache."""
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(launches + 1)]
+    ev[0].record()
+    for i in range(launches):
+        step()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    ts = sorted(ev[i].elapsed_time(ev[i + 1]) * 1e3 for i in range(launches))
+    flush = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0")
+    cold = []
+    for i in range(cold_trials):
+        flush.fill_(i)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        step()
+        e1.record()
+        torch.cuda.synchronize()
+        cold.append(e0.elapsed_time(e1) * 1e3)
+    del flush
+    return {"median": round(ts[len(ts) // 2], 2), "min": round(ts[0], 2), "cold_cache": round(sorted(cold)[len(cold) // 2], 2),
+            "launches": launches}
+
+
 def time_steps_graph(torch, step, steps):
     """The same launches recorded once into a HIP graph and replayed: device time per launch without
     the host's per-call cost (about 15 us per call from Python here, which is longer than the shorter
@@ -290,6 +318,7 @@ def main():
     wall, dev_s = time_steps(torch, step, args.steps, args.warmup)
     tflops = flops / wall / 1e12
     achieved = flops / dev_s / 1e12
+    stats = launch_stats(torch, step)
     line = {
         "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOPS", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 5),
@@ -301,6 +330,7 @@ def main():
                      "traffic": TRAFFIC_BYTES.get(args.workload),
                      "hbm_GBps_algorithmic": round(bytes_ / dev_s / 1e9, 1)},
     }
+    line["launch_us"] = stats
     if not args.no_extras:
         line["also"] = also
         line["cpu_baseline"] = cpu
