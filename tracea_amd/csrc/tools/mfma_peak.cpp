@@ -110,6 +110,68 @@ __global__ void __launch_bounds__(256) mfma_mix_loop(const half8 *src, float *si
   if (s == 12345.678f) sink[tid] = s;
 }
 
+// The same with v_mfma_f32_16x16x32_f16: 32 MFMAs per iteration (8 A fragments x 4 B fragments of a
+// 128x64 wave tile over 32 k: twice the flops of the loop above), hence R = 12 reads and G = 4 requests
+// for the same bytes per flop.
+template <int R, int G>
+__global__ void __launch_bounds__(256) mfma_mix_loop16(const half8 *src, float *sink, int iters) {
+  __shared__ half8 lds[4096];  // 64 KB
+  const int tid = blockIdx.x * 256 + threadIdx.x, t = threadIdx.x;
+  for (int i = t; i < 4096; i += 256) lds[i] = src[(blockIdx.x * 4096 + i) & 0xfffff];
+  __syncthreads();
+  half8 f[12];
+  for (int i = 0; i < 12; ++i) f[i] = src[(tid * 12 + i) & 0xfffff];
+  float4v acc[8][4];
+  for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < 4; ++j)
+      for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
+  __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void *)src, 0, 1 << 24, 0x00020000);
+  int off = t;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) f[r % 12] = lds[(off + r * 256) & 4095];
+    off += 67;
+    if constexpr (G > 0) {
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rs, (__attribute__((address_space(3))) void *)(lds + ((g * 256 + (t & ~63)) & 4095)), 16,
+            ((it * 8 + g) * 4096 + tid * 16) & 0xffffff, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(f[8 + j], f[i], acc[i][j], 0, 0, 0);
+    if constexpr (G > 0) {
+      if ((it & 3) == 3) __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): bounds the requests in flight
+    }
+  }
+  float s = 0.f;
+  for (int i = 0; i < 8; ++i)
+    for (int j = 0; j < 4; ++j)
+      for (int e = 0; e < 4; ++e) s += acc[i][j][e];
+  if (s == 12345.678f) sink[tid] = s;
+}
+
+template <int R, int G>
+static int run_mix16(const half8 *src, float *sink, int blocks, int iters, int launches, const char *what) {
+  hipEvent_t e0, e1;
+  CHECK(hipEventCreate(&e0));
+  CHECK(hipEventCreate(&e1));
+  float ms = 0.f;
+  for (int rep = 0; rep < 2; ++rep) {
+    CHECK(hipEventRecord(e0));
+    for (int q = 0; q < launches; ++q) hipLaunchKernelGGL((mfma_mix_loop16<R, G>), dim3(blocks), dim3(256), 0, 0, src, sink, iters);
+    CHECK(hipGetLastError());
+    CHECK(hipEventRecord(e1));
+    CHECK(hipEventSynchronize(e1));
+    CHECK(hipEventElapsedTime(&ms, e0, e1));
+  }
+  std::printf("N(0,1)/64, 16x16x32, %-44s %7.2f ms, %6.0f TFLOP/s\n", what, ms,
+              (double)launches * blocks * 4.0 * iters * 32.0 * 16384.0 / ms / 1e9);
+  return 0;
+}
+
 template <int R, int G>
 static int run_mix(const half8 *src, float *sink, int blocks, int iters, int launches, const char *what) {
   hipEvent_t e0, e1;
@@ -179,5 +241,10 @@ int main() {
   if (run_mix<0, 2>(src, sink, blocks, iters, launches, "2 tile requests per 8 MFMAs")) return 1;
   if (run_mix<4, 2>(src, sink, blocks, iters, launches, "4 LDS reads + 2 tile requests per 8 MFMAs")) return 1;
   if (run_mix<6, 2>(src, sink, blocks, iters, launches, "6 LDS reads + 2 tile requests per 8 MFMAs")) return 1;
+  if (run_mix16<0, 0>(src, sink, blocks, iters / 2, launches, "no data movement")) return 1;
+  if (run_mix16<12, 0>(src, sink, blocks, iters / 2, launches, "12 LDS reads per 32 MFMAs")) return 1;
+  if (run_mix16<0, 4>(src, sink, blocks, iters / 2, launches, "4 tile requests per 32 MFMAs")) return 1;
+  if (run_mix16<12, 4>(src, sink, blocks, iters / 2, launches, "12 LDS reads + 4 tile requests per 32 MFMAs")) return 1;
+  if (run_mix16<8, 4>(src, sink, blocks, iters / 2, launches, "8 LDS reads + 4 tile requests per 32 MFMAs")) return 1;
   return 0;
 }
