@@ -1209,6 +1209,14 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     if (tid + i * NT < TAB_ENTRIES) table[tid + i * NT] = tabr[i];
   __syncthreads();
   const float *tab = table + wn * TN + ec;
+  // The row map's parameters as scalars of their own: read through `args` inside the row
+  // lambdas below, with more than one 32-row block per wave, they made the compiler keep a copy
+  // of the whole argument block in scratch memory (568 bytes per lane, every later argument read
+  // a scratch load) and the convolution ran at half speed.
+  const bool om_on = CONV && args.out_map != 0;
+  const unsigned om_hw_m = args.hw_m, om_hw_s = args.hw_s, om_w_m = args.w_m, om_w_s = args.w_s;
+  const int om_hw = args.h_out * args.w_out, om_w = args.w_out, om_sh = args.o_sh, om_sw = args.o_sw, om_wo = args.o_wo;
+  const long long om_img = args.o_img;
   static_for<0, FM>([&](auto blk) {
     constexpr int i = decltype(blk)::value;
     static_for<0, FN>([&](auto col) {
@@ -1231,11 +1239,11 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // transposed convolution writing its share of the full output).
     auto out_row = [&](int m) -> long long {
       if constexpr (CONV) {
-        if (args.out_map != 0) {
+        if (om_on) {
           int img, rem, q, pcol;
-          fast_divmod(m, args.hw_m, args.hw_s, args.h_out * args.w_out, img, rem);
-          fast_divmod(rem, args.w_m, args.w_s, args.w_out, q, pcol);
-          return (long long)img * args.o_img + (long long)(o_a + args.o_sh * q) * args.o_wo + o_b + args.o_sw * pcol;
+          fast_divmod(m, om_hw_m, om_hw_s, om_hw, img, rem);
+          fast_divmod(rem, om_w_m, om_w_s, om_w, q, pcol);
+          return (long long)img * om_img + (long long)(o_a + om_sh * q) * om_wo + o_b + om_sw * pcol;
         }
       }
       return zrow + m;
