@@ -8,6 +8,7 @@ without a GPU, so this runs on any machine with ROCm installed.  Each line of
 import argparse
 import concurrent.futures
 import hashlib
+import json
 import os
 import re
 import subprocess
@@ -81,15 +82,42 @@ def _jobs():
 def _compile(job, digest, force):
     src, obj, flags = job
     stamp = obj + ".stamp"
+    device = "--offload-arch=" + ARCH in flags
     key = hashlib.sha1((digest + open(src, "rb").read().hex() + " ".join(flags)).encode()).hexdigest()
-    if not force and os.path.exists(obj) and os.path.exists(stamp) and open(stamp).read() == key:
+    if (not force and os.path.exists(obj) and os.path.exists(stamp) and open(stamp).read() == key and
+            (not device or os.path.exists(obj + ".resources.json"))):
         return obj, False
-    cmd = [hipcc()] + COMMON + flags + ["-c", src, "-o", obj]
+    cmd = [hipcc()] + COMMON + flags + (["-Rpass-analysis=kernel-resource-usage"] if device else []) + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("compile failed: %s\n%s" % (" ".join(cmd), r.stderr[-4000:]))
+    if device:
+        with open(obj + ".resources.json", "w") as f:
+            json.dump(_kernel_resources(r.stderr), f)
     open(stamp, "w").write(key)
     return obj, True
+
+
+_REMARK = re.compile(r"remark:\s+(Function Name|VGPRs|AGPRs|ScratchSize \[bytes/lane\]|VGPRs Spill|"
+                     r"LDS Size \[bytes/block\]|Occupancy \[waves/SIMD\]): (\S+)")
+_FIELDS = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch_bytes", "VGPRs Spill": "vgpr_spills",
+           "LDS Size [bytes/block]": "lds_bytes", "Occupancy [waves/SIMD]": "waves_per_simd"}
+
+
+def _kernel_resources(remarks):
+    """What the compiler reports per kernel (-Rpass-analysis=kernel-resource-usage): registers,
+    scratch bytes per lane, static LDS.  A kernel of this library that needs scratch memory has
+    always been a mistake in its source (a run-time index into registers or into the argument
+    block), costing a factor of two: the numbers are kept so that a test can watch them."""
+    out, cur = [], None
+    for m in _REMARK.finditer(remarks):
+        key, val = m.group(1), m.group(2)
+        if key == "Function Name":
+            cur = {"name": val}
+            out.append(cur)
+        elif cur is not None:
+            cur[_FIELDS[key]] = int(val)
+    return out
 
 
 def build(force=False, jobs=None, verbose=True):
@@ -104,6 +132,14 @@ def build(force=False, jobs=None, verbose=True):
         for obj, did in ex.map(lambda j: _compile(j, digest, force), todo):
             objs.append(obj)
             rebuilt += int(did)
+    # per-kernel resource usage of everything that goes into the library, next to it
+    resources = {}
+    for obj in objs:
+        if os.path.exists(obj + ".resources.json"):
+            for k in json.load(open(obj + ".resources.json")):
+                resources[k["name"]] = {f: v for f, v in k.items() if f != "name"}
+    with open(os.path.join(LIB_DIR, "kernel_resources.json"), "w") as f:
+        json.dump(resources, f, indent=0, sort_keys=True)
     if rebuilt or force or not os.path.exists(LIB):
         cmd = [hipcc(), "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o", LIB] + objs
         r = subprocess.run(cmd, capture_output=True, text=True)
