@@ -1497,7 +1497,10 @@ TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const Ep
         for (int i = 0; i < sw; ++i) c.phase_pad_w[i] = phase_axis(i, sw, plan.pad_w, S, Wo).pad;
       }
       c.epi = chain;
-      int vi = select_contraction_variant(c.M, c.N, c.K, true);
+      // uniform phases go out as one launch: the selector sees the rows of all of them
+      // (VAE layer 65.2 -> 53.8 us on 128x128 tiles instead of 128x64)
+      const long long m_launch = uniform ? (long long)c.M * sh * sw : (long long)c.M;
+      int vi = select_contraction_variant((int)(m_launch < (1ll << 31) - 1 ? m_launch : (1ll << 31) - 1), c.N, c.K, true);
       if (vi < 0) { st = fail(TRACEA_UNKNOWN_ERROR, "tracea_conv_transpose2d: no kernel variant available"); break; }
       const long long w_extent = (long long)K * kg * 2;
       const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
