@@ -76,3 +76,15 @@ def test_patch_and_unpatch():
     finally:
         tracea.unpatch_conv2d()
     assert torch.nn.Conv2d is original
+
+
+def test_operator_arrays_refuse_half_precision_channel_vectors():
+    # BatchNorm / scale-shift vectors are read as fp32 by the kernels; model.half() leaves them f16
+    from tracea_amd import ops
+    v16, v32 = torch.ones(8, dtype=torch.float16), torch.ones(8)
+    with pytest.raises(ValueError):
+        ops._ops_array([(capi.OP_BATCHNORM, v32, v32, v16, v32, 1e-5)])
+    with pytest.raises(ValueError):
+        ops._ops_array([(capi.OP_SCALE_SHIFT, v16, v16)])
+    arr, keep = ops._ops_array([(capi.OP_SCALE_SHIFT, v32, v32), (capi.OP_BIAS_ADD, v16)])
+    assert arr[0].dtype == capi.F32 and arr[1].dtype == capi.F16 and len(keep) == 3

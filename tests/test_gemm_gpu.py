@@ -188,6 +188,29 @@ def test_error_paths(tracea_gpu):
     assert st == capi.INVALID_PARAMS
 
 
+def test_half_precision_batchnorm_parameters_are_refused(tracea_gpu):
+    # the kernels read BatchNorm / scale-shift vectors as fp32: the library refuses an operator
+    # that names another type (straight through the C ABI, past the Python wrapper's own check)
+    from tracea_amd import capi
+    from tracea_amd import ops as raw
+    a = torch.zeros(64, 64, device="cuda", dtype=torch.float16)
+    out = torch.empty(64, 64, device="cuda", dtype=torch.float16)
+    vec = torch.ones(64, device="cuda", dtype=torch.float16)
+    for kind, n_tensors in ((capi.OP_BATCHNORM, 4), (capi.OP_SCALE_SHIFT, 2)):
+        arr = (capi.EpilogueOp * 1)()
+        arr[0].kind = kind
+        arr[0].dtype = capi.F16
+        for slot in ("p0", "p1", "p2", "p3")[:n_tensors]:
+            setattr(arr[0], slot, vec.data_ptr())
+        arr[0].epsilon = 1e-5
+        va, vb, vc = raw._view(a), raw._view(a.t()), raw._view(out)
+        st = capi.lib().tracea_gemm_ex(va.c, vb.c, C.byref(vc.c), capi.GemmParams(0, None), arr, 1)
+        assert st == capi.UNSUPPORTED_CONFIG
+        assert "float32" in capi.last_error()
+    with pytest.raises(ValueError):
+        tracea_gpu.gemm_ex(a, a.t(), [(capi.OP_SCALE_SHIFT, vec, vec)])
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16"])
 def test_operand_beyond_2gib_takes_the_register_staged_kernels(tracea_gpu, dtype):
     # the direct-to-LDS kernels address operands with 32-bit byte offsets; an A whose rows are spread

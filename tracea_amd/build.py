@@ -155,14 +155,6 @@ def build(force=False, jobs=None, verbose=True):
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("tuner link failed:\n" + r.stderr[-4000:])
-    # calibration probe for the matrix-pipe roofline (register-only MFMA loop, stand-alone)
-    src = os.path.join(CSRC, "tools", "mfma_peak.cpp")
-    probe = os.path.join(BIN_DIR, "mfma-peak")
-    if force or not os.path.exists(probe) or os.path.getmtime(probe) < os.path.getmtime(src):
-        cmd = [hipcc(), "-O3", "-x", "hip", "--offload-arch=" + ARCH] + DEVICE_FLAGS + [src, "-o", probe]
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("mfma-peak build failed:\n" + r.stderr[-4000:])
     if verbose:
         print("libtracea.so: %d of %d objects rebuilt -> %s" % (rebuilt, len(todo), LIB))
     return LIB

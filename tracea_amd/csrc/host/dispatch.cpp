@@ -171,11 +171,18 @@ TraceaStatus lower_chain(const char *what, const TraceaEpilogueOp *ops, uint32_t
       case TRACEA_EPI_OP_BATCHNORM:
         if (!op.p0 || !op.p1 || !op.p2 || !op.p3)
           return fail(TRACEA_INVALID_PARAMS, "%s: BatchNorm needs gamma, beta, mean and var", what);
+        // the kernels read these vectors as fp32 whatever the operator says: anything else is refused
+        if (op.dtype != TRACEA_DTYPE_FLOAT32)
+          return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: epilogue operator %u: BatchNorm parameters must be float32, not %s",
+                      what, i, dtype_name(op.dtype));
         d.p0 = op.p0; d.p1 = op.p1; d.p2 = op.p2; d.p3 = op.p3;
         break;
       case TRACEA_EPI_OP_SCALE_SHIFT:
         if (!op.p0 || !op.p1)
           return fail(TRACEA_INVALID_PARAMS, "%s: ScaleShift needs scale and shift", what);
+        if (op.dtype != TRACEA_DTYPE_FLOAT32)
+          return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: epilogue operator %u: scale and shift must be float32, not %s",
+                      what, i, dtype_name(op.dtype));
         d.p0 = op.p0; d.p1 = op.p1;
         break;
       default:

@@ -155,6 +155,13 @@ def _ops_array(ops):
         kind = op[0]
         tensors = [t for t in op[1:] if isinstance(t, torch.Tensor)]
         scalars = [t for t in op[1:] if not isinstance(t, torch.Tensor)]
+        if kind in (capi.OP_BATCHNORM, capi.OP_SCALE_SHIFT):
+            # the kernels read these per-channel vectors as fp32 (the library refuses anything else);
+            # all of them are checked here, the library only sees the first one's type
+            for t in tensors:
+                if t.dtype != torch.float32:
+                    raise ValueError("BatchNorm / scale-shift parameters must be float32 tensors, got %s "
+                                     "(convert once with .float())" % (t.dtype,))
         arr[i].kind = kind
         arr[i].dtype = _DTYPES[tensors[0].dtype] if tensors else capi.F32
         for slot, t in zip(("p0", "p1", "p2", "p3"), tensors):
