@@ -308,6 +308,25 @@ void tracea_set_split_k(int32_t enabled);
 void tracea_set_conv_transpose_by_phase(int32_t enabled);
 int32_t tracea_last_split_k(void);
 
+/* tracea_gemm for callers that cannot allocate device memory: code whose stream is being
+ * captured into a HIP graph, tight serving loops, harnesses that forbid hipMalloc.  No
+ * counterpart in the reference (its runtime allocates freely).  Arguments, results and errors
+ * are those of tracea_gemm, and the same kernels run; the only difference is where the fp32
+ * partial products of a launch split along K go: into a workspace of
+ * TRACEA_STATIC_SCRATCH_BYTES that is part of the library's device image (one copy per GPU,
+ * held until the process ends) instead of the per-stream buffer that tracea_gemm grows on
+ * demand.  The call makes no hipMalloc / hipFree and no allocating library call.  A launch
+ * whose split would need more than the workspace holds (splits * M * N * 4 bytes) returns
+ * TRACEA_UNSUPPORTED_CONFIG with the two sizes in the error text; launches that are not split
+ * need no workspace and have no limit.  All calls on one GPU share that GPU's workspace, on
+ * every stream: two such calls that may overlap in time on one GPU race on it, so issue them on
+ * one stream or order them with events.  Nothing in the workspace needs to start at zero (every
+ * element the reduction reads is written by the launch before it). */
+#define TRACEA_STATIC_SCRATCH_BYTES (16u << 20)
+TraceaStatus tracea_gemm_noalloc(TraceaTensorView a, TraceaTensorView b, const TraceaTensorView *bias,
+                                 const TraceaTensorView *residual, TraceaTensorView *c,
+                                 TraceaGemmParams params);
+
 /* Kernel-variant control for tuners and benchmarks.  `op` is "gemm", "conv2d"
  * or "attention".  A variant forced with tracea_force_variant (index >= 0) is
  * used by every later call of that operator in the process whenever it is

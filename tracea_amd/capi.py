@@ -81,6 +81,8 @@ SIGNATURES = {
                                           ConvTranspose2dParams]),
     "tracea_gemm": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), C.POINTER(TensorView),
                               C.POINTER(TensorView), GemmParams]),
+    "tracea_gemm_noalloc": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), C.POINTER(TensorView),
+                                      C.POINTER(TensorView), GemmParams]),
     "tracea_attention": (C.c_int, [TensorView, TensorView, TensorView, C.POINTER(TensorView),
                                    AttentionParams]),
     "tracea_get_last_error": (C.c_int32, [C.c_char_p, C.c_size_t]),

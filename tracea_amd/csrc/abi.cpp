@@ -91,6 +91,12 @@ TraceaStatus tracea_gemm(TraceaTensorView a, TraceaTensorView b, const TraceaTen
   TRACEA_GUARDED(dispatch_gemm_kind(a, b, bias, residual, c, params))
 }
 
+TraceaStatus tracea_gemm_noalloc(TraceaTensorView a, TraceaTensorView b, const TraceaTensorView *bias,
+                                 const TraceaTensorView *residual, TraceaTensorView *c,
+                                 TraceaGemmParams params) {
+  TRACEA_GUARDED(dispatch_gemm_kind(a, b, bias, residual, c, params, true))
+}
+
 TraceaStatus tracea_gemm_ex(TraceaTensorView a, TraceaTensorView b, TraceaTensorView *c,
                             TraceaGemmParams params, const TraceaEpilogueOp *ops, uint32_t n_ops) {
   TRACEA_GUARDED(dispatch_gemm_ops(a, b, c, params, ops, n_ops))

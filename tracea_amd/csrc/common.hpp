@@ -126,6 +126,10 @@ struct SplitKReduceArgs {
 };
 int launch_splitk_reduce(const SplitKReduceArgs &args, hipStream_t stream);
 
+// Device address of the calling process's copy of the static split-K workspace
+// (TRACEA_STATIC_SCRATCH_BYTES) on `device`; returns hipError_t as int.
+int static_scratch_address(int device, void **ptr);
+
 // Second stage of the transposed convolution: gathers the per-tap partial
 // products `cols` (one row per input pixel, one column per (r, s, k)) into the
 // output pixels and applies the operator chain.

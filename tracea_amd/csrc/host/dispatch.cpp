@@ -501,12 +501,35 @@ void *splitk_scratch(int device, hipStream_t stream, size_t bytes) {
 
 // Launches `args` on variant v, split along K when that pays; `chain` is the operator chain
 // of the call (args.epi is ignored).
+// The workspace of a launch split `splits` ways: the per-stream buffer (null when it cannot be had:
+// the launch then runs unsplit), or, for the entry point that must not allocate, the static one,
+// where a workspace that does not fit is an error (*st).
+void *split_workspace(const char *what, bool static_only, int device, hipStream_t stream, int splits, long long M,
+                      long long N, TraceaStatus *st) {
+  *st = TRACEA_SUCCESS;
+  if (splits <= 1) return nullptr;
+  const size_t bytes = (size_t)splits * (size_t)M * (size_t)N * 4;
+  if (!static_only) return splitk_scratch(device, stream, bytes);
+  if (bytes > (size_t)TRACEA_STATIC_SCRATCH_BYTES) {
+    *st = fail(TRACEA_UNSUPPORTED_CONFIG,
+               "%s: the launch is split %d ways along K and needs a workspace of %zu bytes; the static workspace "
+               "of the no-allocation entry point holds %zu", what, splits, bytes, (size_t)TRACEA_STATIC_SCRATCH_BYTES);
+    return nullptr;
+  }
+  void *p = nullptr;
+  const int e = static_scratch_address(device, &p);
+  if (e != 0) *st = hip_status("static workspace address", e);
+  return p;
+}
+
 TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, ContractionArgs args,
                                 const EpilogueChain &chain, bool conv, int dtype, bool b_ncontig, int device,
-                                hipStream_t stream) {
+                                hipStream_t stream, bool static_only = false) {
   int k_split = 0;
   const int splits = g_split_k_enabled.load() ? choose_split(v, args.M, args.N, args.K, &k_split) : 1;
-  void *scratch = splits > 1 ? splitk_scratch(device, stream, (size_t)splits * args.M * args.N * 4) : nullptr;
+  TraceaStatus ws = TRACEA_SUCCESS;
+  void *scratch = split_workspace(what, static_only, device, stream, splits, args.M, args.N, &ws);
+  if (ws != TRACEA_SUCCESS) return ws;
   t_last_splits = scratch != nullptr ? splits : 1;
   if (scratch == nullptr) {
     args.epi = chain;
@@ -530,7 +553,7 @@ TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, C
 
 // ---- GEMM ----------------------------------------------------------------------
 TraceaStatus run_gemm(const View &a, const View &b, const View &c, const EpilogueChain &chain,
-                      hipStream_t stream) {
+                      hipStream_t stream, bool static_only = false) {
   const long long M = a.shape[0], K = a.shape[1], N = b.shape[1];
   t_last_contraction = -1;
   if (M == 0 || N == 0) return TRACEA_SUCCESS;
@@ -565,7 +588,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.b_bytes = (unsigned)(small ? b_extent : 0);
       fill_grid(&args, v);
       t_last_contraction = vi;
-      return launch_maybe_split("gemm launch", v, args, chain, false, a.dtype, !b_kcontig, c.device, stream);
+      return launch_maybe_split("gemm launch", v, args, chain, false, a.dtype, !b_kcontig, c.device, stream, static_only);
     }
   }
   if (a.dtype == TRACEA_DTYPE_FLOAT32 && b.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32 && K > 0 &&
@@ -595,7 +618,9 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     const ContractionVariant &f32_tile = tile == 64 ? f32_tile64 : f32_tile128;
     int k_split = 0;
     const int splits = g_split_k_enabled.load() ? choose_split(f32_tile, (int)M, (int)N, (int)K, &k_split, tile == 64 ? 16 : 4) : 1;
-    void *scratch = splits > 1 ? splitk_scratch(c.device, stream, (size_t)splits * M * N * 4) : nullptr;
+    TraceaStatus ws = TRACEA_SUCCESS;
+    void *scratch = split_workspace("gemm_f32 launch", static_only, c.device, stream, splits, M, N, &ws);
+    if (ws != TRACEA_SUCCESS) return ws;
     t_last_splits = scratch != nullptr ? splits : 1;
     if (scratch == nullptr) {
       args.epi = chain;
@@ -651,7 +676,7 @@ TraceaStatus gemm_common(const TraceaTensorView &ta, const TraceaTensorView &tb,
 
 TraceaStatus dispatch_gemm_kind(const TraceaTensorView &ta, const TraceaTensorView &tb,
                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
-                                TraceaTensorView *tc, const TraceaGemmParams &params) {
+                                TraceaTensorView *tc, const TraceaGemmParams &params, bool static_only) {
   View a, b, c;
   TraceaStatus st = gemm_common(ta, tb, tc, &a, &b, &c);
   if (st != TRACEA_SUCCESS) return st;
@@ -663,7 +688,7 @@ TraceaStatus dispatch_gemm_kind(const TraceaTensorView &ta, const TraceaTensorVi
   EpilogueChain chain{};
   st = lower_chain("tracea_gemm", ops, (uint32_t)n, c.shape[1], c.shape[1], &chain);
   if (st != TRACEA_SUCCESS) return st;
-  return run_gemm(a, b, c, chain, (hipStream_t)params.stream);
+  return run_gemm(a, b, c, chain, (hipStream_t)params.stream, static_only);
 }
 
 TraceaStatus dispatch_gemm_ops(const TraceaTensorView &ta, const TraceaTensorView &tb,

@@ -43,7 +43,7 @@ int last_split_k();
 
 TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorView &b,
                                 const TraceaTensorView *bias, const TraceaTensorView *residual,
-                                TraceaTensorView *c, const TraceaGemmParams &params);
+                                TraceaTensorView *c, const TraceaGemmParams &params, bool static_only = false);
 TraceaStatus dispatch_gemm_ops(const TraceaTensorView &a, const TraceaTensorView &b,
                                TraceaTensorView *c, const TraceaGemmParams &params,
                                const TraceaEpilogueOp *ops, uint32_t n_ops);

@@ -1,5 +1,7 @@
 // Kernels around the half-precision MFMA family: the fp32 GEMM, the
 // any-layout fallback GEMM and the coordinate-table dump of the convolution.
+#include <mutex>
+
 #include "contraction_kernel.hpp"
 
 namespace tracea_amd {
@@ -443,6 +445,39 @@ int launch_splitk_reduce(const SplitKReduceArgs &a, hipStream_t stream) {
   if (vec) hipLaunchKernelGGL(splitk_reduce_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(splitk_reduce_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
   return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// Split-K workspace for callers that cannot allocate device memory (code under HIP
+// graph capture, serving loops, harnesses that forbid hipMalloc): a file-scope device
+// array instead of the per-stream buffer the other entry points grow on demand.  Every
+// GPU the library runs on holds its own copy of the array, at its own address, until the
+// process ends.  In host code the array's name is only a stand-in for the symbol: the
+// address kernels may use comes from hipGetSymbolAddress, asked once per device with that
+// device current, and is what every launch and copy is given.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[TRACEA_STATIC_SCRATCH_BYTES];
+
+int static_scratch_address(int device, void **ptr) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static void *address[kMaxDevices] = {};
+  if (device < 0 || device >= kMaxDevices) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (address[device] == nullptr) {
+    int current = -1;
+    hipError_t e = hipGetDevice(&current);
+    if (e != hipSuccess) return (int)e;
+    if (current != device && (e = hipSetDevice(device)) != hipSuccess) return (int)e;
+    void *p = nullptr;
+    e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+    if (current != device) (void)hipSetDevice(current);
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return (int)hipErrorInvalidSymbol;
+    address[device] = p;
+  }
+  *ptr = address[device];
+  return 0;
 }
 
 // ---------------------------------------------------------------------------

@@ -81,6 +81,20 @@ def gemm(a, b, out=None, bias=None, residual=None, epilogue="none", out_dtype=No
     return out
 
 
+def gemm_noalloc(a, b, out, bias=None, residual=None, epilogue="none"):
+    """tracea_gemm_noalloc: as :func:`gemm` with the split-K workspace taken from the library's
+    static device array.  ``out`` is required (this wrapper allocates no device memory either);
+    calls that may overlap on one GPU share the workspace and must be ordered by the caller."""
+    va, vb, vc = _view(a), _view(b), _view(out)
+    vbias = _view(bias) if bias is not None else None
+    vres = _view(residual) if residual is not None else None
+    params = capi.GemmParams(parse_epilogue(epilogue), _stream(a))
+    st = capi.lib().tracea_gemm_noalloc(va.c, vb.c, C.byref(vbias.c) if vbias else None,
+                                        C.byref(vres.c) if vres else None, C.byref(vc.c), params)
+    capi.check("tracea_gemm_noalloc", st)
+    return out
+
+
 def low_rank_mlp(x, a, b, out=None, bias=None, residual=None, epilogue="none", out_dtype=None):
     """out[M,N] = epilogue((x[M,K] @ a[K,R]) @ b[R,N]); the rank-R product is rounded to the
     operands' type in between (the reference's LowRankMlp operator)."""
