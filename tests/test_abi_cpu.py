@@ -113,7 +113,8 @@ def test_conv_params_block_equals_oracle_bit_for_bit(shape):
 def test_variant_table():
     gemm = capi.variants("gemm")
     assert gemm and gemm == capi.variants("conv2d")
-    assert all(re.match(r"t\d+x\d+x\d+_w\dx\d", n) or re.match(r"c\d+x\d+_w\dx\d_s\d_patch", n) for n in gemm)
+    assert all(re.match(r"t\d+x\d+x\d+_w\dx\d", n) or re.match(r"c\d+x\d+_w\dx\d_s\d_patch", n) or
+               re.match(r"c\d+x\d+_k\d+_resident", n) for n in gemm)
     attn = capi.variants("attention")
     assert any("d128" in n for n in attn)
     l = capi.lib()

@@ -135,6 +135,106 @@ def test_patch_resident_variants(tracea_gpu, dtype):
     assert {names[i] for i in patch} <= ran, "a patch-resident variant never ran: %s" % sorted(ran)
 
 
+RESIDENT_SHAPES = [  # n, h, w, k, stride, pad, dilation: 64 input channels, 3x3 (K = 576, the kernel's filter size)
+    (2, 20, 20, 64, 1, 1, 1),     # 400 pixels per image
+    (3, 56, 56, 64, 1, 1, 1),     # tiles of whole rows, as configuration 3 cuts them
+    (1, 33, 17, 128, 1, 1, 1),    # two filter slabs, tiles that start and end inside rows
+    (2, 15, 22, 40, 1, 1, 1),     # 40 filters: partial channel groups (general epilogue)
+    (2, 19, 19, 64, 2, 1, 1),     # stride 2
+    (1, 24, 18, 64, 1, 2, 2),     # dilation 2
+    (2, 12, 30, 64, 1, 0, 1),     # no padding
+    (1, 9, 70, 64, 1, (1, 3), 1), # wide rows, asymmetric padding
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_filter_resident_variant(tracea_gpu, dtype):
+    """The kernel that keeps input patch and filter bank in LDS together (64 filters of 3x3x64),
+    forced, against the oracle: tile cuts, strides, dilation, padding, partial filter slabs."""
+    from tracea_amd import capi
+    names = capi.variants("conv2d")
+    vi = [i for i, nm in enumerate(names) if nm.endswith("_resident")]
+    assert vi, "no filter-resident variant in the build"
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rnd = round_f16 if dtype == "f16" else round_bf16
+    capi.force_variant("conv2d", vi[0])
+    try:
+        for shape in RESIDENT_SHAPES:
+            n, h, w, k, stride, pad, dil = shape
+            rng = np.random.default_rng(h * 31 + w + k)
+            x = rnd(rng.standard_normal((n, h, w, 64)))
+            wk = rnd(rng.standard_normal((k, 3, 3, 64)) * np.sqrt(2.0 / 576))
+            bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+            ref = torch.nn.functional.conv2d(
+                torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
+                bias=torch.from_numpy(bias).double(), stride=stride, padding=pad, dilation=dil)
+            ref = torch.relu(ref).permute(0, 2, 3, 1).numpy()
+            if isinstance(pad, int):  # the oracle takes symmetric geometry: torch is cross-checked with it
+                acc = oracle.conv2d_nhwc(x, np.ascontiguousarray(wk.transpose(1, 2, 3, 0)), stride, pad, dil)
+                want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+                assert np.abs(want - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+            y = tracea_gpu.conv2d(_dev(x, tdt), _dev(wk, tdt), bias=_dev(bias), stride=stride, padding=pad,
+                                  dilation=dil, epilogue="bias+relu")
+            assert capi.last_variant("conv2d") == names[vi[0]], "the resident kernel refused %s" % (shape,)
+            assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(576, dtype), "%s %s" % (dtype, shape))
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
+def test_filter_resident_variant_operator_chains(tracea_gpu):
+    """Every form of its straight-line epilogue ([affine] [ReLU] [residual] [ReLU]) and chains outside it,
+    against the oracle's chain on the oracle's accumulator."""
+    from tracea_amd import capi
+    names = capi.variants("conv2d")
+    vi = [i for i, nm in enumerate(names) if nm.endswith("_resident")][0]
+    n, h, w, k = 2, 18, 25, 64
+    rng = np.random.default_rng(77)
+    x = round_f16(rng.standard_normal((n, h, w, 64)))
+    w_rsck = round_f16(rng.standard_normal((3, 3, 64, k)) * np.sqrt(2.0 / 576))
+    acc = oracle.conv2d_nhwc(x, w_rsck, 1, 1, 1)
+    bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+    (gamma, beta, mean, var), (scale, shift) = _bn_params(rng, k)
+    res = round_f16(rng.standard_normal(acc.shape))
+    dx, dw = _dev(x, torch.float16), _dev(w_rsck, torch.float16).permute(3, 0, 1, 2).contiguous()
+    dres, dbias = _dev(res, torch.float16), _dev(bias)
+    O, E = capi, oracle
+    aff = {"bias": ((O.OP_BIAS_ADD, dbias), (E.EPI_BIAS_ADD, bias)),
+           "bias16": ((O.OP_BIAS_ADD, _dev(round_f16(bias), torch.float16)), (E.EPI_BIAS_ADD, round_f16(bias))),
+           "ss": ((O.OP_SCALE_SHIFT, _dev(scale), _dev(shift)), (E.EPI_SCALE_SHIFT, scale, shift)),
+           "bn": ((O.OP_BATCHNORM, _dev(gamma), _dev(beta), _dev(mean), _dev(var), 1e-5), (E.EPI_BATCHNORM, gamma, beta, mean, var, 1e-5))}
+    relu = ((O.OP_RELU,), (E.EPI_RELU,))
+    resid = ((O.OP_RESIDUAL_ADD, dres), (E.EPI_RESIDUAL_ADD, res))
+    gelu = ((O.OP_GELU,), (E.EPI_GELU,))
+    chains = [[]]
+    for a in (None, "bias", "ss", "bn"):                      # the 16 forms (each affine kind once over them)
+        for r1 in (False, True):
+            for rs in (False, True):
+                for r2 in (False, True):
+                    c = ([aff[a]] if a else []) + ([relu] if r1 else []) + ([resid] if rs else []) + ([relu] if r2 else [])
+                    if c and (a != "bn" or rs):                # keep the list short: BatchNorm with a residual only
+                        chains.append(c)
+    chains += [[aff["bias16"], relu], [relu, aff["bias"]], [resid, aff["ss"]], [aff["bias"], gelu], [resid, resid, relu],
+               [aff["ss"], aff["bias"], relu]]                # outside the fast form: general path
+    capi.force_variant("conv2d", vi)
+    try:
+        for chain in chains:
+            want = oracle.epilogue_apply(acc, [c[1] for c in chain])
+            y = tracea_gpu.conv2d_ex(dx, dw, [c[0] for c in chain], stride=1, padding=1)
+            assert capi.last_variant("conv2d") == names[vi]
+            assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "chain %s" % ([c[1][0] for c in chain],))
+        # fp32 output and a bf16 residual on f16 operands leave the fast form too
+        y = tracea_gpu.conv2d_ex(dx, dw, [aff["bias"][0], relu[0]], stride=1, padding=1, out_dtype=torch.float32)
+        want = oracle.epilogue_apply(acc, [aff["bias"][1], relu[1]])
+        assert y.dtype == torch.float32
+        assert_close_scaled(y.cpu().numpy(), want, tol_for_k(576), "fp32 output")
+        resb = round_bf16(res)
+        y = tracea_gpu.conv2d_ex(dx, dw, [(O.OP_RESIDUAL_ADD, _dev(resb, torch.bfloat16)), relu[0]], stride=1, padding=1)
+        want = oracle.epilogue_apply(acc, [(E.EPI_RESIDUAL_ADD, resb), relu[1]])
+        assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "bf16 residual on f16 operands")
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
 def test_asymmetric_stride_and_padding_bf16(tracea_gpu):
     torch_f = torch.nn.functional
     rng = np.random.default_rng(9)

@@ -69,7 +69,20 @@ struct ContractionArgs {
   // load iterations per thread, LDS bytes reserved for the patch, and the
   // reciprocals of the chunk count and of the padded width
   int r_sz, p_tiles, p_pw, p_cpp, p_iters, p_np_bytes;
+  // pipeline 5 only: output pixels per workgroup (pipeline 4 has them in its tile shape), load
+  // instructions per padded patch row, pixels per load instruction, reciprocal of p_seg
+  int p_tm, p_seg, p_ppi;
+  unsigned p_seg_m, p_seg_s;
   unsigned p_cpp_m, p_cpp_s, p_pw_m, p_pw_s;
+  // pipeline 5 only: the chain in the fast form of conv_resident_kernel.hpp, or sig < 0
+  struct FastEpilogue {
+    int sig;                  // bit 0 affine, 1 ReLU, 2 residual, 3 ReLU (in this order); < 0: not of this form
+    int aff_kind, aff_dtype;  // TraceaEpilogueOpKind of the affine part and the DataType of a bias
+    const void *p0, *p1, *p2, *p3;
+    float epsilon;
+    const void *res;          // residual tensor (operand type), row stride res_ld elements
+    long long res_ld;
+  } fe;
   EpilogueChain epi;
 };
 
@@ -94,6 +107,8 @@ struct ContractionVariant {
                  //    and fetched with transposing LDS reads);
                  // 3: ring of `stages` LDS buffers, direct-to-LDS loads stages-1 tiles ahead
                  // 4: convolution only: input patch resident in LDS, filter tiles through a ring of `stages`
+                 // 5: convolution only: input patch and filter bank both resident in LDS
+                 //    (conv_resident_kernel.hpp); bm = most pixels per workgroup, K = 16 * stages exactly
   size_t lds_bytes;
   // launch: returns hipError_t as int
   int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);

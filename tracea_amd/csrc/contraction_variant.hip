@@ -3,6 +3,7 @@
 // -DV_NAME=... -DV_BM=... -DV_BN=... -DV_BK=... -DV_WM=... -DV_WN=... -DV_STAGES=... -DV_DIRECT=<pipeline mode>
 #include "contraction_kernel.hpp"
 #include "conv_patch_kernel.hpp"
+#include "conv_resident_kernel.hpp"
 
 #define TRACEA_CAT2(a, b) a##b
 #define TRACEA_CAT(a, b) TRACEA_CAT2(a, b)
@@ -17,6 +18,9 @@ const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
 #if V_DIRECT == 4
       (size_t)V_STAGES * V_BN * V_BK * 2,  // filter ring only; the patch size depends on the problem
       &launch_conv_patch<V_BM, V_BN, V_WM, V_WN, V_STAGES>};
+#elif V_DIRECT == 5
+      (size_t)rs_filter_bytes(V_STAGES) + RS_TABLE_BYTES,  // the patch, sized by the problem, comes on top
+      &launch_conv_resident<V_STAGES, 4>};  // 64 input channels: 4 k-steps per tap
 #else
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
       &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT>};

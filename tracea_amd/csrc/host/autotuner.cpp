@@ -66,7 +66,7 @@ std::vector<PipelineConfig> propose_contraction(uint32_t m, uint32_t n, uint32_t
     if (i == pick) continue;
     const ContractionVariant &v = contraction_variant(i);
     if (v.lds_bytes > hw.shared_memory_per_block) continue;
-    if (v.pipeline == 4 && !conv) continue;  // patch-resident kernels compute convolutions only
+    if (v.pipeline >= 4 && !conv) continue;  // patch-resident kernels compute convolutions only
     out.push_back(config_for_contraction_variant(i));
   }
   return out;

@@ -344,10 +344,14 @@ TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s,
 // entry, when present, wins over this.
 namespace {
 // Number of K ranges for a launch of variant v (1: no split) and the extent of one range.
+// Pipelines 4 and 5 are convolution kernels of their own (input patch in LDS): they need the
+// convolution geometry (plan_conv_patch / plan_conv_filter_resident), never split K and run no GEMM.
+inline bool conv_only(const ContractionVariant &v) { return v.pipeline >= 4; }
+
 int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split, int min_tiles = 4) {
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
-  if (v.pipeline == 4 || tiles * 2 > 256 || nk < 2 * min_tiles) return 1;
+  if (conv_only(v) || tiles * 2 > 256 || nk < 2 * min_tiles) return 1;
   long long splits = 256 / tiles;
   if (splits > nk / min_tiles) splits = nk / min_tiles;  // at least min_tiles K tiles per range
   if (splits < 2) return 1;
@@ -372,7 +376,7 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
   double best_cost = 0.0;
   for (int i = 0; i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
-    if (v.pipeline == 4) continue;  // needs the convolution geometry: see plan_conv_patch
+    if (conv_only(v)) continue;  // needs the convolution geometry: see plan_conv_patch
     const double gm = (double)((m + v.bm - 1) / v.bm), gn = (double)((n + v.bn - 1) / v.bn);
     int k_split = 0;
     const int splits = g_split_k_enabled.load() ? choose_split(v, m, n, k, &k_split) : 1;
@@ -440,7 +444,7 @@ int twin(int vi, int pipeline) {
 // register-staged pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
 int resolve_variant(int vi, bool conv, bool staged, bool k_exact) {
   int pipe = contraction_variant(vi).pipeline;
-  if (pipe == 4) pipe = 2;  // a convolution-only kernel asked for a GEMM: same tile with streamed operands, if any
+  if (pipe >= 4) pipe = 2;  // a convolution-only kernel asked for a GEMM: same tile with streamed operands, if any
   if (pipe >= 2 && staged) pipe = 1;
   if (pipe == 1 && !conv && !k_exact) pipe = 0;
   if (pipe == contraction_variant(vi).pipeline) return vi;
@@ -757,14 +761,14 @@ TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &ta, const TraceaTensorV
   // the variant: forced if its tile fits, else the most pipelined one with this macro-tile
   int vi = -1;
   const int forced = forced_variant("gemm");
-  if (forced >= 0 && contraction_variant(forced).pipeline != 4 && contraction_variant(forced).bm == (int)layout.mt &&
+  if (forced >= 0 && !conv_only(contraction_variant(forced)) && contraction_variant(forced).bm == (int)layout.mt &&
       contraction_variant(forced).bn == (int)layout.nt)
     vi = forced;
   static const int rank_of_pipeline[5] = {0, 1, 3, 2, -1};
   const bool use_forced = vi >= 0;
   for (int i = 0; !use_forced && i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
-    if (v.pipeline == 4 || v.bm != (int)layout.mt || v.bn != (int)layout.nt) continue;
+    if (conv_only(v) || v.bm != (int)layout.mt || v.bn != (int)layout.nt) continue;
     if (vi < 0) { vi = i; continue; }
     const ContractionVariant &best = contraction_variant(vi);
     const int r = rank_of_pipeline[v.pipeline], rb = rank_of_pipeline[best.pipeline];
@@ -1175,6 +1179,122 @@ bool plan_conv_patch(const ConvGeometry &g, const ContractionVariant &v, bool w_
   return true;
 }
 
+// The same for the kernel that keeps patch and filter bank in LDS together (pipeline 5,
+// conv_resident_kernel.hpp): K-contiguous filters, C a multiple of 16, K = 16 * stages exactly;
+// a workgroup takes p_tm consecutive output pixels of one image and 64 filters.  p_tm: every
+// workgroup costs the same whatever its tile holds (the kernel runs all its pixel blocks), so
+// the fewest rounds over the CUs win, and within that the most workgroups (smaller patches,
+// more CUs busy): N32 56x56 -> 8 tiles of 392 pixels per image, 256 workgroups.
+bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  const TraceaConvParamsBlock &b = g.block;
+  const int C = b.c_in;
+  if (v.pipeline != 5 || w_ncontig || C % 16 != 0 || g.k_gemm != 16 * v.stages) return false;
+  const long long img_bytes = (long long)b.h_in * b.w_in * C * 2;
+  const long long w_bytes = (long long)g.n_gemm * g.k_gemm * 2;
+  if (img_bytes >= (1ll << 31) || w_bytes >= (1ll << 31)) return false;
+  const long long pw = (long long)b.w_in + 2ll * g.pad_w;
+  const long long ph = (long long)b.h_in + 2ll * g.pad_h;
+  if (pw * ph >= (1ll << 30)) return false;
+  const int hw = b.h_out * b.w_out;
+  const int grid_n = (g.n_gemm + v.bn - 1) / v.bn;
+  const long long cus = 256;
+  const long long t_min = (hw + v.bm - 1) / v.bm;
+  const long long rounds = ((long long)b.batch * t_min * grid_n + cus - 1) / cus;
+  long long tiles = rounds * cus / ((long long)b.batch * grid_n);
+  if (tiles < t_min) tiles = t_min;
+  if (tiles > (hw + 15) / 16) tiles = (hw + 15) / 16;
+  const int tm = (int)((hw + tiles - 1) / tiles);
+  tiles = (hw + tm - 1) / tm;
+  const int cpp = (C / 8) | 1;
+  const int nt = 256;
+  // the patch holds whole padded rows: p_seg load instructions of ppi pixels each per row; the largest
+  // tile whose rows fit the kernel's fixed number of load instructions and the LDS left beside the
+  // filters (shrinking the tile makes more workgroups)
+  const int ppi = 64 / cpp;
+  if (ppi < 1) return false;
+  const int seg = (int)((pw + ppi - 1) / ppi);
+  int tm_fit = tm;
+  long long rows = 0, iters = 0, patch_bytes = 0;
+  for (;;) {
+    // most output rows one of the image's tiles spans (tiles start at multiples of tm_fit), then padded input rows
+    long long out_rows = 1;
+    for (int p0 = 0; p0 < hw; p0 += tm_fit) {
+      const int last = (p0 + tm_fit < hw ? p0 + tm_fit : hw) - 1;
+      const long long span = last / b.w_out - p0 / b.w_out + 1;
+      if (span > out_rows) out_rows = span;
+    }
+    rows = (out_rows - 1) * g.stride_h + (long long)(b.r_sz - 1) * g.dil_h + 1;
+    iters = (rows * seg + 7) / 8;
+    patch_bytes = (rows * pw * cpp + 1) * 16;  // (+1: the repeated first part behind the last pixel)
+    patch_bytes = (patch_bytes + 1023) / 1024 * 1024;
+    if (patch_bytes + (long long)v.lds_bytes <= 160 * 1024) break;
+    if (tm_fit <= 32) return false;
+    int next = tm_fit * 7 / 8 / 32 * 32;  // strictly smaller: rounded down to whole pixel blocks
+    if (next >= tm_fit) next = tm_fit - 32;
+    tm_fit = next < 32 ? 32 : next;
+  }
+  if ((long long)b.h_in * b.w_in >= (1ll << 24)) return false;
+  a->r_sz = b.r_sz;
+  a->p_tm = tm_fit;
+  a->p_tiles = (hw + tm_fit - 1) / tm_fit;
+  a->p_pw = (int)pw;
+  a->p_cpp = cpp;
+  a->p_iters = (int)iters;
+  a->p_np_bytes = (int)patch_bytes;
+  a->p_seg = seg;
+  a->p_ppi = ppi;
+  magic_for_divisor((uint32_t)cpp, 64, &a->p_cpp_m, &a->p_cpp_s);
+  magic_for_divisor((uint32_t)seg, (uint64_t)(rows * seg + 8), &a->p_seg_m, &a->p_seg_s);
+  a->p_pw_m = a->p_pw_s = 0;
+  a->grid_m = b.batch * a->p_tiles;
+  a->grid_n = grid_n;
+  a->group_m = 1;
+  a->b_bytes = (unsigned)w_bytes;
+  a->a_bytes = 0;
+  return true;
+}
+
+// The operator chain in the fast form of the filter-resident kernel: [affine] [ReLU] [residual] [ReLU],
+// each part at most once and in this order, affine = bias / scale-shift / BatchNorm; every tile has all 64
+// channels, output rows and residual rows are 8-byte aligned and addressable with 32-bit byte offsets
+// inside a tile, output and residual have the operand type.  Anything else: sig = -1 (general path).
+void fast_epilogue_form(const EpilogueChain &chain, int dtype, ContractionArgs *a) {
+  ContractionArgs::FastEpilogue fe{};
+  fe.sig = -1;
+  a->fe = fe;
+  bool ok = a->N % 64 == 0 && (a->ldc & 3) == 0 && aligned(a->C, 8) && a->out_dtype == dtype &&
+            (long long)a->p_tm * a->ldc * 2 < (1ll << 31);
+  int sig = 0, stage = 0;
+  for (int o = 0; o < chain.n_ops && ok; ++o) {
+    const EpilogueOpDev &op = chain.ops[o];
+    const bool aff = op.kind == TRACEA_EPI_OP_BIAS_ADD || op.kind == TRACEA_EPI_OP_SCALE_SHIFT || op.kind == TRACEA_EPI_OP_BATCHNORM;
+    int part;
+    if (op.kind == TRACEA_EPI_OP_NONE) continue;
+    else if (aff) part = 0;
+    else if (op.kind == TRACEA_EPI_OP_RELU) part = stage <= 2 ? 1 : 3;
+    else if (op.kind == TRACEA_EPI_OP_RESIDUAL_ADD) part = 2;
+    else { ok = false; break; }
+    if (part < stage) { ok = false; break; }
+    sig |= 1 << part;
+    stage = part + 1;
+    if (aff) {
+      fe.aff_kind = op.kind; fe.aff_dtype = op.dtype;
+      fe.p0 = op.p0; fe.p1 = op.p1; fe.p2 = op.p2; fe.p3 = op.p3; fe.epsilon = op.epsilon;
+    }
+    if (part == 2) {
+      fe.res = op.p0; fe.res_ld = op.ld;
+      ok = op.dtype == dtype && (op.ld & 3) == 0 && aligned(op.p0, 8) && (long long)a->p_tm * op.ld * 2 < (1ll << 31);
+    }
+  }
+  if (!ok) return;
+  fe.sig = sig;
+  a->fe = fe;
+}
+
+bool plan_conv_resident(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  return v.pipeline == 5 ? plan_conv_filter_resident(g, v, w_ncontig, a) : plan_conv_patch(g, v, w_ncontig, a);
+}
+
 TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStream_t stream) {
   const ConvGeometry &g = plan.geo;
   DeviceScope scope(plan.out.device);
@@ -1197,6 +1317,23 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
            g.pad_h, tuning_device_name());
   int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
   if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
+  // Default choice of the filter-resident variant (patch and 64 filters of K = 576 in LDS together, no
+  // barrier in its main loop): wherever it can run and the launch fills most of the device with tiles of
+  // at least 10 pixel blocks.  Measured in a replayed HIP graph against the best other variant: N32
+  // 56x56x64->64 14.1 us / 16.7; N64 25.2 / 28.6; N32 64->128 24.5 / 28.8; N8 10.3 / 9.5 (not taken).
+  bool resident_chosen = false;
+  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0) {
+    for (int i = 0; i < contraction_variant_count() && !resident_chosen; ++i) {
+      const ContractionVariant &cv = contraction_variant(i);
+      if (cv.pipeline != 5) continue;
+      ContractionArgs probe = a;
+      if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= 192 &&
+          probe.p_tm >= 320) {
+        vi = i;
+        resident_chosen = true;
+      }
+    }
+  }
   // Default choice of a patch-resident variant: stride-1 convolutions with a real filter
   // window whose K fits 40 filter tiles (the kernel has no split along K).  Fitted on the
   // ResNet-18/50 layer shapes at batch 1, 8 and 32, every variant timed inside a replayed
@@ -1208,7 +1345,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // short K (one 56x56x64->64 image: 7.4 us against 8.4).  Everywhere else the streamed
   // 8-wave 128x64 and pipelined 64x64 tiles are as fast or faster.  A tuning-cache entry or
   // a forced variant wins over this rule, and tracea_autotune_conv2d measures every variant.
-  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && g.stride_h == 1 &&
+  if (!resident_chosen && forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && g.stride_h == 1 &&
       g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 && a.K % 64 == 0 && a.K / 64 <= 40) {
     const long long hw = (long long)g.block.h_out * g.block.w_out;
     int chosen = -1;
@@ -1233,7 +1370,8 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   const long long x_extent = (long long)g.block.batch * g.block.h_in * g.block.w_in * g.block.c_in * 2;
   const long long w_extent = (long long)g.n_gemm * g.k_gemm * 2;
   const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
-  if (contraction_variant(vi).pipeline == 4 && plan_conv_patch(g, contraction_variant(vi), plan.w_ncontig, &a)) {
+  if (conv_only(contraction_variant(vi)) && plan_conv_resident(g, contraction_variant(vi), plan.w_ncontig, &a)) {
+    if (contraction_variant(vi).pipeline == 5) fast_epilogue_form(chain, plan.x.dtype, &a);
     t_last_conv = vi;
     return hip_status("conv2d launch",
                       contraction_variant(vi).launch(a, true, plan.x.dtype, false, stream));
@@ -1241,7 +1379,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // a patch-resident variant that cannot run this problem (asked for by a forced
   // index or a cache entry) gives way to the selector's choice, not to whatever
   // shares its tile shape
-  if (contraction_variant(vi).pipeline == 4) {
+  if (conv_only(contraction_variant(vi))) {
     vi = select_contraction_variant(a.M, a.N, a.K, true);
     if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
   }
