@@ -70,9 +70,8 @@ struct ContractionArgs {
   // reciprocals of the chunk count and of the padded width
   int r_sz, p_tiles, p_pw, p_cpp, p_iters, p_np_bytes;
   // pipeline 5 only: output pixels per workgroup (pipeline 4 has them in its tile shape), load
-  // instructions per padded patch row, pixels per load instruction, reciprocal of p_seg
+  // instructions per padded patch row, pixels per load instruction
   int p_tm, p_seg, p_ppi;
-  unsigned p_seg_m, p_seg_s;
   unsigned p_cpp_m, p_cpp_s, p_pw_m, p_pw_s;
   // pipeline 5 only: the chain in the fast form of conv_resident_kernel.hpp, or sig < 0
   struct FastEpilogue {

@@ -95,38 +95,43 @@ __global__ void __launch_bounds__(512) conv_resident_kernel(const ContractionArg
                                              0);
   }
 
-  // ---- patch, row by row ----
+  // ---- patch, by columns of load instructions ----
   // One load instruction moves the PPI = 64 / cpp pixels wp0 .. wp0 + PPI - 1 of one padded row (lane l:
   // pixel l / cpp, 16-byte part l % cpp; the part past the channels is padding and is written as zeros;
-  // a last lane, if any, repeats the first part of the next pixel), so what depends on the lane is a
-  // constant and what depends on the instruction is uniform.  Padding pixels and rows get an
-  // out-of-range offset and are written as zeros; lanes past the row's end are switched off (they would
-  // land on the next row's pixels).  Instruction n = row * p_seg + segment goes to wave n % 8.
+  // a last lane, if any, repeats the first part of the next pixel).  A wave takes segment j = wave,
+  // wave + 8, ... of EVERY row: what depends on the lane (its pixel's column, whether that is padding)
+  // is then fixed per segment and worked out once, and a load costs fourteen instructions with its loop --
+  // row test, two selects, address updates -- where a mapping by instruction number, with the lane tests
+  // redone for every load, cost thirty-six: with 160 loads per tile that was a seventh of the kernel's time.
+  // Padding pixels and rows get an out-of-range offset and are written as zeros; lanes past the row's
+  // end are switched off (they would land on the next row's pixels).
   int ho_f, wo_f, ho_l, wo_l;
   fast_divmod(p0, args.w_m, args.w_s, args.w_out, ho_f, wo_f);
   fast_divmod(p0 + npix - 1, args.w_m, args.w_s, args.w_out, ho_l, wo_l);
   const int hp0 = ho_f * args.stride_h;
   const int tap_h = args.dil_h * PW;  // pixel index step of one filter row
   const int n_rows = ho_l * args.stride_h + (args.r_sz - 1) * args.dil_h - hp0 + 1;
-  const int SEG = args.p_seg, n_inst = n_rows * SEG;
-  const int PPI = args.p_ppi;
+  const int SEG = args.p_seg, PPI = args.p_ppi;
   const int cdata = C >> 3;  // 16-byte parts of a pixel that hold channels
   int ldl, lpart;
   fast_divmod(lane, args.p_cpp_m, args.p_cpp_s, cpp, ldl, lpart);
   const int lane_off = (ldl - args.pad_w) * C * 2 + lpart * 16;  // byte offset from the row's first real pixel
-  for (int n = wave_u; n < n_inst; n += 8) {
-    int r, j;
-    fast_divmod(n, args.p_seg_m, args.p_seg_s, SEG, r, j);
-    const int hi = hp0 + r - args.pad_h;
-    const bool row_ok = (unsigned)hi < (unsigned)args.h_in;
+  const int row_bytes = args.w_in * C * 2, row_pitch = PW * pitch;
+  for (int j = wave_u; j < SEG; j += 8) {
     const int wp = j * PPI + ldl;
-    const bool ok = row_ok & ((unsigned)(wp - args.pad_w) < (unsigned)args.w_in) & (lpart < cdata);
-    const unsigned voff = ok ? (unsigned)(lane_off + j * PPI * C * 2) : OOB;
-    const int soff = row_ok ? hi * args.w_in * C * 2 : 0;
-    unsigned char *dst = patch + (r * PW + j * PPI) * pitch;
-    if (wp < PW)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void *)dst, 16, (int)voff, soff,
-                                               0, 0);
+    const bool lane_ok = ((unsigned)(wp - args.pad_w) < (unsigned)args.w_in) & (lpart < cdata);
+    const unsigned v_seg = lane_ok ? (unsigned)(lane_off + j * PPI * C * 2) : OOB;
+    if (wp < PW) {
+      int hi = hp0 - args.pad_h;
+      unsigned char *dst = patch + j * PPI * pitch;
+      for (int r = 0; r < n_rows; ++r) {
+        const bool row_ok = (unsigned)hi < (unsigned)args.h_in;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void *)dst, 16,
+                                                 (int)(row_ok ? v_seg : OOB), row_ok ? hi * row_bytes : 0, 0, 0);
+        hi += 1;
+        dst += row_pitch;
+      }
+    }
   }
 
   // ---- epilogue form and this thread's entry of the operand table (requested now, read after the wait) ----

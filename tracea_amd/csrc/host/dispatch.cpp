@@ -1244,7 +1244,6 @@ bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &
   a->p_seg = seg;
   a->p_ppi = ppi;
   magic_for_divisor((uint32_t)cpp, 64, &a->p_cpp_m, &a->p_cpp_s);
-  magic_for_divisor((uint32_t)seg, (uint64_t)(rows * seg + 8), &a->p_seg_m, &a->p_seg_s);
   a->p_pw_m = a->p_pw_s = 0;
   a->grid_m = b.batch * a->p_tiles;
   a->grid_n = grid_n;
