@@ -339,36 +339,40 @@ fa2_fwd_kernel(const AttentionArgs a) {
 // takes the maximum of a tile past the end, all of whose scores are masked:
 // nothing moves.
 // ---------------------------------------------------------------------------
-template <int DT, int D, bool EARLY_MAX>
-__global__ void __launch_bounds__(FA_WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// WAVES: waves of 32 queries per workgroup (4 or 8: 128 or 256 queries share every K/V tile);
+// NSTG: LDS stages per K and per V ring (2: tiles requested one iteration ahead, 3: two).
+template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG>
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
 fa2_fwd_pipe_kernel(const AttentionArgs a) {
+  constexpr int BQ = 32 * WAVES;
   constexpr int ROW_BYTES = D * 2;
   constexpr int CH = D / 8;
   constexpr int TILE_BYTES = FA_BKV * ROW_BYTES;
   constexpr int KS = D / 16;
   constexpr int DB = D / 32;
   constexpr int RPI = 64 / CH;                 // tile rows per wave-wide load instruction
-  constexpr int NI = FA_BKV / (RPI * FA_WAVES); // load instructions per wave per tensor per tile
+  constexpr int NI = FA_BKV / (RPI * WAVES); // load instructions per wave per tensor per tile
   constexpr int RP = 256 / ROW_BYTES > 0 ? 256 / ROW_BYTES : 1;
   constexpr int WIN = ROW_BYTES / 64;
-  static_assert(D % 32 == 0 && FA_BKV % (RPI * FA_WAVES) == 0, "unsupported head dim");
+  static_assert(D % 32 == 0 && FA_BKV % (RPI * WAVES) == 0, "unsupported head dim");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  unsigned char *const sKbase = smem;                   // 2 stages
-  unsigned char *const sVbase = smem + 2 * TILE_BYTES;  // 2 stages
+  static_assert(NSTG == 2 || NSTG == 3, "ring depth");
+  unsigned char *const sKbase = smem;                      // NSTG stages
+  unsigned char *const sVbase = smem + NSTG * TILE_BYTES;  // NSTG stages
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int lrow = lane & 31, g = lane >> 5;
 
-  const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
+  const int nqb = (a.S + BQ - 1) / BQ;
   const int total = nqb * a.B * a.H;
   int vid = blockIdx.x;
   if ((total & 7) == 0) vid = (vid & 7) * (total >> 3) + (vid >> 3);
   const int bh = vid / nqb;
   const int qb = nqb - 1 - (vid - bh * nqb);
   const int b = bh / a.H, h = bh - b * a.H;
-  const int q0 = qb * FA_BQ;
+  const int q0 = qb * BQ;
   const int S = a.S;
 
   const unsigned short *Qg = (const unsigned short *)a.Q + (long long)b * a.q_sb + (long long)h * a.q_sh;
@@ -398,13 +402,13 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       (void *)Kg, 0, (int)(((long long)(S - 1) * a.k_ss + D) * 2), 0x00020000);
   __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
       (void *)Vg, 0, (int)(((long long)(S - 1) * a.v_ss + D) * 2), 0x00020000);
-  // Load instruction i of this wave covers tile rows (i*FA_WAVES + wave)*RPI + lane/CH; the lane's
+  // Load instruction i of this wave covers tile rows (i*WAVES + wave)*RPI + lane/CH; the lane's
   // LDS slot is 16-byte column lane%CH of that row, so it fetches the global column that the
   // swizzle of the tensor maps there.
   unsigned k_voff[NI], v_voff[NI];
 #pragma unroll
   for (int i = 0; i < NI; ++i) {
-    const int row = (i * FA_WAVES + wave) * RPI + lane / CH;
+    const int row = (i * WAVES + wave) * RPI + lane / CH;
     const int p = lane % CH;
     k_voff[i] = (unsigned)(row * (int)a.k_ss * 2 + ((p ^ ((row / RP) & (CH - 1))) << 4));
     v_voff[i] = (unsigned)(row * (int)a.v_ss * 2 + ((p ^ (((row / RP) % WIN) << 2)) << 4));
@@ -414,7 +418,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc_k, (__attribute__((address_space(3))) void *)(dst + (i * FA_WAVES + wave_u) * RPI * ROW_BYTES),
+          rsrc_k, (__attribute__((address_space(3))) void *)(dst + (i * WAVES + wave_u) * RPI * ROW_BYTES),
           16, (int)(k_voff[i] + adv), 0, 0, 0);
   };
   auto load_v = [&](int t, unsigned char *dst) {
@@ -422,13 +426,13 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
     for (int i = 0; i < NI; ++i)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(
-          rsrc_v, (__attribute__((address_space(3))) void *)(dst + (i * FA_WAVES + wave_u) * RPI * ROW_BYTES),
+          rsrc_v, (__attribute__((address_space(3))) void *)(dst + (i * WAVES + wave_u) * RPI * ROW_BYTES),
           16, (int)(v_voff[i] + adv), 0, 0, 0);
   };
 
   int ntiles = (S + FA_BKV - 1) / FA_BKV;
   if (a.causal) {
-    const int last_q = (q0 + FA_BQ - 1 < S ? q0 + FA_BQ - 1 : S - 1);
+    const int last_q = (q0 + BQ - 1 < S ? q0 + BQ - 1 : S - 1);
     const int need = last_q / FA_BKV + 1;
     ntiles = need < ntiles ? need : ntiles;
   }
@@ -455,10 +459,18 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   float m_run = -1.0e30f, l_run = 0.0f;
 
   // tiles at or beyond the end of the sequence lie outside the buffers and load as zeros
+  // requests of a wave that may stay in flight where an iteration waits for its tiles: those of the
+  // iteration before (NSTG = 3), none (NSTG = 2)
+  constexpr int FLIGHT = (NSTG - 2) * 2 * NI;
+  constexpr int WAIT_TILES = (FLIGHT & 15) | (7 << 4) | (15 << 8) | ((FLIGHT >> 4) << 14);
   load_k(0, sKbase);
   load_v(0, sVbase);
   load_k(1, sKbase + TILE_BYTES);
-  __builtin_amdgcn_s_waitcnt(0x0f70);
+  if constexpr (NSTG == 3) {
+    load_v(1, sVbase + TILE_BYTES);
+    load_k(2, sKbase + 2 * TILE_BYTES);
+  }
+  __builtin_amdgcn_s_waitcnt(WAIT_TILES);
   __syncthreads();
   f32x16 s_cur[2], s_nxt[2];
   scores(sKbase, s_cur);
@@ -506,7 +518,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // the vector ALU.
   u32x4 pf[4];
   auto softmax_and_next_scores = [&](int t) {
-    const unsigned char *sKn = sKbase + ((t + 1) & 1) * TILE_BYTES;
+    const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -557,7 +569,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // interleaved instruction by instruction.  For EARLY_MAX the tag describes
   // tile t+1, the one whose maximum the iteration takes.
   auto iteration = [&](int t, auto edge_tag) {
-    const unsigned char *sV = sVbase + (t & 1) * TILE_BYTES;
+    const unsigned char *sV = sVbase + (t % NSTG) * TILE_BYTES;
     if constexpr (!EARLY_MAX) {
       const bool moved = take_max(t, edge_tag, s_cur);
       rescale(moved);
@@ -574,7 +586,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       // matrix pipe works on its MFMAs, whatever order the compiler gives them
       // inside the chunk.
       constexpr bool EDGE = decltype(edge_tag)::value;
-      const unsigned char *sKn = sKbase + ((t + 1) & 1) * TILE_BYTES;
+      const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
       // ---- phase A: S^T(t+1) = K(t+1) Q^T  with  P(t) = exp2(S(t)*scale - m), row sums ----
       // chunk ks: the two MFMAs of k-step ks (operands read one chunk ahead) and
       // 32/KS of the 32 exponentials
@@ -674,18 +686,20 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // body is the interior one while that tile is interior
   const int interior_end = EARLY_MAX ? first_edge - 1 : first_edge;
   int t = 0;
+  // The barrier at the head of iteration t publishes K(t+1) and V(t) and retires K(t) and V(t-1),
+  // whose stages then receive K(t+NSTG) and V(t+NSTG-1).
   for (; t < interior_end; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1) and V(t), requested one iteration ago
+    __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(t+1) and V(t), requested NSTG-1 iterations ago
     __syncthreads();
-    load_k(t + 2, sKbase + (t & 1) * TILE_BYTES);
-    load_v(t + 1, sVbase + ((t + 1) & 1) * TILE_BYTES);
+    load_k(t + NSTG, sKbase + (t % NSTG) * TILE_BYTES);
+    load_v(t + NSTG - 1, sVbase + ((t + NSTG - 1) % NSTG) * TILE_BYTES);
     iteration(t, std::false_type{});
   }
   for (; t < ntiles; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __builtin_amdgcn_s_waitcnt(WAIT_TILES);
     __syncthreads();
-    load_k(t + 2, sKbase + (t & 1) * TILE_BYTES);
-    load_v(t + 1, sVbase + ((t + 1) & 1) * TILE_BYTES);
+    load_k(t + NSTG, sKbase + (t % NSTG) * TILE_BYTES);
+    load_v(t + NSTG - 1, sVbase + ((t + NSTG - 1) % NSTG) * TILE_BYTES);
     iteration(t, std::true_type{});
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // look-ahead loads must not land on the output staging
@@ -722,14 +736,15 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   }
 }
 
-template <int D, bool EARLY_MAX>
+template <int D, bool EARLY_MAX, int WAVES, int NSTG>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
-  constexpr size_t lds = 4 * (size_t)FA_BKV * D * 2;
-  const int nqb = (a.S + FA_BQ - 1) / FA_BQ;
-  const dim3 grid((unsigned)(nqb * a.B * a.H)), block(FA_WAVES * 64);
+  constexpr size_t ring = 2 * (size_t)NSTG * FA_BKV * D * 2, staging = (size_t)WAVES * 32 * D * 2;
+  constexpr size_t lds = ring > staging ? ring : staging;
+  const int nqb = (a.S + 32 * WAVES - 1) / (32 * WAVES);
+  const dim3 grid((unsigned)(nqb * a.B * a.H)), block(WAVES * 64);
 #define TRACEA_FA_LAUNCH(DTV)                                                                  \
   do {                                                                                         \
-    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX>;                                                    \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG>;                            \
     static bool attr_done = false;                                                             \
     if (!attr_done) {                                                                          \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
@@ -747,8 +762,8 @@ static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream
 
 // The buffer loads address a (batch, head) slice with 32-bit byte offsets.
 static bool slice_fits(const AttentionArgs &a) {
-  const long long k_ext = ((long long)(a.S - 1 + 3 * FA_BKV) * a.k_ss + a.D) * 2;
-  const long long v_ext = ((long long)(a.S - 1 + 3 * FA_BKV) * a.v_ss + a.D) * 2;
+  const long long k_ext = ((long long)(a.S - 1 + 4 * FA_BKV) * a.k_ss + a.D) * 2;  // (tiles up to 3 past the end are requested)
+  const long long v_ext = ((long long)(a.S - 1 + 4 * FA_BKV) * a.v_ss + a.D) * 2;
   return k_ext < (1ll << 31) && v_ext < (1ll << 31);
 }
 // (the running maximum is taken over raw scores, which needs a positive scale)
@@ -781,16 +796,25 @@ static int launch_fa2(const AttentionArgs &a, int dtype, hipStream_t stream) {
 static bool feasible_d128(const AttentionArgs &a) { return a.D == 128; }
 static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 
+// The kernel family: queries per workgroup (32 per wave, 4 or 8 waves), K/V ring depth (2 or 3 stages per
+// tensor), head dimension, and the three kernel forms (pipe2 / pipe: direct-to-LDS tiles, maximum taken
+// under the P.V MFMAs or in a phase of its own; tr / u16: the register-staged cross-check).  The tuner
+// measures every feasible member (tracea_tune_fa2); the first feasible entry is the default.  (Head
+// dimension 128 has no 3-stage member: the third set of per-lane tile addresses does not fit the 256
+// registers of two waves per SIMD and the kernel spills.)
 static const AttentionVariant kAttentionVariants[] = {
-    // the first feasible entry is the default
-    {"fa2_q128_kv64_d128_pipe2", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<128, true>, &feasible_pipe_d128},
-    {"fa2_q128_kv64_d64_pipe2", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<64, true>, &feasible_pipe_d64},
-    {"fa2_q128_kv64_d128_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<128, false>, &feasible_pipe_d128},
-    {"fa2_q128_kv64_d64_pipe", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2_pipe<64, false>, &feasible_pipe_d64},
-    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, true>, &feasible_d128},
-    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<128, false>, &feasible_d128},
-    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<64, true>, &feasible_d64},
-    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, &launch_fa2<64, false>, &feasible_d64},
+    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128},
+    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64},
+    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128},
+    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64},
+    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64},
+    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3>, &feasible_pipe_d64},
+    {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128},
+    {"fa2_q128_kv64_d64_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, false, 4, 2>, &feasible_pipe_d64},
+    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, true>, &feasible_d128},
+    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, false>, &feasible_d128},
+    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, true>, &feasible_d64},
+    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, false>, &feasible_d64},
 };
 
 int attention_variant_count() { return (int)(sizeof(kAttentionVariants) / sizeof(kAttentionVariants[0])); }

@@ -210,6 +210,7 @@ int launch_softmax_rows(const void *x, void *out, int dtype, int out_dtype, long
 struct AttentionVariant {
   const char *name;
   int block_q, block_kv, waves;
+  int stages;  // LDS stages per K and per V ring
   int (*launch)(const AttentionArgs &, int dtype, hipStream_t);
   bool (*feasible)(const AttentionArgs &);
 };

@@ -153,7 +153,7 @@ int contraction_variant_for_config(const PipelineConfig &c) {
 
 PipelineConfig config_for_attention_variant(int index) {
   const AttentionVariant &v = attention_variant(index);
-  PipelineConfig c(2, (uint32_t)v.block_q, (uint32_t)v.block_kv, 32);
+  PipelineConfig c((uint32_t)v.stages, (uint32_t)v.block_q, (uint32_t)v.block_kv, 32);
   c.instruction = "RocmMFMA";
   c.swizzle_mode = "Xor8";
   c.has_force_num_warps = true;
