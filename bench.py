@@ -20,10 +20,15 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak
 PEAKS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}  # dense MFMA peak of the type a workload computes in
-# HBM-side bytes per launch of the dominant kernel of each workload, from the rocprofv3
-# FETCH_SIZE / WRITE_SIZE counters scaled by a copy kernel of known size
-# (profiles/bench_kernels_mi355x.md); None where no counter run exists.
-TRAFFIC_BYTES = {"gemm": 235.2e6, "conv": 26.5e6, "attention": 537.1e6, "attention_causal": None, "gemm_rowmajor": None, "conv_transpose": None, "copy": None}
+FLOP_PER_CLK_PER_CU = {"f16": 4096.0, "bf16": 4096.0, "f32": 256.0}  # dense MFMA rate of one compute unit
+# What the roofline blocks take from the rocprofv3 counter runs: HBM-side bytes per launch of a
+# workload's dominant kernel (FETCH_SIZE / WRITE_SIZE scaled by a copy of known size) and the shader
+# clock that kernel ran at (SQ_BUSY_CYCLES over its duration).  The table is written by
+# `python -m tracea_amd.profile_summary` from the counter files of the commands that
+# profiles/bench_kernels_mi355x.md lists, and names the kernel each row was measured on.
+ROOFLINE_INPUTS = os.path.join(ROOT, "profiles", "roofline_inputs.json")
+KERNEL_OF = {"gemm": "gemm", "gemm_nonsquare": "gemm", "gemm_rowmajor": "gemm", "conv": "conv2d",
+             "attention": "attention", "attention_causal": "attention"}  # operator whose variant a workload runs
 METRIC = "TFLOPS + % fp16 MFMA peak: GEMM 4096^3, 3x3 implicit-GEMM conv, FA2 fwd"
 
 
@@ -176,6 +181,34 @@ def make_workload(name, torch, ops):
     raise SystemExit("unknown workload " + name)
 
 
+def roofline_inputs():
+    try:
+        with open(ROOFLINE_INPUTS) as f:
+            return json.load(f).get("workloads", {})
+    except (OSError, ValueError):
+        return {}
+
+
+def roofline_block(name, flops, dev_s, dtype, cus, variant, inputs):
+    """achieved = algorithmic flops / HIP-event time per launch; peak = the published one; traffic and the
+    peak at the clock the kernel was measured at come from the counter table, with `stale` set when
+    the kernel that just ran is not the one the table's row was measured on."""
+    peak = PEAKS.get(dtype, PEAK_TFLOPS)
+    row = inputs.get(name) or {}
+    achieved = flops / dev_s / 1e12
+    block = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+             "frac": round(achieved / peak, 4), "traffic": row.get("traffic_bytes")}
+    if row.get("clock_ghz"):
+        at_clock = cus * FLOP_PER_CLK_PER_CU.get(dtype, 4096.0) * row["clock_ghz"] * 1e9 / 1e12
+        block["peak_at_measured_clock"] = round(at_clock, 1)
+        block["clock_ghz"] = row["clock_ghz"]
+        block["frac_of_peak_at_measured_clock"] = round(achieved / at_clock, 4)
+    if row:
+        block["counters_from"] = row.get("variant")
+        block["stale"] = bool(variant) and row.get("variant") not in (None, variant)
+    return block
+
+
 def time_steps(torch, step, steps, warmup):
     """Wall clock around exactly `steps` launches, plus HIP-event time on the launch stream."""
     for _ in range(warmup):
@@ -295,6 +328,8 @@ def main():
     # first 50 launches, 116 us from the 150th on); with the side workloads first the headline's
     # warm-up and timed steps run on a device that is already in its steady state.
     cpu = also = None
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    inputs = roofline_inputs()
     if not args.no_extras:
         cpu = cpu_baseline()
         also = {}
@@ -307,29 +342,34 @@ def main():
             also[name] = {"workload": lab, "tflops": round(fl / d / 1e12, 2),
                           "pct_of_peak": round(100.0 * fl / d / 1e12 / PEAKS.get(dt, PEAK_TFLOPS), 2),
                           "us_per_launch": round(d * 1e6, 2), "dtype": dt}
+            dk = d
             if name in ("conv", "gemm_f32", "basic_block", "downsample_block"):  # launches shorter than the host's per-call cost: also as a replayed graph
                 dg = time_steps_graph(torch, st, 40)
                 also[name]["us_per_launch_graph"] = round(dg * 1e6, 2)
                 also[name]["tflops_graph"] = round(fl / dg / 1e12, 2)
+                dk = min(d, dg)
+            if name in ("conv", "attention", "attention_causal", "gemm"):  # the workloads the metric names
+                # the kernel's duration: events over back-to-back launches, from Python or (where a Python
+                # call takes longer than the kernel) over the replayed graph
+                also[name]["roofline"] = roofline_block(name, fl, dk, dt, cus, capi.last_variant(KERNEL_OF[name]), inputs)
+                also[name]["roofline"]["timed"] = "graph replay" if dk < d else "stream launches"
             del st
             torch.cuda.empty_cache()
 
     label, flops, bytes_, dtype, step = make_workload(args.workload, torch, ops)
     wall, dev_s = time_steps(torch, step, args.steps, args.warmup)
     tflops = flops / wall / 1e12
-    achieved = flops / dev_s / 1e12
     stats = launch_stats(torch, step)
     line = {
         "metric": METRIC, "value": round(tflops, 2), "unit": "TFLOPS", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall * 1e3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
-        "data": "synthetic", "config": {"workload": label},
+        "data": "synthetic", "config": {"workload": label, "variant": capi.last_variant(KERNEL_OF[args.workload]) if args.workload in KERNEL_OF else None},
         "pct_of_peak": round(100.0 * tflops / PEAKS.get(dtype, PEAK_TFLOPS), 2),
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAKS.get(dtype, PEAK_TFLOPS),
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAKS.get(dtype, PEAK_TFLOPS), 4),
-                     "traffic": TRAFFIC_BYTES.get(args.workload),
-                     "hbm_GBps_algorithmic": round(bytes_ / dev_s / 1e9, 1)},
+        "roofline": roofline_block(args.workload, flops, dev_s, dtype, cus,
+                                   capi.last_variant(KERNEL_OF[args.workload]) if args.workload in KERNEL_OF else None, inputs),
     }
+    line["roofline"]["hbm_GBps_algorithmic"] = round(bytes_ / dev_s / 1e9, 1)
     line["launch_us"] = stats
     if not args.no_extras:
         line["also"] = also
