@@ -127,9 +127,10 @@ PipelineConfig config_for_contraction_variant(int index) {
   c.force_num_warps = (uint32_t)(v.waves_m * v.waves_n);
   c.micro_m = (uint32_t)(v.bm / v.waves_m);
   c.micro_n = (uint32_t)(v.bn / v.waves_n);
-  // the two MFMA block shapes of the kernel family under the reference's names for them
-  // (src/core/config.rs:166-181): 32x32x16 -> M32N32K2, 16x16x32 -> M16N16K4
-  c.intrinsic_shape = v.pipeline == 5 ? "M16N16K4" : "M32N32K2";
+  // every half-precision kernel of the family multiplies with v_mfma_f32_32x32x16 (the 16x16x32 shape
+  // sustained two thirds of its rate in these loops), under the reference's name for a 32x32 MFMA block
+  // (src/core/config.rs:166-181)
+  c.intrinsic_shape = "M32N32K2";
   c.gemm_variant = "Simd";
   c.double_buffer = true;
   c.cp_async_distance = (uint32_t)v.pipeline;  // operand prefetch distance in k-steps
@@ -145,7 +146,7 @@ int contraction_variant_for_config(const PipelineConfig &c) {
     if (c.has_force_num_warps && (uint32_t)(v.waves_m * v.waves_n) != c.force_num_warps) continue;
     if (c.micro_m > 1 && (uint32_t)(v.bm / v.waves_m) != c.micro_m) continue;
     if (c.cp_async_distance != (uint32_t)v.pipeline) continue;
-    if (c.intrinsic_shape == "M16N16K4" && v.pipeline != 5) continue;
+    if (c.intrinsic_shape == "M16N16K4") continue;  // no member with 16x16 MFMA blocks
     return i;
   }
   return -1;
