@@ -47,6 +47,20 @@ struct Interleave3 {
   }
 };
 
+// kMfmas steps of: one MFMA, kValu vector-ALU instructions, and an LDS read in the first kReads steps.
+// A wave that has its SIMD to itself must be given this order explicitly: MFMAs issued back to back
+// hold the wave's issue slot while each waits for the matrix pipe, and the vector work of the chunk
+// then runs behind the last of them instead of under all of them.
+template <int kStep, int kMfmas, int kValu, int kReads>
+struct MfmaValu {
+  static __device__ __forceinline__ void run() {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (kValu > 0) __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+    if constexpr (kStep < kReads) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    if constexpr (kStep + 1 < kMfmas) MfmaValu<kStep + 1, kMfmas, kValu, kReads>::run();
+  }
+};
+
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
 template <int DT>
@@ -341,10 +355,12 @@ fa2_fwd_kernel(const AttentionArgs a) {
 // ---------------------------------------------------------------------------
 // WAVES: waves of 32 queries per workgroup (4 or 8: 128 or 256 queries share every K/V tile);
 // NSTG: LDS stages per K and per V ring (2: tiles requested one iteration ahead, 3: two).
-template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG>
-__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB>
+__global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 fa2_fwd_pipe_kernel(const AttentionArgs a) {
-  constexpr int BQ = 32 * WAVES;
+  static_assert(QB == 1 || (QB == 2 && EARLY_MAX), "two query blocks per wave exist in the two-phase form only");
+  constexpr int WQ = 32 * QB;  // queries per wave
+  constexpr int BQ = WQ * WAVES;
   constexpr int ROW_BYTES = D * 2;
   constexpr int CH = D / 8;
   constexpr int TILE_BYTES = FA_BKV * ROW_BYTES;
@@ -380,20 +396,22 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   const unsigned short *Vg = (const unsigned short *)a.V + (long long)b * a.v_sb + (long long)h * a.v_sh;
   unsigned short *Og = (unsigned short *)a.O + (long long)b * a.o_sb + (long long)h * a.o_sh;
 
-  const int q_wave0 = q0 + wave * 32;
-  const int q_mine = q_wave0 + lrow;
-  u32x4 qf[KS];
-  {
-    const int qr = q_mine < S ? q_mine : S - 1;
+  const int q_wave0 = q0 + wave * WQ;
+  int q_mine[QB];  // this lane's query in each of the wave's blocks of 32
+  u32x4 qf[QB][KS];
+#pragma unroll
+  for (int qi = 0; qi < QB; ++qi) {
+    q_mine[qi] = q_wave0 + qi * 32 + lrow;
+    const int qr = q_mine[qi] < S ? q_mine[qi] : S - 1;
     const unsigned short *qp = Qg + (long long)qr * a.q_ss + g * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4 *)(qp + ks * 16);
+    for (int ks = 0; ks < KS; ++ks) qf[qi][ks] = *(const u32x4 *)(qp + ks * 16);
   }
 
-  auto k_piece = [&](int row, int c) -> int {
+  auto k_piece = [&](int row, int c) __attribute__((always_inline)) -> int {
     return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
   };
-  auto v_piece = [&](int row, int c) -> int {
+  auto v_piece = [&](int row, int c) __attribute__((always_inline)) -> int {
     return row * ROW_BYTES + ((c ^ (((row / RP) % WIN) << 2)) << 4);
   };
 
@@ -413,7 +431,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     k_voff[i] = (unsigned)(row * (int)a.k_ss * 2 + ((p ^ ((row / RP) & (CH - 1))) << 4));
     v_voff[i] = (unsigned)(row * (int)a.v_ss * 2 + ((p ^ (((row / RP) % WIN) << 2)) << 4));
   }
-  auto load_k = [&](int t, unsigned char *dst) {
+  auto load_k = [&](int t, unsigned char *dst) __attribute__((always_inline)) {
     const unsigned adv = (unsigned)t * (unsigned)(FA_BKV * 2) * (unsigned)a.k_ss;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -421,7 +439,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           rsrc_k, (__attribute__((address_space(3))) void *)(dst + (i * WAVES + wave_u) * RPI * ROW_BYTES),
           16, (int)(k_voff[i] + adv), 0, 0, 0);
   };
-  auto load_v = [&](int t, unsigned char *dst) {
+  auto load_v = [&](int t, unsigned char *dst) __attribute__((always_inline)) {
     const unsigned adv = (unsigned)t * (unsigned)(FA_BKV * 2) * (unsigned)a.v_ss;
 #pragma unroll
     for (int i = 0; i < NI; ++i)
@@ -437,26 +455,38 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     ntiles = need < ntiles ? need : ntiles;
   }
 
-  auto scores = [&](const unsigned char *sK, f32x16 (&s)[2]) {
+  // (a key fragment read from LDS serves all QB query blocks of the wave: with one block every MFMA
+  // needs 1 KB of LDS, which is all that LDS delivers while the four matrix pipes of the CU run)
+  auto scores = [&](const unsigned char *sK, f32x16 (&s)[QB][2]) {
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
+    for (int qi = 0; qi < QB; ++qi)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) s[blk][e] = 0.0f;
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[qi][blk][e] = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
         const u32x4 kf = *(const u32x4 *)(sK + k_piece(blk * 32 + lrow, ks * 2 + g));
-        s[blk] = Mfma32<DT>::run(kf, qf[ks], s[blk]);
+#pragma unroll
+        for (int qi = 0; qi < QB; ++qi) s[qi][blk] = Mfma32<DT>::run(kf, qf[qi][ks], s[qi][blk]);
       }
   };
 
-  f32x16 o[DB];
+  f32x16 o[QB][DB];
 #pragma unroll
-  for (int d = 0; d < DB; ++d)
+  for (int qi = 0; qi < QB; ++qi)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) o[d][e] = 0.0f;
-  float m_run = -1.0e30f, l_run = 0.0f;
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[qi][d][e] = 0.0f;
+  float m_run[QB], l_run[QB];
+#pragma unroll
+  for (int qi = 0; qi < QB; ++qi) {
+    m_run[qi] = -1.0e30f;
+    l_run[qi] = 0.0f;
+  }
 
   // tiles at or beyond the end of the sequence lie outside the buffers and load as zeros
   // requests of a wave that may stay in flight where an iteration waits for its tiles: those of the
@@ -472,7 +502,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   }
   __builtin_amdgcn_s_waitcnt(WAIT_TILES);
   __syncthreads();
-  f32x16 s_cur[2], s_nxt[2];
+  f32x16 s_cur[QB][2], s_nxt[QB][2];
   scores(sKbase, s_cur);
 
   // Masks tile `tile`'s scores in s (EDGE only) and folds them into the running
@@ -480,55 +510,63 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // the scale is folded into the exponent's multiply-add.  Leaves the rescale
   // factor of the earlier tiles in `alpha` (exactly 1 where the maximum did not
   // move) and returns whether this lane's maximum moved.
-  float alpha = 1.0f;
-  auto take_max = [&](int tile, auto edge_tag, f32x16 (&s)[2]) -> bool {
+  float alpha[QB];
+#pragma unroll
+  for (int qi = 0; qi < QB; ++qi) alpha[qi] = 1.0f;
+  auto take_max = [&](int tile, auto edge_tag, f32x16 (&s)[QB][2]) -> bool {
     constexpr bool EDGE = decltype(edge_tag)::value;
     const int kv0 = tile * FA_BKV;
-    float mx = -INFINITY;
+    bool moved = false;
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk)
+    for (int qi = 0; qi < QB; ++qi) {
+      float mx = -INFINITY;
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        if constexpr (EDGE) {
-          const int kv = kv0 + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-          const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine));
-          s[blk][e] = dead ? -INFINITY : s[blk][e];
+      for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          if constexpr (EDGE) {
+            const int kv = kv0 + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+            const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine[qi]));
+            s[qi][blk][e] = dead ? -INFINITY : s[qi][blk][e];
+          }
+          mx = fmaxf(mx, s[qi][blk][e]);
         }
-        mx = fmaxf(mx, s[blk][e]);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx * a.scale_log2);
-    const bool moved = m_new > m_run;
-    alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[qi], mx * a.scale_log2);
+      moved |= m_new > m_run[qi];
+      alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - m_new);
+      m_run[qi] = m_new;
+    }
     return moved;
   };
   // alpha is exactly 1 for every lane whose maximum did not move: the 16*DB
   // multiplies are skipped unless some lane of the wave needs them
-  auto rescale = [&](bool moved) {
+  auto rescale = [&](bool moved) __attribute__((always_inline)) {
     if (__any(moved)) {
 #pragma unroll
-      for (int d = 0; d < DB; ++d)
+      for (int qi = 0; qi < QB; ++qi)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o[qi][d][e] *= alpha[qi];
     }
   };
   // One scheduling region: the score product of tile t+1 on the matrix pipe, the
   // exponentials and row sums of tile t (maximum m_run, rescale factor alpha) on
   // the vector ALU.
-  u32x4 pf[4];
-  auto softmax_and_next_scores = [&](int t) {
+  u32x4 pf[QB][4];
+  auto softmax_and_next_scores = [&](int t) __attribute__((always_inline)) {  // (one query block per wave)
     const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) s_nxt[blk][e] = 0.0f;
+      for (int e = 0; e < 16; ++e) s_nxt[0][blk][e] = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
         const u32x4 kf = *(const u32x4 *)(sKn + k_piece(blk * 32 + lrow, ks * 2 + g));
-        s_nxt[blk] = Mfma32<DT>::run(kf, qf[ks], s_nxt[blk]);
+        s_nxt[0][blk] = Mfma32<DT>::run(kf, qf[0][ks], s_nxt[0][blk]);
       }
     float lsum = 0.0f;
 #pragma unroll
@@ -538,17 +576,17 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         float p[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[blk][hh * 8 + j], a.scale_log2, -m_run));
+          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[0][blk][hh * 8 + j], a.scale_log2, -m_run[0]));
           lsum += p[j];
         }
-        pf[blk * 2 + hh] = pack8<DT>(p);
+        pf[0][blk * 2 + hh] = pack8<DT>(p);
       }
-    l_run = l_run * alpha + lsum;
+    l_run[0] = l_run[0] * alpha[0] + lsum;
     Interleave3<0, 2 * KS>::run();
     __builtin_amdgcn_sched_barrier(0);
   };
   // The transposed V operand of P.V step (kk, d): V rows kk*16.., head-dim block d.
-  auto read_v = [&](const unsigned char *sV, int kk, int d) -> u32x4 {
+  auto read_v = [&](const unsigned char *sV, int kk, int d) __attribute__((always_inline)) -> u32x4 {
     const int r = lane & 15;
     const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
     const int row_lo = kk * 16 + g * 4 + (r >> 2);
@@ -568,7 +606,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // branch-free up to the optional rescale, so MFMAs and vector-ALU work can be
   // interleaved instruction by instruction.  For EARLY_MAX the tag describes
   // tile t+1, the one whose maximum the iteration takes.
-  auto iteration = [&](int t, auto edge_tag) {
+  auto iteration = [&](int t, auto edge_tag) __attribute__((always_inline)) {
     const unsigned char *sV = sVbase + (t % NSTG) * TILE_BYTES;
     if constexpr (!EARLY_MAX) {
       const bool moved = take_max(t, edge_tag, s_cur);
@@ -578,7 +616,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-        for (int d = 0; d < DB; ++d) o[d] = Mfma32<DT>::run(read_v(sV, kk, d), pf[kk], o[d]);
+        for (int d = 0; d < DB; ++d) o[0][d] = Mfma32<DT>::run(read_v(sV, kk, d), pf[0][kk], o[0][d]);
     } else {
       // Both phases are written as short chunks -- a few MFMAs and their share of
       // the vector-ALU work -- each closed by a full scheduling fence: MFMA issue
@@ -588,18 +626,22 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       constexpr bool EDGE = decltype(edge_tag)::value;
       const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
       // ---- phase A: S^T(t+1) = K(t+1) Q^T  with  P(t) = exp2(S(t)*scale - m), row sums ----
-      // chunk ks: the two MFMAs of k-step ks (operands read one chunk ahead) and
-      // 32/KS of the 32 exponentials
-      constexpr int EPC = 32 / KS;  // exponentials per chunk
-      static_assert(32 % KS == 0 && (EPC == 4 || EPC == 8), "exponentials must divide over the k-steps");
+      // chunk ks: the 2*QB MFMAs of k-step ks (operands read one chunk ahead) and
+      // 32*QB/KS of the 32*QB exponentials
+      constexpr int EPC = 32 * QB / KS;  // exponentials per chunk
+      static_assert((32 * QB) % KS == 0 && (EPC == 4 || EPC == 8 || EPC == 16), "exponentials must divide over the k-steps");
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk)
+      for (int qi = 0; qi < QB; ++qi)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) s_nxt[blk][e] = 0.0f;
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) s_nxt[qi][blk][e] = 0.0f;
       u32x4 kf0 = *(const u32x4 *)(sKn + k_piece(lrow, g));
       u32x4 kf1 = *(const u32x4 *)(sKn + k_piece(32 + lrow, g));
-      float lsum = 0.0f;
+      float lsum[QB];
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) lsum[qi] = 0.0f;
       float p[8];
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
@@ -608,32 +650,41 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           kn0 = *(const u32x4 *)(sKn + k_piece(lrow, (ks + 1) * 2 + g));
           kn1 = *(const u32x4 *)(sKn + k_piece(32 + lrow, (ks + 1) * 2 + g));
         }
-        s_nxt[0] = Mfma32<DT>::run(kf0, qf[ks], s_nxt[0]);
-        s_nxt[1] = Mfma32<DT>::run(kf1, qf[ks], s_nxt[1]);
+#pragma unroll
+        for (int qi = 0; qi < QB; ++qi) {
+          s_nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], s_nxt[qi][0]);
+          s_nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], s_nxt[qi][1]);
+        }
 #pragma unroll
         for (int j = 0; j < EPC; ++j) {
-          const int idx = ks * EPC + j;  // 0..31 over (blk, hh, j8): blk = idx/16, element idx%16
-          const float x = __builtin_amdgcn_exp2f(fmaf(s_cur[idx >> 4][idx & 15], a.scale_log2, -m_run));
+          const int idx = ks * EPC + j;  // 0..32*QB-1 over (query block, blk, element): block idx/32, blk (idx%32)/16
+          const int qi = idx >> 5, w = idx & 31;
+          const float x = __builtin_amdgcn_exp2f(fmaf(s_cur[qi][w >> 4][w & 15], a.scale_log2, -m_run[qi]));
           p[idx & 7] = x;
-          lsum += x;
-          if ((idx & 7) == 7) pf[idx >> 3] = pack8<DT>(p);
+          lsum[qi] += x;
+          if ((idx & 7) == 7) pf[qi][w >> 3] = pack8<DT>(p);
         }
         // The row sum is not needed before the next iteration, and the compiler would sink
-        // its 32 additions, one dependent chain, out of the chunks into the tail of the loop
+        // its additions, one dependent chain, out of the chunks into the tail of the loop
         // body, behind every MFMA: pinning the partial sum at the end of each chunk keeps
         // the additions where the matrix pipe hides them.
-        asm volatile("" : "+v"(lsum));
+#pragma unroll
+        for (int qi = 0; qi < QB; ++qi) asm volatile("" : "+v"(lsum[qi]));
         kf0 = kn0;
         kf1 = kn1;
+        if constexpr (QB > 1) MfmaValu<0, 2 * QB, (EPC * 7 / 2 + 2 * QB - 1) / (2 * QB), 2>::run();
         __builtin_amdgcn_sched_barrier(0);
       }
-      l_run = l_run * alpha + lsum;
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) l_run[qi] = l_run[qi] * alpha[qi] + lsum[qi];
 
       // ---- phase B: O^T += V^T(t) P^T(t)  with  the running maximum of tile t+1 ----
-      // chunk kk: the DB MFMAs of key block kk (operand reads one MFMA ahead) and
-      // the maximum over 8 of the 32 scores of S(t+1)
+      // chunk kk: the DB*QB MFMAs of key block kk (operand reads one fragment ahead) and
+      // the maximum over 8 of the 32 scores of S(t+1) of each query block
       const int kv0n = (t + 1) * FA_BKV;
-      float mx = -INFINITY;
+      float mx[QB];
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) mx[qi] = -INFINITY;
       u32x4 vf = read_v(sV, 0, 0);
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
@@ -641,30 +692,40 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         for (int d = 0; d < DB; ++d) {
           const int nxt = kk * DB + d + 1;
           const u32x4 vn = nxt < 4 * DB ? read_v(sV, nxt / DB, nxt % DB) : vf;
-          o[d] = Mfma32<DT>::run(vf, pf[kk], o[d]);
+#pragma unroll
+          for (int qi = 0; qi < QB; ++qi) o[qi][d] = Mfma32<DT>::run(vf, pf[qi][kk], o[qi][d]);
           vf = vn;
         }
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const int idx = kk * 8 + j, blk = idx >> 4, e = idx & 15;
-          if constexpr (EDGE) {
-            const int kv = kv0n + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-            const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine));
-            s_nxt[blk][e] = dead ? -INFINITY : s_nxt[blk][e];
+        for (int qi = 0; qi < QB; ++qi)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            const int idx = kk * 8 + j, blk = idx >> 4, e = idx & 15;
+            if constexpr (EDGE) {
+              const int kv = kv0n + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
+              const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine[qi]));
+              s_nxt[qi][blk][e] = dead ? -INFINITY : s_nxt[qi][blk][e];
+            }
+            mx[qi] = fmaxf(mx[qi], s_nxt[qi][blk][e]);
           }
-          mx = fmaxf(mx, s_nxt[blk][e]);
-        }
+        if constexpr (QB > 1) MfmaValu<0, DB * QB, (8 * QB * (EDGE ? 4 : 1) + DB * QB - 1) / (DB * QB), 2 * DB>::run();
         __builtin_amdgcn_sched_barrier(0);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx * a.scale_log2);
-      const bool moved = m_new > m_run;
-      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      m_run = m_new;
+      bool moved = false;
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) {
+        const float mw = fmaxf(mx[qi], __shfl_xor(mx[qi], 32, 64));
+        const float m_new = fmaxf(m_run[qi], mw * a.scale_log2);
+        moved |= m_new > m_run[qi];
+        alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - m_new);
+        m_run[qi] = m_new;
+      }
       rescale(moved);
     }
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) s_cur[blk] = s_nxt[blk];
+    for (int qi = 0; qi < QB; ++qi)
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) s_cur[qi][blk] = s_nxt[qi][blk];
   };
 
   // Interior tiles first, then the edge tiles (they are the last ones: the tail of
@@ -705,29 +766,32 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);  // look-ahead loads must not land on the output staging
   __syncthreads();
 
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv_l = 1.0f / l_tot;
-  unsigned char *so = smem + wave * (32 * ROW_BYTES);
+  unsigned char *so = smem + wave * (WQ * ROW_BYTES);
 #pragma unroll
-  for (int d = 0; d < DB; ++d)
+  for (int qi = 0; qi < QB; ++qi) {
+    const float l_tot = l_run[qi] + __shfl_xor(l_run[qi], 32, 64);
+    const float inv_l = 1.0f / l_tot;
 #pragma unroll
-    for (int v4 = 0; v4 < 4; ++v4) {
-      float x[4];
+    for (int d = 0; d < DB; ++d)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[e] = o[d][v4 * 4 + e] * inv_l;
-      u32x2 w;
-      if constexpr (DT == DT_F16) {
-        f16x4 hq = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
-        w = __builtin_bit_cast(u32x2, hq);
-      } else {
-        bf16x4 hq = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
-        w = __builtin_bit_cast(u32x2, hq);
+      for (int v4 = 0; v4 < 4; ++v4) {
+        float x[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[e] = o[qi][d][v4 * 4 + e] * inv_l;
+        u32x2 w;
+        if constexpr (DT == DT_F16) {
+          f16x4 hq = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+          w = __builtin_bit_cast(u32x2, hq);
+        } else {
+          bf16x4 hq = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
+          w = __builtin_bit_cast(u32x2, hq);
+        }
+        *(u32x2 *)(so + (qi * 32 + lrow) * ROW_BYTES + (d * 32 + v4 * 8 + g * 4) * 2) = w;
       }
-      *(u32x2 *)(so + lrow * ROW_BYTES + (d * 32 + v4 * 8 + g * 4) * 2) = w;
-    }
+  }
   __syncthreads();
 #pragma unroll
-  for (int i = 0; i < 32 * CH / 64; ++i) {
+  for (int i = 0; i < WQ * CH / 64; ++i) {
     const int p = lane + i * 64;
     const int row = p / CH, c = p % CH;
     const int q = q_wave0 + row;
@@ -736,15 +800,15 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   }
 }
 
-template <int D, bool EARLY_MAX, int WAVES, int NSTG>
+template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
-  constexpr size_t ring = 2 * (size_t)NSTG * FA_BKV * D * 2, staging = (size_t)WAVES * 32 * D * 2;
+  constexpr size_t ring = 2 * (size_t)NSTG * FA_BKV * D * 2, staging = (size_t)WAVES * 32 * QB * D * 2;
   constexpr size_t lds = ring > staging ? ring : staging;
-  const int nqb = (a.S + 32 * WAVES - 1) / (32 * WAVES);
+  const int nqb = (a.S + 32 * QB * WAVES - 1) / (32 * QB * WAVES);
   const dim3 grid((unsigned)(nqb * a.B * a.H)), block(WAVES * 64);
 #define TRACEA_FA_LAUNCH(DTV)                                                                  \
   do {                                                                                         \
-    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG>;                            \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB>;                        \
     static bool attr_done = false;                                                             \
     if (!attr_done) {                                                                          \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
@@ -805,6 +869,8 @@ static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 static const AttentionVariant kAttentionVariants[] = {
     {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128},
     {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64},
+    {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128},
+    {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64},
     {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128},
     {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64},
     {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64},
