@@ -101,6 +101,22 @@ char *tracea_tuning_cache_get(const char *key);
 int32_t tracea_tuning_cache_put(const char *key, const char *config_json, float score, uint64_t timestamp);
 /* Forgets the in-memory copy; the next access re-reads the file. */
 void tracea_tuning_cache_reload(void);
+/* ---- tuning history: src/optimizer/history.rs:7-51 ----------------------------------- */
+/* The reference's second record of tuning results, tuning_history.json in the working directory
+ * (override: TRACEA_TUNING_HISTORY): a map key -> {backend, config, tflops, timestamp, explanation},
+ * keys "HardwareId:OpFingerprint:Precision" (history.rs:17).  tracea_tune_* record the winner of every
+ * measurement here under "<device name>:<cache key>:<F16|BF16|FP32>" with backend "Rocm". */
+char *tracea_tuning_history_path(void);
+/* TuningHistory::record (history.rs:38-41): inserts / replaces and rewrites the file.  The explanation is
+ * generate_explanation's sentence (history.rs:47-52) built from backend, tflops and `reason`.  0 ok, -1 bad
+ * argument. */
+int32_t tracea_tuning_history_record(const char *key, const char *config_json, float tflops, uint64_t timestamp,
+                                     const char *reason);
+/* TuningHistory::query (history.rs:43-45): the entry as JSON, or NULL when the key is absent. */
+char *tracea_tuning_history_query(const char *key);
+/* Forgets the in-memory copy; the next access re-reads the file (load_or_create, history.rs:22-29). */
+void tracea_tuning_history_reload(void);
+
 /* Keys as the reference spells them (tuning.rs:66-78). */
 char *tracea_tuning_key_gemm(uint64_t m, uint64_t n, uint64_t k, const char *device_name);
 char *tracea_tuning_key_conv2d(uint32_t batch, uint32_t h, uint32_t w, uint32_t c, uint32_t k, uint32_t r,

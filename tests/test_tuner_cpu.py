@@ -340,6 +340,49 @@ def test_cache_file_format_and_reload(cache_file):
     assert got["score"] == 1.5 and got["config"]["num_stages"] == 3 and got["config"]["fusion_count"] == 1
 
 
+# ---- tuning history (src/optimizer/history.rs:7-51) -----------------------------------
+def test_history_file_format_and_reload(tmp_path, monkeypatch):
+    path = tmp_path / "tuning_history.json"
+    monkeypatch.setenv("TRACEA_TUNING_HISTORY", str(path))
+    T.history_reload()
+    try:
+        assert T.history_path() == str(path)
+        assert T.history_query("all:gemm:FP16") is None
+        cfg = T.pipeline_config(2, 128, 128, 64)
+        T.history_record("all:gemm:FP16", cfg, 1234.567, 0, "Selected based on highest benchmarking score in real-time.")
+        on_disk = json.loads(path.read_text())
+        assert list(on_disk) == ["all:gemm:FP16"]
+        entry = on_disk["all:gemm:FP16"]
+        # HistoryEntry's fields (history.rs:7-13); DeviceBackend::Rocm as serde spells a unit variant
+        assert set(entry) == {"backend", "config", "tflops", "timestamp", "explanation"}
+        assert entry["backend"] == "Rocm" and entry["config"] == cfg and entry["timestamp"] == 0
+        assert abs(entry["tflops"] - 1234.567) < 1e-3
+        # generate_explanation (history.rs:47-52): "{:?}" of the backend, "{:.2}" of the score
+        assert entry["explanation"] == ("Selected Rocm because it achieved 1234.57 TFLOPS. Reason: "
+                                        "Selected based on highest benchmarking score in real-time.")
+        assert "\n  " in path.read_text()  # to_string_pretty
+        # record replaces (HashMap::insert)
+        T.history_record("all:gemm:FP16", cfg, 2.0, 7, "again")
+        assert T.history_query("all:gemm:FP16")["tflops"] == 2.0
+        # a file written by the reference (another backend, the placeholder timestamp) is read after a reload
+        on_disk["all:conv:FP16"] = {"backend": "Cuda", "config": {"num_stages": 3, "m_tile": 64, "n_tile": 64, "k_tile": 32},
+                                    "tflops": 9.5, "timestamp": 0, "explanation": "Selected Cuda because it achieved 9.50 TFLOPS. Reason: x"}
+        path.write_text(json.dumps(on_disk))
+        assert T.history_query("all:conv:FP16") is None
+        T.history_reload()
+        got = T.history_query("all:conv:FP16")
+        assert got["backend"] == "Cuda" and got["tflops"] == 9.5 and got["config"]["m_tile"] == 64
+        # a file that does not parse is an empty history (load_or_create)
+        path.write_text("{ not json")
+        T.history_reload()
+        assert T.history_query("all:conv:FP16") is None
+        with pytest.raises(ValueError):
+            T.history_record("", cfg, 1.0)
+    finally:
+        monkeypatch.delenv("TRACEA_TUNING_HISTORY")
+        T.history_reload()
+
+
 # ---- AutoTuner ----------------------------------------------------------------------
 def test_autotune_grid_search_caches_the_winner(cache_file):
     cands = T.propose_gemm_configs(1024, 1024, 1024)

@@ -19,10 +19,14 @@ def cache_file(tmp_path, monkeypatch):
     from tracea_amd import tuner as T
     path = tmp_path / "tuning_cache_v2.json"
     monkeypatch.setenv("TRACEA_TUNING_CACHE", str(path))
+    monkeypatch.setenv("TRACEA_TUNING_HISTORY", str(tmp_path / "tuning_history.json"))
     T.cache_reload()
+    T.history_reload()
     yield path
     monkeypatch.delenv("TRACEA_TUNING_CACHE")
+    monkeypatch.delenv("TRACEA_TUNING_HISTORY")
     T.cache_reload()
+    T.history_reload()
 
 
 def _device_name():
@@ -40,6 +44,11 @@ def test_tune_gemm_records_a_runnable_winner(tracea_gpu, cache_file):
     keys = [k for k in disk if k.startswith("gemm_1024_1024_512_")]
     assert len(keys) == 1
     assert disk[keys[0]]["config"] == cfg and disk[keys[0]]["score"] == pytest.approx(score)
+    # the same winner in the tuning history (src/optimizer/history.rs), key "HardwareId:OpFingerprint:Precision"
+    hist = json.loads((cache_file.parent / "tuning_history.json").read_text())
+    entry = hist["%s:%s:F16" % (_device_name(), keys[0])]
+    assert entry["backend"] == "Rocm" and entry["config"] == cfg and entry["tflops"] == pytest.approx(score)
+    assert entry["explanation"].startswith("Selected Rocm because it achieved %.2f TFLOPS." % score)
     # the operator still computes the right product afterwards (forced variant restored)
     rng = np.random.default_rng(5)
     a = round_f16(rng.standard_normal((1024, 512)).astype(np.float32) / np.sqrt(512))

@@ -188,6 +188,10 @@ SIGNATURES.update({
     "tracea_tuning_cache_get": (_STR, [C.c_char_p]),
     "tracea_tuning_cache_put": (C.c_int32, [C.c_char_p, C.c_char_p, C.c_float, C.c_uint64]),
     "tracea_tuning_cache_reload": (None, []),
+    "tracea_tuning_history_path": (_STR, []),
+    "tracea_tuning_history_record": (C.c_int32, [C.c_char_p, C.c_char_p, C.c_float, C.c_uint64, C.c_char_p]),
+    "tracea_tuning_history_query": (_STR, [C.c_char_p]),
+    "tracea_tuning_history_reload": (None, []),
     "tracea_tuning_key_gemm": (_STR, [C.c_uint64] * 3 + [C.c_char_p]),
     "tracea_tuning_key_conv2d": (_STR, [C.c_uint32] * 9 + [C.c_char_p]),
     "tracea_autotune_candidates": (Result, [C.c_char_p, C.c_char_p, MEASURE_FN, C.c_void_p]),

@@ -107,6 +107,80 @@ void tuning_cache_reload() {
   g_loaded = false;
 }
 
+// ---- tuning history (src/optimizer/history.rs) ----
+namespace {
+std::mutex g_hist_mu;
+std::map<std::string, HistoryEntry> g_hist;
+bool g_hist_loaded = false;
+
+void hist_load_locked() {
+  if (g_hist_loaded) return;
+  g_hist_loaded = true;
+  std::ifstream f(tuning_history_path());
+  if (!f) return;
+  std::stringstream ss;
+  ss << f.rdbuf();
+  Json root;
+  std::string err;
+  // (a file that does not parse is an empty history, as load_or_create has it)
+  if (!Json::parse(ss.str(), &root, &err) || root.type != Json::Object) return;
+  for (const auto &kv : root.obj) {
+    const Json *cfg = kv.second.find("config");
+    HistoryEntry e;
+    if (!cfg || !PipelineConfig::from_json_value(*cfg, &e.config, &err)) continue;
+    if (const Json *b = kv.second.find("backend")) e.backend = b->str;
+    if (const Json *t = kv.second.find("tflops")) e.tflops = (float)t->num;
+    if (const Json *t = kv.second.find("timestamp")) e.timestamp = (uint64_t)t->num;
+    if (const Json *x = kv.second.find("explanation")) e.explanation = x->str;
+    g_hist[kv.first] = e;
+  }
+}
+}  // namespace
+
+std::string tuning_history_path() {
+  const char *env = getenv("TRACEA_TUNING_HISTORY");
+  return env && *env ? std::string(env) : std::string("tuning_history.json");
+}
+
+std::string tuning_history_explanation(const std::string &backend, float tflops, const std::string &reason) {
+  char buf[96];
+  snprintf(buf, sizeof(buf), "%.2f", (double)tflops);
+  return "Selected " + backend + " because it achieved " + buf + " TFLOPS. Reason: " + reason;
+}
+
+bool tuning_history_query(const std::string &key, HistoryEntry *out) {
+  std::lock_guard<std::mutex> lk(g_hist_mu);
+  hist_load_locked();
+  auto it = g_hist.find(key);
+  if (it == g_hist.end()) return false;
+  if (out) *out = it->second;
+  return true;
+}
+
+void tuning_history_record(const std::string &key, const HistoryEntry &e) {
+  std::lock_guard<std::mutex> lk(g_hist_mu);
+  hist_load_locked();
+  g_hist[key] = e;
+  Json root = Json::make_obj();
+  for (const auto &kv : g_hist) {
+    Json j = Json::make_obj();
+    j.set("backend", Json::make_str(kv.second.backend));
+    j.set("config", kv.second.config.to_json_value());
+    j.set("tflops", Json::make_num(kv.second.tflops));
+    j.set("timestamp", Json::make_num((double)kv.second.timestamp));
+    j.set("explanation", Json::make_str(kv.second.explanation));
+    root.set(kv.first, j);
+  }
+  std::ofstream f(tuning_history_path());
+  if (f) f << root.dump(2) << "\n";
+}
+
+void tuning_history_reload() {
+  std::lock_guard<std::mutex> lk(g_hist_mu);
+  g_hist.clear();
+  g_hist_loaded = false;
+}
+
 int tuning_cache_lookup_variant(const std::string &key) {
   CacheEntry e;
   if (!tuning_cache_get(key, &e)) return -1;
@@ -354,6 +428,17 @@ bool conv_dims_ok(size_t n, size_t c, size_t h, size_t w, size_t k, size_t r, si
 
 }  // namespace
 
+// The winner of a measurement, in the tuning history as well (the reference's orchestrator records what
+// it selects, src/optimizer/orchestrator.rs:68-81): key "HardwareId:OpFingerprint:Precision".
+static void record_history(const std::string &cache_key, const CacheEntry &e, const char *precision) {
+  HistoryEntry h;
+  h.config = e.config;
+  h.tflops = e.score;
+  h.timestamp = e.timestamp;
+  h.explanation = tuning_history_explanation(h.backend, h.tflops, "Selected based on highest benchmarking score in real-time.");
+  tuning_history_record(std::string(tuning_device_name()) + ":" + cache_key + ":" + precision, h);
+}
+
 TraceaResult tune_gemm(size_t m, size_t n, size_t k) {
   if (!runtime_ready()) return failure("tracea_init has not been called");
   if (!gemm_dims_ok(m, n, k)) return failure("tune_gemm: dimensions must be positive, K a multiple of 8");
@@ -374,6 +459,7 @@ TraceaResult tune_gemm(size_t m, size_t n, size_t k) {
   e.score = best_tflops;
   e.timestamp = now_seconds();
   tuning_cache_put(gemm_cache_key(m, n, k, tuning_device_name()), e, true);
+  record_history(gemm_cache_key(m, n, k, tuning_device_name()), e, "F16");
   return success(e.config, e.score);
 }
 
@@ -404,6 +490,7 @@ TraceaResult tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_
   p.c_out = (uint32_t)k; p.kernel_h = (uint32_t)r; p.kernel_w = (uint32_t)s;
   p.stride = (uint32_t)stride; p.pad = (uint32_t)pad; p.dilation = (uint32_t)dilation;
   tuning_cache_put(conv_cache_key(p, tuning_device_name()), e, true);
+  record_history(conv_cache_key(p, tuning_device_name()), e, "F16");
   return success(e.config, e.score);
 }
 
@@ -546,6 +633,7 @@ TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
   char key[200];
   snprintf(key, sizeof(key), "fa2_kernel:b%zu_s%zu_h%zu_d%zu_%s", b, s, h, d, causal ? "causal" : "dense");
   tuning_cache_put(key, e, true);
+  record_history(key, e, "BF16");
   return success(e.config, e.score);
 }
 

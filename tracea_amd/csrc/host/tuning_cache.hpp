@@ -25,6 +25,21 @@ void tuning_cache_put(const std::string &key, const CacheEntry &e, bool persist)
 // Drops the in-memory copy so that the next lookup re-reads the file.
 void tuning_cache_reload();
 
+// Tuning history (src/optimizer/history.rs:7-51): key -> {backend, config, tflops, timestamp, explanation}
+// in tuning_history.json (TRACEA_TUNING_HISTORY overrides the path).
+struct HistoryEntry {
+  std::string backend = "Rocm";
+  PipelineConfig config;
+  float tflops = 0.0f;
+  uint64_t timestamp = 0;
+  std::string explanation;
+};
+std::string tuning_history_path();
+std::string tuning_history_explanation(const std::string &backend, float tflops, const std::string &reason);
+bool tuning_history_query(const std::string &key, HistoryEntry *out);
+void tuning_history_record(const std::string &key, const HistoryEntry &e);
+void tuning_history_reload();
+
 // Index of the contraction variant a cached config names, or -1.
 int tuning_cache_lookup_variant(const std::string &key);
 

@@ -294,6 +294,31 @@ int32_t tracea_tuning_cache_put(const char *key, const char *config_json, float 
 
 void tracea_tuning_cache_reload(void) { tuning_cache_reload(); }
 
+char *tracea_tuning_history_path(void) {
+  TUNER_GUARDED(nullptr, return dup_cstr(tuning_history_path());)
+}
+
+int32_t tracea_tuning_history_record(const char *key, const char *config_json, float tflops, uint64_t timestamp,
+                                     const char *reason) {
+  TUNER_GUARDED(-1, HistoryEntry e; if (key == nullptr || *key == 0) {
+    fail(TRACEA_INVALID_PARAMS, "tuning_history_record: empty key");
+    return -1;
+  } if (!parse_config(config_json, &e.config)) return -1;
+                e.tflops = tflops; e.timestamp = timestamp;
+                e.explanation = tuning_history_explanation(e.backend, tflops, reason ? reason : "");
+                tuning_history_record(key, e); return 0;)
+}
+
+char *tracea_tuning_history_query(const char *key) {
+  TUNER_GUARDED(nullptr, HistoryEntry e; if (key == nullptr || !tuning_history_query(key, &e)) return nullptr;
+                Json j = Json::make_obj(); j.set("backend", Json::make_str(e.backend));
+                j.set("config", e.config.to_json_value()); j.set("tflops", Json::make_num(e.tflops));
+                j.set("timestamp", Json::make_num((double)e.timestamp));
+                j.set("explanation", Json::make_str(e.explanation)); return dup_cstr(j.dump());)
+}
+
+void tracea_tuning_history_reload(void) { tuning_history_reload(); }
+
 char *tracea_tuning_key_gemm(uint64_t m, uint64_t n, uint64_t k, const char *device_name) {
   TUNER_GUARDED(nullptr, return dup_cstr(gemm_cache_key(m, n, k, device_name ? device_name : ""));)
 }

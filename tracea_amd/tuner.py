@@ -194,6 +194,25 @@ def cache_reload():
     capi.lib().tracea_tuning_cache_reload()
 
 
+# ---- tuning history (src/optimizer/history.rs) ---------------------------------------
+def history_path():
+    return capi.take_string(capi.lib().tracea_tuning_history_path())
+
+
+def history_record(key, config, tflops, timestamp=0, reason=""):
+    if capi.lib().tracea_tuning_history_record(key.encode(), _cfg(config), tflops, timestamp, reason.encode()) != 0:
+        raise ValueError(capi.last_error())
+
+
+def history_query(key):
+    text = capi.take_string(capi.lib().tracea_tuning_history_query(key.encode()))
+    return None if text is None else json.loads(text)
+
+
+def history_reload():
+    capi.lib().tracea_tuning_history_reload()
+
+
 def key_gemm(m, n, k, device):
     return capi.take_string(capi.lib().tracea_tuning_key_gemm(m, n, k, device.encode()))
 
