@@ -14,6 +14,7 @@
 #include <map>
 #include <mutex>
 
+#include "tuner.hpp"
 #include "tuning_cache.hpp"
 
 namespace tracea_amd {
@@ -342,6 +343,38 @@ TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s,
 // (operand re-use of the tile shape x measured gain of its pipeline).  Partial
 // tiles at the edges are paid in full through the tile count.  A tuning-cache
 // entry, when present, wins over this.
+// What the selector knows of the device: CU count, LDS per workgroup and shader clock from the device
+// properties of device 0, read once after tracea_init; before that (variant queries without a device)
+// the figures of an MI355X.  The rate of a workgroup slot was calibrated at the MI355X's 2.4 GHz and
+// scales with the clock; a tuning-cache record of the calibration product (the 4096^3 GEMM on a
+// 256x256 direct-to-LDS tile) replaces it by what that device measured.
+const DeviceLimits &device_limits() {
+  static std::mutex mu;
+  static DeviceLimits lim;
+  static bool from_device = false;
+  std::lock_guard<std::mutex> lk(mu);
+  if (!from_device && runtime_ready()) {
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, 0) == hipSuccess) {
+      if (prop.multiProcessorCount > 0) lim.cus = prop.multiProcessorCount;
+      if (prop.sharedMemPerBlockOptin >= 64 * 1024) lim.lds_bytes = (long long)prop.sharedMemPerBlockOptin;
+      if (prop.clockRate > 0) lim.clock_ghz = prop.clockRate * 1e-6;
+      lim.slot_rate = 1.43e6 * lim.clock_ghz / 2.4;
+      CacheEntry e;
+      if (tuning_cache_get(gemm_cache_key(4096, 4096, 4096, prop.name), &e) && e.score > 0.0f) {
+        const int vi = contraction_variant_for_config(e.config);
+        if (vi >= 0 && contraction_variant(vi).bm == 256 && contraction_variant(vi).bn == 256 &&
+            contraction_variant(vi).pipeline == 2)
+          // score TFLOP/s = 2 MAC: MAC per microsecond and CU at the variant's efficiency prior (1.5, x1.04 on 8 waves)
+          lim.slot_rate = (double)e.score * 1e6 / 2.0 / lim.cus /
+                          (1.5 * (contraction_variant(vi).waves_m * contraction_variant(vi).waves_n == 8 ? 1.04 : 1.0));
+      }
+    }
+    from_device = true;
+  }
+  return lim;
+}
+
 namespace {
 // Number of K ranges for a launch of variant v (1: no split) and the extent of one range.
 // Pipelines 4 and 5 are convolution kernels of their own (input patch in LDS): they need the
@@ -351,8 +384,9 @@ inline bool conv_only(const ContractionVariant &v) { return v.pipeline >= 4; }
 int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split, int min_tiles = 4) {
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
-  if (conv_only(v) || tiles * 2 > 256 || nk < 2 * min_tiles) return 1;
-  long long splits = 256 / tiles;
+  const long long cus = device_limits().cus;
+  if (conv_only(v) || tiles * 2 > cus || nk < 2 * min_tiles) return 1;
+  long long splits = cus / tiles;
   if (splits > nk / min_tiles) splits = nk / min_tiles;  // at least min_tiles K tiles per range
   if (splits < 2) return 1;
   const int per = (int)((nk + splits - 1) / splits);
@@ -371,7 +405,8 @@ int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split,
 // unsplit 64x64 tiles / 128x128 tiles split four ways, where 53.7 / 29.6 us were measured.
 int select_contraction_variant(int m, int n, int k, bool conv) {
   (void)conv;
-  const double cus = 256.0, slot_rate = 1.43e6;  // multiply-accumulates per microsecond at efficiency 1
+  const DeviceLimits &dev = device_limits();
+  const double cus = (double)dev.cus, slot_rate = dev.slot_rate;  // multiply-accumulates per microsecond and CU at efficiency 1
   int best = -1;
   double best_cost = 0.0;
   for (int i = 0; i < contraction_variant_count(); ++i) {
@@ -401,7 +436,7 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
       // 128x64 tiles where the former leave CUs idle, and leaves the other choices alone
       // (defaults within 1.4 % / 1.6 % of the per-shape best in total on the two sets).
       const double lds = (double)v.stages * (v.bm + v.bn) * v.bk * 2.0;
-      const double fit = std::floor(160.0 * 1024.0 / lds) < 1.0 ? 1.0 : std::floor(160.0 * 1024.0 / lds);
+      const double fit = std::floor((double)dev.lds_bytes / lds) < 1.0 ? 1.0 : std::floor((double)dev.lds_bytes / lds);
       const double per_cu = units / cus < 1.0 ? 1.0 : (units / cus > fit ? fit : units / cus);
       const double waves = per_cu * v.waves_m * v.waves_n;
       if (waves < 8.0) prior *= std::sqrt(std::sqrt(waves / 8.0));
@@ -618,7 +653,8 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     static const ContractionVariant f32_tile128 = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr};
     static const ContractionVariant f32_tile64 = {"f32_64x64x16", 64, 64, 16, 2, 2, 1, 0, 0, nullptr};
     const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
-    const int tile = args.a_bytes != 0 && (double)((tiles64 + 255) / 256) * 1.06 < (double)((tiles128 + 255) / 256) * 4.0 ? 64 : 128;
+    const long long ncu = device_limits().cus;
+    const int tile = args.a_bytes != 0 && (double)((tiles64 + ncu - 1) / ncu) * 1.06 < (double)((tiles128 + ncu - 1) / ncu) * 4.0 ? 64 : 128;
     const ContractionVariant &f32_tile = tile == 64 ? f32_tile64 : f32_tile128;
     int k_split = 0;
     const int splits = g_split_k_enabled.load() ? choose_split(f32_tile, (int)M, (int)N, (int)K, &k_split, tile == 64 ? 16 : 4) : 1;
@@ -1162,7 +1198,7 @@ bool plan_conv_patch(const ConvGeometry &g, const ContractionVariant &v, bool w_
   const long long iters = (chunks + nt - 1) / nt;
   const long long patch_bytes = iters * nt * 16;
   const long long ring = (long long)v.stages * v.bn * 128;
-  if (patch_bytes + ring > 160 * 1024) return false;
+  if (patch_bytes + ring > device_limits().lds_bytes) return false;
   a->r_sz = b.r_sz;
   a->p_tiles = (hw + v.bm - 1) / v.bm;
   a->p_pw = (int)pw;
@@ -1197,7 +1233,7 @@ bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &
   if (pw * ph >= (1ll << 30)) return false;
   const int hw = b.h_out * b.w_out;
   const int grid_n = (g.n_gemm + v.bn - 1) / v.bn;
-  const long long cus = 256;
+  const long long cus = device_limits().cus;
   const long long t_min = (hw + v.bm - 1) / v.bm;
   const long long rounds = ((long long)b.batch * t_min * grid_n + cus - 1) / cus;
   long long tiles = rounds * cus / ((long long)b.batch * grid_n);
@@ -1206,7 +1242,6 @@ bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &
   const int tm = (int)((hw + tiles - 1) / tiles);
   tiles = (hw + tm - 1) / tm;
   const int cpp = (C / 8) | 1;
-  const int nt = 256;
   // the patch holds whole padded rows: p_seg load instructions of ppi pixels each per row; the largest
   // tile whose rows fit the kernel's fixed number of load instructions and the LDS left beside the
   // filters (shrinking the tile makes more workgroups)
@@ -1227,7 +1262,7 @@ bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &
     iters = (rows * seg + 7) / 8;
     patch_bytes = (rows * pw * cpp + 1) * 16;  // (+1: the repeated first part behind the last pixel)
     patch_bytes = (patch_bytes + 1023) / 1024 * 1024;
-    if (patch_bytes + (long long)v.lds_bytes <= 160 * 1024) break;
+    if (patch_bytes + (long long)v.lds_bytes <= device_limits().lds_bytes) break;
     if (tm_fit <= 32) return false;
     int next = tm_fit * 7 / 8 / 32 * 32;  // strictly smaller: rounded down to whole pixel blocks
     if (next >= tm_fit) next = tm_fit - 32;
@@ -1326,7 +1361,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline != 5) continue;
       ContractionArgs probe = a;
-      if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= 192 &&
+      if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n * 4 >= device_limits().cus * 3 &&
           probe.p_tm >= 320) {
         vi = i;
         resident_chosen = true;
@@ -1352,7 +1387,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline != 4 || cv.bm != 256 || cv.bn != 64) continue;
       ContractionArgs probe = a;
-      if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= 256 &&
+      if (plan_conv_patch(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n >= device_limits().cus &&
           hw * 4 >= (long long)probe.p_tiles * cv.bm * 3)
         chosen = i;
     }

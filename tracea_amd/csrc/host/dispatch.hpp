@@ -14,6 +14,15 @@ TraceaStatus fail(TraceaStatus st, const char *fmt, ...) __attribute__((format(p
 bool runtime_ready();
 int runtime_device_count();
 
+// Device figures the variant selector and the convolution plans work with (see device_limits()).
+struct DeviceLimits {
+  long long cus = 256;              // compute units
+  long long lds_bytes = 160 * 1024; // LDS a workgroup may use
+  double clock_ghz = 2.4;           // shader clock the device reports
+  double slot_rate = 1.43e6;        // multiply-accumulates per microsecond of one workgroup slot at efficiency 1
+};
+const DeviceLimits &device_limits();
+
 // Convolution geometry with the reciprocal ("magic") numbers of every divisor
 // the coordinate mapping uses.
 struct ConvGeometry {
