@@ -172,6 +172,35 @@ def test_epilogue_chain_on_listed_tiles_only(tracea_gpu):
     _check(out, want, listed, k, "f16", "chain on a lower-triangular layout")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_unevenly_shared_tiles_are_summed_and_unlisted_ones_left_alone(tracea_gpu, dtype):
+    # Tiles with different numbers of records (src/runtime/ttg_builder.rs:140-296 builds such lists when only
+    # some tiles split their K range): every listed tile is the sum of its own records, a tile without a
+    # record keeps its contents.  Ragged edges, an operator chain, records of one tile far apart in the list.
+    m, n, k = 320, 200, 384
+    a, b, da, db, tdt = _operands(m, n, k, dtype, 31)
+    recs = [(0, 0, 0, 128, 0), (1, 1, 0, 384, 0), (0, 0, 128, 256, 0), (2, 3, 64, 320, 0), (0, 0, 256, 384, 0),
+            (4, 0, 0, 192, 0), (4, 0, 192, 384, 0), (3, 2, 0, 384, 0)]
+    table = np.array(recs, dtype=TILE_DTYPE)
+    lay = TileLayout.from_tables(m, n, k, 64, 64, 32, list(range(len(recs))), table)
+    rng = np.random.default_rng(8)
+    bias = rng.standard_normal(n).astype(np.float32)
+    start = np.full((m, n), SENTINEL, np.float32)
+    out = _dev(start, tdt)
+    gemm_ttg(da, db, lay, out, ops=[(capi.OP_BIAS_ADD, torch.from_numpy(bias).cuda()), (capi.OP_RELU,)])
+    assert capi.lib().tracea_last_split_k() == 3
+    want, listed = _expected(a, b, lay, start, chain=lambda v, rows, cols: np.maximum(v + bias[None, cols], 0.0))
+    assert listed.sum() > 0 and (~listed).sum() > 0
+    _check(out, want, listed, k, dtype, "uneven sharing")
+    # the same list with every tile's records merged into one gives the same tiles (accumulation order aside)
+    merged = np.array([(0, 0, 0, 384, 0), (1, 1, 0, 384, 0), (2, 3, 64, 320, 0), (4, 0, 0, 384, 0), (3, 2, 0, 384, 0)],
+                      dtype=TILE_DTYPE)
+    out2 = _dev(start, tdt)
+    gemm_ttg(da, db, TileLayout.from_tables(m, n, k, 64, 64, 32, list(range(5)), merged), out2,
+             ops=[(capi.OP_BIAS_ADD, torch.from_numpy(bias).cuda()), (capi.OP_RELU,)])
+    _check(out2, want, listed, k, dtype, "merged records")
+
+
 def test_tables_in_a_caller_arena(tracea_gpu):
     # DeviceTTG::new_from_arena (src/runtime/ttg.rs:26-61): both tables inside one caller buffer
     m = n = 512
@@ -211,9 +240,6 @@ def test_empty_list_writes_nothing_and_bad_layouts_are_refused(tracea_gpu):
     empty = np.array([(0, 0, 64, 64, 0)], dtype=TILE_DTYPE)
     with pytest.raises(capi.TraceaError, match="empty k range"):
         gemm_ttg(da, db, TileLayout.from_tables(m, n, k, 64, 64, 32, [0], empty), out)
-    uneven = np.array([(0, 0, 0, 128, 0), (0, 0, 128, 256, 0), (1, 1, 0, 256, 0)], dtype=TILE_DTYPE)
-    with pytest.raises(capi.TraceaError, match="same number"):
-        gemm_ttg(da, db, TileLayout.from_tables(m, n, k, 64, 64, 32, [0, 1, 2], uneven), out)
     f32 = torch.zeros(m, k, device="cuda")
     with pytest.raises(capi.TraceaError, match="fp16 or bf16"):
         gemm_ttg(f32, f32, TileLayout.from_dense(m, n, k, 64, 64), torch.zeros(m, n, device="cuda"))

@@ -137,6 +137,11 @@ struct SplitKReduceArgs {
   int splits, M, N;
   long long ldc;
   EpilogueChain epi;
+  // Tile lists whose tiles have different numbers of records: tile_counts[tile row * grid_n + tile column]
+  // planes are summed for an element of that mt x nt tile, and a tile with none is left untouched.
+  // nullptr: every element sums `splits` planes.
+  const unsigned *tile_counts;
+  int mt, nt, grid_n;
 };
 int launch_splitk_reduce(const SplitKReduceArgs &args, hipStream_t stream);
 

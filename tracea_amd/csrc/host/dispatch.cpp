@@ -837,9 +837,10 @@ TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &ta, const TraceaTensorV
     args.epi = chain;
     return hip_status("gemm tile-list launch", v.launch(args, false, a.dtype, !b_kcontig, stream));
   }
-  if ((long long)tables.count != (long long)tables.slices * args.grid_m * args.grid_n)
-    return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: records that share a tile are summed only when every tile of the "
-                "grid has the same number of them", what);
+  // (tiles with different numbers of records: tables.counts tells the reduction how many planes each
+  // tile has, and to leave unlisted tiles alone)
+  if (tables.counts == nullptr && (long long)tables.count != (long long)tables.slices * args.grid_m * args.grid_n)
+    return fail(TRACEA_INVALID_PARAMS, "%s: the layout's tables carry no per-tile record counts", what);
   void *scratch = splitk_scratch(c.device, stream, (size_t)tables.slices * M * N * 4);
   if (scratch == nullptr)
     return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: %u partial products of %lldx%lld exceed the 64 MiB workspace", what,
@@ -850,6 +851,8 @@ TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &ta, const TraceaTensorV
   r.out = c.ptr; r.out_dtype = c.dtype;
   r.splits = (int)tables.slices; r.M = (int)M; r.N = (int)N; r.ldc = c.stride[0];
   r.epi = chain;
+  r.tile_counts = tables.counts;
+  r.mt = (int)layout.mt; r.nt = (int)layout.nt; r.grid_n = args.grid_n;
   args.C = scratch;
   args.ldc = N;
   args.out_dtype = DT_F32;

@@ -65,8 +65,9 @@ struct DeviceTileTables {
   const unsigned *l1 = nullptr;
   const unsigned *l2 = nullptr;
   const unsigned *slice = nullptr;
+  const unsigned *counts = nullptr;  // records per tile of the grid, when tiles differ in that (else nullptr)
   uint32_t count = 0;   // workgroups
-  uint32_t slices = 1;  // records per tile (all tiles alike when > 1)
+  uint32_t slices = 1;  // most records any tile has
   uint32_t k_gcd = 0;      // gcd of the k range lengths (k_end clipped to K) of all listed records
   uint32_t start_gcd = 0;  // gcd of their k_start (0: all start at 0)
 };

@@ -403,10 +403,15 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const SplitKReduceAr
   for (int e = 0; e < V; ++e) v[e] = 0.0f;
   const float *p = a.partial + m * a.N + n;
   const long long plane = (long long)a.M * a.N;
+  int splits = a.splits;
+  if (a.tile_counts != nullptr) {
+    splits = (int)a.tile_counts[(m / a.mt) * a.grid_n + n / a.nt];
+    if (splits == 0) return;  // no record names this tile: its elements are not written
+  }
   // eight planes at a time, loads first: with a few thousand threads and a serial chain of
   // loads per thread the kernel would be bound by memory latency times the split count
   int z = 0;
-  for (; z + 8 <= a.splits; z += 8) {
+  for (; z + 8 <= splits; z += 8) {
     if constexpr (V == 4) {
       f32x4 t[8];
 #pragma unroll
@@ -423,7 +428,7 @@ __global__ void __launch_bounds__(256) splitk_reduce_kernel(const SplitKReduceAr
       for (int u = 0; u < 8; ++u) v[0] += t[u];
     }
   }
-  for (; z < a.splits; ++z) {
+  for (; z < splits; ++z) {
     if constexpr (V == 4) {
       const f32x4 t = *(const f32x4 *)(p + z * plane);
 #pragma unroll

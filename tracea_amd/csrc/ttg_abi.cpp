@@ -20,14 +20,15 @@ static_assert(sizeof(TraceaTileEdge) == sizeof(TileEdge), "edge layout");
 namespace {
 
 struct DeviceCopy {
-  void *l1 = nullptr, *l2 = nullptr, *slice = nullptr;
-  bool owns_tables = false;  // l1 / l2 allocated here (slice always is)
+  void *l1 = nullptr, *l2 = nullptr, *slice = nullptr, *counts = nullptr;
+  bool owns_tables = false;  // l1 / l2 allocated here (slice and counts always are)
 };
 
 // What a launch needs to know about the listed records, found once per layout.
 struct LaunchInfo {
   std::vector<uint32_t> physical;  // workgroup -> record: the ordered level-1 map, regrouped per XCD
   std::vector<uint32_t> slice;     // workgroup -> how many earlier records (in table order) share its tile
+  std::vector<uint32_t> counts;    // records per tile of the grid; filled when the tiles differ in that
   uint32_t slices = 1, k_gcd = 0, start_gcd = 0;
   std::string error;               // non-empty: the layout cannot be launched, and why
 };
@@ -93,12 +94,16 @@ void analyse(TraceaTtgLayout *h) {
   }
   info.slice.resize(info.physical.size());
   for (size_t p = 0; p < info.physical.size(); ++p) info.slice[p] = occurrence[info.physical[p]];
-  if (info.slices > 1)
-    for (const auto &kv : seen)
-      if (kv.second != info.slices) {
-        info.slices = UINT32_MAX;  // uneven sharing: refused at launch
-        break;
-      }
+  // Tiles that share records unevenly (a K range split for some tiles only, or a partial list with
+  // shared tiles): the reduction then needs the count of every tile (0: unlisted, left untouched).
+  if (info.slices > 1) {
+    bool even = seen.size() == (size_t)gm * gn;
+    for (const auto &kv : seen) even = even && kv.second == info.slices;
+    if (!even) {
+      info.counts.assign((size_t)gm * gn, 0u);
+      for (const auto &kv : seen) info.counts[kv.first] = kv.second;
+    }
+  }
 }
 
 TraceaTtgLayout *finish(TileLayout &&l) {
@@ -153,9 +158,13 @@ TraceaStatus device_tables(TraceaTtgLayout *h, int device, void *l1_dst, void *l
     }
     if (e == hipSuccess && n1 > 0) e = hipMemcpy(copy.l1, h->info.physical.data(), n1, hipMemcpyHostToDevice);
     if (e == hipSuccess && n2 > 0) e = hipMemcpy(copy.l2, h->layout.l2_table.data(), n2, hipMemcpyHostToDevice);
-    if (e == hipSuccess && h->info.slices > 1 && h->info.slices != UINT32_MAX && copy.slice == nullptr) {
+    if (e == hipSuccess && h->info.slices > 1 && copy.slice == nullptr) {
       e = hipMalloc(&copy.slice, std::max<size_t>(n1, 4));
       if (e == hipSuccess && n1 > 0) e = hipMemcpy(copy.slice, h->info.slice.data(), n1, hipMemcpyHostToDevice);
+    }
+    if (e == hipSuccess && !h->info.counts.empty() && copy.counts == nullptr) {
+      e = hipMalloc(&copy.counts, h->info.counts.size() * 4);
+      if (e == hipSuccess) e = hipMemcpy(copy.counts, h->info.counts.data(), h->info.counts.size() * 4, hipMemcpyHostToDevice);
     }
     (void)hipSetDevice(prev);
     if (e != hipSuccess) {
@@ -164,6 +173,7 @@ TraceaStatus device_tables(TraceaTtgLayout *h, int device, void *l1_dst, void *l
         (void)hipFree(copy.l2);
       }
       (void)hipFree(copy.slice);
+      (void)hipFree(copy.counts);
       h->copies.erase(device);
       return hip_fail("tile tables", e);
     }
@@ -174,6 +184,7 @@ TraceaStatus device_tables(TraceaTtgLayout *h, int device, void *l1_dst, void *l
     out->l1 = (const unsigned *)it->second.l1;
     out->l2 = (const unsigned *)it->second.l2;
     out->slice = (const unsigned *)it->second.slice;
+    out->counts = (const unsigned *)it->second.counts;
     out->count = (uint32_t)h->info.physical.size();
     out->slices = h->info.slices;
     out->k_gcd = h->info.k_gcd;
@@ -189,9 +200,6 @@ TraceaStatus gemm_tiles(const TraceaTensorView &a, const TraceaTensorView &b, co
   if (h == nullptr || c == nullptr) return fail(TRACEA_INVALID_PARAMS, "tracea_gemm_ttg: layout or output view is NULL");
   if (c->device_id < 0 || c->device_id >= runtime_device_count())
     return fail(TRACEA_INVALID_PARAMS, "tracea_gemm_ttg: device %d does not exist", c->device_id);
-  if (h->info.slices == UINT32_MAX)
-    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_gemm_ttg: records that share a tile are summed only when every "
-                "tile of the grid has the same number of them");
   DeviceTileTables tables;
   if (h->info.physical.empty()) {
     if (!h->info.error.empty()) return fail(TRACEA_INVALID_PARAMS, "tile layout: %s", h->info.error.c_str());
@@ -302,6 +310,7 @@ void tracea_ttg_destroy(TraceaTtgLayout *layout) {
       (void)hipFree(kv.second.l2);
     }
     (void)hipFree(kv.second.slice);
+    (void)hipFree(kv.second.counts);
     (void)hipSetDevice(prev);
   }
   delete layout;
