@@ -43,6 +43,15 @@ TraceaStatus tracea_plan_output(const TraceaPlan *plan, uint64_t op_id, size_t *
  * "weight": filters [K,R,S,C] of a Conv2d node, right operand [K,N] of a Linear / Gemm node;
  * "weight_rsck" / "weight_t": the same in [R,S,C,K] / [N,K] storage. */
 TraceaStatus tracea_plan_bind(TraceaPlan *plan, uint64_t op_id, const char *slot, void *device_ptr);
+/* The same for callers that know what lies behind the pointer: `bytes` of memory holding elements of
+ * `dtype` (a TraceaDType, or -1 when unknown).  TRACEA_INVALID_PARAMS when a consumer of the Input node
+ * reads more bytes than that or reads another element type (data in the plan's type; the parameters of a
+ * BatchNorm are float32 channel vectors, given in the order gamma, beta, mean, var after the data input
+ * of a BatchNorm node and as gamma_id .. var_id of a fused one), or when a weight bank is shorter than
+ * K*R*S*C (Conv2d) or K*N (Linear, Gemm) elements of the plan's type.  (The reference's executor receives
+ * sized buffers from its runtime manager, src/runtime/plan.rs:40-53; a raw pointer carries no size.) */
+TraceaStatus tracea_plan_bind_sized(TraceaPlan *plan, uint64_t op_id, const char *slot, void *device_ptr,
+                                    size_t bytes, int32_t dtype);
 
 /* Launches every step on `stream`.  `arena` holds tracea_plan_arena_size bytes on `device`,
  * 256-byte aligned. */

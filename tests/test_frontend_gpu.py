@@ -79,6 +79,13 @@ def test_context_methods_write_the_callers_output_and_check_shapes(tracea):
         ctx.gemm(a, b, c, 64, 48, 16)
     q = torch.randn(1, 1, 128, 64, device="cuda").half()
     o = torch.empty_like(q)
+    # conv_transpose2d returns the kernel that ran: a convolution variant when the call went out by phase
+    xt = torch.randn(1, 8, 8, 16, device="cuda").half()
+    wt = torch.randn(16, 4, 4, 16, device="cuda").half() * 0.1
+    ot = torch.zeros(1, 16, 16, 16, device="cuda", dtype=torch.float16)
+    from tracea_amd import capi
+    kid_t = ctx.conv_transpose2d(xt, wt, ot, 1, 16, 8, 8, 16, 4, 4, stride=2, pad=1)
+    assert kid_t >= 0 and capi.variants("conv2d")[kid_t] == capi.last_variant("conv2d") and capi.last_variant("gemm") is None
     ctx.attention(q, q, q, o, 1, 1, 128, 64, 64, causal=False, scale_sqrt=False)
     want = torch.softmax(q[0, 0].float() @ q[0, 0].float().t(), dim=-1) @ q[0, 0].float()
     assert torch.allclose(o[0, 0].float(), want, atol=2e-2, rtol=0)
@@ -92,15 +99,20 @@ def test_module_matches_torch_and_falls_back(tracea):
     x = torch.randn(2, 16, 14, 14, device="cuda").half()
     from tracea_amd import capi
     capi.lib().tracea_force_variant(b"conv2d", -1)
-    y = m(x)
-    assert capi.last_variant("conv2d") is not None          # the library ran, not torch
-    assert tuple(y.shape) == tuple(ref(x).shape)
-    assert torch.allclose(y.float(), ref(x).float(), atol=3e-2, rtol=0)
-    # a changed weight is picked up (the repacked copy is per weight version)
     with torch.no_grad():
+        y = m(x)
+        assert capi.last_variant("conv2d") is not None          # the library ran, not torch
+        assert y.grad_fn is None and tuple(y.shape) == tuple(ref(x).shape)
+        assert torch.allclose(y.float(), ref(x).float(), atol=3e-2, rtol=0)
+        # a changed weight is picked up (the repacked copy is per weight version)
         m.weight.mul_(2.0)
         ref.weight.mul_(2.0)
-    assert torch.allclose(m(x).float(), ref(x).float(), atol=6e-2, rtol=0)
+        assert torch.allclose(m(x).float(), ref(x).float(), atol=6e-2, rtol=0)
+    # a step that needs gradients goes through PyTorch: the kernels here are forward only
+    yg = m(x)
+    assert yg.grad_fn is not None
+    yg.float().sum().backward()
+    assert m.weight.grad is not None and torch.isfinite(m.weight.grad.float()).all()
     # fp32 modules and grouped convolutions take torch's path and agree exactly
     ref32 = torch.nn.Conv2d(16, 32, 3, padding=1, groups=2).cuda()
     m32 = tracea.TraceaConv2d(16, 32, 3, padding=1, groups=2).cuda()
@@ -115,7 +127,8 @@ def test_patch_conv2d_builds_tracea_modules(tracea):
         layer = torch.nn.Conv2d(8, 8, 3, padding=1).cuda().half()
         assert isinstance(layer, tracea.TraceaConv2d)
         x = torch.randn(1, 8, 12, 12, device="cuda").half()
-        y = layer(x)
+        with torch.no_grad():
+            y = layer(x)
     finally:
         tracea.unpatch_conv2d()
     ref = torch.nn.functional.conv2d(x.float(), layer.weight.float(), layer.bias.float(), padding=1)

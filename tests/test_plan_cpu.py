@@ -129,6 +129,37 @@ def test_malformed_graphs_are_refused(graph, message):
         compile_plan(graph)
 
 
+def test_bind_sized_refuses_short_and_wrongly_typed_tensors():
+    # what a bound pointer must hold is known from the consumers of the Input node: the data input of the
+    # first convolution and the skip tensor in the plan's type, BatchNorm parameters as float32 vectors
+    n, ch, hw = 2, 16, 8
+    h = capi.lib().tracea_plan_compile(json.dumps(G.fuse(basic_block(n, ch, hw))).encode(), capi.F16)
+    assert h
+    try:
+        desc = json.loads(capi.take_string(capi.lib().tracea_plan_describe(h)))
+        first, second = desc["steps"]
+        bind = capi.lib().tracea_plan_bind_sized
+        ptr = C.c_void_p(4096)
+        x_bytes = n * hw * hw * ch * 2
+        assert bind(h, 0, b"input", ptr, x_bytes, capi.F16) == capi.SUCCESS
+        assert bind(h, 0, b"input", ptr, x_bytes + 512, -1) == capi.SUCCESS        # larger, type not stated
+        assert bind(h, 0, b"input", ptr, x_bytes - 2, capi.F16) == capi.INVALID_PARAMS
+        assert "holds %d bytes, the plan reads %d" % (x_bytes - 2, x_bytes) in capi.last_error()
+        assert bind(h, 0, b"input", ptr, x_bytes, capi.BF16) == capi.INVALID_PARAMS
+        gamma = first["epilogue"][0]["tensors"][0]
+        assert bind(h, gamma, b"input", ptr, ch * 4, capi.F32) == capi.SUCCESS
+        assert bind(h, gamma, b"input", ptr, ch * 2, capi.F16) == capi.INVALID_PARAMS   # a half-precision parameter vector
+        assert bind(h, gamma, b"input", ptr, ch * 4, capi.F16) == capi.INVALID_PARAMS
+        w_bytes = ch * 3 * 3 * ch * 2
+        assert bind(h, first["op_id"], b"weight", ptr, w_bytes, capi.F16) == capi.SUCCESS
+        assert bind(h, second["op_id"], b"weight_rsck", ptr, w_bytes, capi.F16) == capi.SUCCESS
+        assert bind(h, first["op_id"], b"weight", ptr, w_bytes - 2, capi.F16) == capi.INVALID_PARAMS
+        assert bind(h, first["op_id"], b"weight", ptr, w_bytes, capi.F32) == capi.INVALID_PARAMS
+        assert bind(h, 12345, b"weight", ptr, w_bytes, capi.F16) == capi.INVALID_PARAMS   # no such step
+    finally:
+        capi.lib().tracea_plan_destroy(h)
+
+
 def test_dtype_and_null_arguments():
     g = {"operators": [G.input_node(1, "x"), G.relu_node(2, "a", 8)], "dependencies": [[1, 2]]}
     with pytest.raises(ValueError, match="f16 or bf16"):

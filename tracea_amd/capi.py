@@ -105,6 +105,7 @@ SIGNATURES = {
     "tracea_plan_describe": (C.c_void_p, [C.c_void_p]),
     "tracea_plan_output": (C.c_int, [C.c_void_p, C.c_uint64, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
     "tracea_plan_bind": (C.c_int, [C.c_void_p, C.c_uint64, C.c_char_p, C.c_void_p]),
+    "tracea_plan_bind_sized": (C.c_int, [C.c_void_p, C.c_uint64, C.c_char_p, C.c_void_p, C.c_size_t, C.c_int32]),
     "tracea_plan_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p]),
     "tracea_apply_epilogue": (C.c_int, [TensorView, C.POINTER(TensorView), C.POINTER(EpilogueOp), C.c_uint32,
                                         C.c_void_p]),

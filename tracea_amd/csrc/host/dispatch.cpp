@@ -1733,6 +1733,10 @@ TraceaStatus run_conv_transpose(const ConvTransposePlan &plan, const EpilogueCha
   const long long J = plan.fm.columns;
   DeviceScope scope(out.device);
   if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  // tracea_last_variant afterwards names what THIS call launched: a convolution variant (by phase) or a
+  // GEMM variant (partial products), the other one reads -1
+  t_last_contraction = -1;
+  t_last_conv = -1;
   if (g_conv_transpose_by_phase.load() && conv_transpose_by_phase_ok(plan))
     return run_conv_transpose_by_phase(plan, chain, stream);
   // Images per pass: the partial products of a pass stay below 512 MiB, the GEMM

@@ -276,6 +276,26 @@ bool ExecutionPlan::compile(const Json &graph, int dtype, std::string *err) {
       *err = st.kind + " '" + st.name + "' reads " + std::to_string(reads) + " elements, its producer writes " + std::to_string(in0.elems);
       return false;
     }
+    // what this node reads from Input nodes, for bind_sized: data in the plan's type, BatchNorm
+    // parameters as float32 channel vectors (gamma, beta, mean, var, in that order: the order of a
+    // BatchNorm node's dependency list after its data input, and of the ids of a fused BatchNorm)
+    auto needs = [&](Id id, long long elems, int dt) {
+      PlanTensor &p = tensors_[id];
+      if (!p.external || elems <= 0) return;
+      const long long bytes = elems * (long long)elem_bytes(dt);
+      if (bytes > p.need_bytes) p.need_bytes = bytes;
+      p.need_dtype = dt;
+    };
+    needs(st.inputs[0], reads, dtype_);
+    if (st.kind == "Elementwise") needs(st.inputs[1], out.elems, dtype_);
+    if (st.kind == "Attention") { needs(st.inputs[1], out.elems, dtype_); needs(st.inputs[2], out.elems, dtype_); }
+    if (st.kind == "BatchNorm")
+      for (int i = 1; i < 5; ++i) needs(st.inputs[i], out.channels, TRACEA_DTYPE_FLOAT32);
+    for (const PlanEpilogue &pe : st.epilogue) {
+      if (pe.kind == TRACEA_EPI_OP_BATCHNORM)
+        for (int i = 0; i < pe.n_ids; ++i) needs(pe.ids[i], out.channels, TRACEA_DTYPE_FLOAT32);
+      if (pe.kind == TRACEA_EPI_OP_RESIDUAL_ADD) needs(pe.ids[0], out.elems, dtype_);
+    }
   }
 
   // ---- steps, liveness, arena ----
@@ -382,6 +402,34 @@ TraceaStatus ExecutionPlan::bind(uint64_t op_id, const std::string &slot, void *
       return TRACEA_SUCCESS;
     }
   return fail(TRACEA_INVALID_PARAMS, "tracea_plan_bind: no step with op_id %llu", (unsigned long long)op_id);
+}
+
+TraceaStatus ExecutionPlan::bind_sized(uint64_t op_id, const std::string &slot, void *ptr, size_t bytes, int dtype) {
+  if (slot == "input") {
+    auto it = tensors_.find(op_id);
+    if (it != tensors_.end() && it->second.external) {
+      const PlanTensor &t = it->second;
+      if (t.need_bytes > 0 && (long long)bytes < t.need_bytes)
+        return fail(TRACEA_INVALID_PARAMS, "tracea_plan_bind: the tensor bound to input %llu holds %zu bytes, the plan reads %lld",
+                    (unsigned long long)op_id, bytes, t.need_bytes);
+      if (t.need_dtype >= 0 && dtype >= 0 && dtype != t.need_dtype)
+        return fail(TRACEA_INVALID_PARAMS, "tracea_plan_bind: the tensor bound to input %llu has element type %d, the plan reads it as %d",
+                    (unsigned long long)op_id, dtype, t.need_dtype);
+    }
+  } else {
+    for (const PlanStep &st : steps_)
+      if (st.id == op_id && (st.kind == "Conv2d" || st.kind == "Gemm" || st.kind == "Linear")) {
+        const long long elems = st.kind == "Conv2d" ? st.g[4] * st.g[5] * st.g[6] * st.g[1] : st.g[2] * st.g[1];
+        const long long need = elems * (long long)elem_bytes(dtype_);
+        if ((long long)bytes < need)
+          return fail(TRACEA_INVALID_PARAMS, "tracea_plan_bind: the weights bound to %s '%s' hold %zu bytes, the node reads %lld",
+                      st.kind.c_str(), st.name.c_str(), bytes, need);
+        if (dtype >= 0 && dtype != dtype_)
+          return fail(TRACEA_INVALID_PARAMS, "tracea_plan_bind: the weights bound to %s '%s' have element type %d, the plan computes in %d",
+                      st.kind.c_str(), st.name.c_str(), dtype, dtype_);
+      }
+  }
+  return bind(op_id, slot, ptr);
 }
 
 void *ExecutionPlan::address(uint64_t id, void *arena) const {

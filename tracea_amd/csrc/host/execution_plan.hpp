@@ -28,6 +28,8 @@ struct PlanTensor {
   long long elems = 0;     // 0 for an Input whose size no consumer states
   int channels = 0;        // innermost extent (NHWC channels, GEMM N); 0 if unknown
   size_t offset = 0, bytes = 0;  // place in the arena (256-byte aligned)
+  long long need_bytes = 0;      // an Input node: the most bytes any consumer reads from it (0: unknown)
+  int need_dtype = -1;           // ... and the element type they read it as (-1: unknown)
   int born = -1, last_use = -1;  // step indices; last_use = steps.size() for graph outputs
 };
 
@@ -58,6 +60,9 @@ class ExecutionPlan {
   // slot "input": memory of an Input node; "weight" / "weight_rsck" / "weight_t": the filter
   // bank or right operand of a Conv2d / Linear / Gemm node.
   TraceaStatus bind(uint64_t op_id, const std::string &slot, void *ptr);
+  // The same with the extent and element type (TraceaDType, or -1) of the memory behind `ptr`: refused
+  // when a consumer of the node reads more bytes than that, or reads another type.
+  TraceaStatus bind_sized(uint64_t op_id, const std::string &slot, void *ptr, size_t bytes, int dtype);
   TraceaStatus run(void *arena, int device, void *stream) const;
   bool output(uint64_t op_id, size_t *offset, size_t *bytes) const;
 

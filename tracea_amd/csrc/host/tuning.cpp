@@ -357,6 +357,12 @@ struct GemmBenchmark {
       error = last_error_text();
       return 0.0f;
     }
+    // the dispatcher replaces a variant that cannot run the problem by the nearest one that can: such a
+    // time belongs to that other variant and must not be recorded under this one
+    if (last_variant("gemm") != variant) {
+      error = "the dispatcher ran another variant in its place";
+      return 0.0f;
+    }
     return (float)(2.0 * (double)m * (double)n * (double)k / t * 1e-12);
   }
 };
@@ -403,6 +409,10 @@ struct ConvBenchmark {
     set_forced_variant("conv2d", saved);
     if (t <= 0.0) {
       error = last_error_text();
+      return 0.0f;
+    }
+    if (last_variant("conv2d") != variant) {  // (as for the GEMM: a substitute's time is not this variant's)
+      error = "the dispatcher ran another variant in its place";
       return 0.0f;
     }
     return (float)(2.0 * (double)g.m_gemm * (double)g.n_gemm * (double)g.k_gemm / t * 1e-12);

@@ -72,6 +72,14 @@ TraceaStatus tracea_plan_bind(TraceaPlan *plan, uint64_t op_id, const char *slot
   })
 }
 
+TraceaStatus tracea_plan_bind_sized(TraceaPlan *plan, uint64_t op_id, const char *slot, void *device_ptr,
+                                    size_t bytes, int32_t dtype) {
+  PLAN_GUARDED(TRACEA_UNKNOWN_ERROR, {
+    if (plan == nullptr || slot == nullptr) return fail(TRACEA_INVALID_PARAMS, "tracea_plan_bind: NULL argument");
+    return plan->plan.bind_sized(op_id, slot, device_ptr, bytes, dtype);
+  })
+}
+
 TraceaStatus tracea_plan_run(const TraceaPlan *plan, void *arena, int32_t device, void *stream) {
   PLAN_GUARDED(TRACEA_UNKNOWN_ERROR, {
     if (plan == nullptr) return fail(TRACEA_INVALID_PARAMS, "tracea_plan_run: plan is NULL");

@@ -15,6 +15,7 @@ import torch
 from . import capi
 
 _DT = {torch.float16: capi.F16, torch.bfloat16: capi.BF16}
+_TENSOR_DT = {torch.float16: capi.F16, torch.bfloat16: capi.BF16, torch.float32: capi.F32}
 
 
 class Plan:
@@ -51,7 +52,11 @@ class Plan:
         (slot "weight", "weight_rsck", "weight_t").  The tensor is kept alive by the plan."""
         if not tensor.is_cuda or not tensor.is_contiguous():
             raise ValueError("plan tensors must be contiguous device tensors")
-        capi.check("tracea_plan_bind", capi.lib().tracea_plan_bind(self._h, op_id, slot.encode(), tensor.data_ptr()))
+        # with its extent and element type: a tensor that is too small or of another type than the plan
+        # reads is refused here instead of being read out of bounds by a later run
+        capi.check("tracea_plan_bind", capi.lib().tracea_plan_bind_sized(
+            self._h, op_id, slot.encode(), tensor.data_ptr(), tensor.numel() * tensor.element_size(),
+            _TENSOR_DT.get(tensor.dtype, -1)))
         self._keep[(op_id, slot)] = tensor
         return self
 

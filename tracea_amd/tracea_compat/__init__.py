@@ -94,7 +94,10 @@ class Context:
             raise ValueError("conv_transpose2d: dilation must be 1")
         _ops.conv_transpose2d_ex(x, w, parse_epilogue(epilogue, bias, residual), stride=stride, padding=pad,
                                  output_padding=output_padding, out=o, weight_layout="krsc")
-        return _variant_index("gemm")
+        # the kernel that ran: a convolution variant when the call went out by output phase, else the
+        # GEMM of the partial-product form (an index into the one variant table both operators share)
+        by_phase = _variant_index("conv2d")
+        return by_phase if by_phase >= 0 else _variant_index("gemm")
 
     def attention(self, q, k, v, o, b_in, h_in, s_in, d_in, dh_in, causal=False, scale_sqrt=True, m_tile=None,
                   n_tile=None, stages=None, warps=None, softmax_mode=None, variant=None):
@@ -137,8 +140,14 @@ class TraceaConv2d(torch.nn.Conv2d):
             self._tracea_w = cached
         return cached[1]
 
+    def _needs_grad(self, x):
+        # the kernels here are forward only and their result carries no grad_fn: a training step
+        # must go through PyTorch, or it would silently get no gradients
+        return torch.is_grad_enabled() and (x.requires_grad or self.weight.requires_grad
+                                            or (self.bias is not None and self.bias.requires_grad))
+
     def forward(self, x):
-        if not self._tracea_supported(x):
+        if not self._tracea_supported(x) or self._needs_grad(x):
             return super().forward(x)
         x_nhwc = x.permute(0, 2, 3, 1).contiguous()  # free for a channels_last tensor
         bias = self.bias.detach() if self.bias is not None else None
