@@ -86,7 +86,7 @@ def make_workload(name, torch, ops):
         flops = 4.0 * b * h * d * (s * (s + 1) / 2.0 if causal else float(s) * s)
         return ("bf16 FA2 forward B4 H32 S4096 D128 %s" % ("causal" if causal else "dense"),
                 flops, 2.0 * 4 * q.numel(), "bf16", lambda: ops.attention(q, k, v, causal=causal, out=o))
-    if name == "conv_transpose":
+    if name in ("conv_transpose", "conv_transpose_cached"):
         # the reference's VAE decoder layer at batch 8 (src/optimizer/benchmark.rs:572-575); FLOPs are
         # the products that are not structurally zero, 1/stride^2 of the reference's 2*M*N*K count
         n, h, w, cin, cout, r, st, pd = 8, 32, 32, 512, 256, 4, 2, 1
@@ -94,9 +94,15 @@ def make_workload(name, torch, ops):
         wt = (torch.randn(cin, r, r, cout, device=dev, generator=g) * (1.0 / (4 * cin)) ** 0.5).half()
         ho = (h - 1) * st - 2 * pd + r
         y = torch.empty(n, ho, ho, cout, device=dev, dtype=torch.float16)
-        return ("fp16 NHWC transposed conv N8 32x32x512->64x64x256 4x4 s2 p1",
-                2.0 * n * h * w * cin * r * r * cout, 2.0 * (x.numel() + wt.numel() + y.numel()), "f16",
-                lambda: ops.conv_transpose2d(x, wt, stride=st, padding=pd, out=y))
+        from tracea_amd import capi
+        cached = name.endswith("cached")  # the regrouped filter bank kept between calls (constant filters)
+
+        def step():
+            capi.lib().tracea_set_conv_transpose_filter_cache(1 if cached else 0)
+            ops.conv_transpose2d(x, wt, stride=st, padding=pd, out=y)
+            capi.lib().tracea_set_conv_transpose_filter_cache(0)
+        return ("fp16 NHWC transposed conv N8 32x32x512->64x64x256 4x4 s2 p1" + (", filter cache on" if cached else ""),
+                2.0 * n * h * w * cin * r * r * cout, 2.0 * (x.numel() + wt.numel() + y.numel()), "f16", step)
     if name in ("resnet18_b1", "resnet18_b32"):
         # the reference's network benchmark graph (src/bin/network_bench.rs:41-215), fused, compiled into
         # an execution plan and replayed as one HIP graph; random weights, BatchNorm parameters near identity
@@ -334,7 +340,7 @@ def main():
         cpu = cpu_baseline()
         also = {}
         for name in ("gemm", "gemm_nonsquare", "gemm_rowmajor", "gemm_f32", "gemm_f32_4096", "conv", "basic_block", "downsample_block", "attention", "attention_causal",
-                     "conv_transpose", "resnet18_b1", "resnet18_b32", "gemm_tiles_half"):
+                     "conv_transpose", "conv_transpose_cached", "resnet18_b1", "resnet18_b32", "gemm_tiles_half"):
             if name == args.workload:
                 continue
             lab, fl, by, dt, st = make_workload(name, torch, ops)

@@ -306,6 +306,17 @@ void tracea_set_split_k(int32_t enabled);
  * partial products followed by a gather.  The two formulations agree within the tolerance of the
  * operator (fp32 accumulation in a different order). */
 void tracea_set_conv_transpose_by_phase(int32_t enabled);
+/* The by-phase formulation regroups the filter bank at every call (one helper launch).  With the filter
+ * cache on, the regrouped bank of a (device, filter pointer, shape, strides, stride, padding) is built once,
+ * kept in device memory of its own and reused by later calls, which then launch nothing but the phase
+ * convolutions and allocate nothing: for callers whose filters do not change between calls (inference).
+ * Off by default: the library cannot see an in-place update of the filters.  After changing filters in place
+ * call tracea_conv_transpose_filter_cache_clear (also frees the copies; it waits for the device).  At most 64
+ * banks are kept; a miss while the stream is being captured regroups per call as without the cache.  (The
+ * reference's kernel indexes its [C*R*S, K] bank in place, src/emitter/conv_transpose.rs:207-236, and has
+ * no such state.) */
+void tracea_set_conv_transpose_filter_cache(int32_t enabled);
+void tracea_conv_transpose_filter_cache_clear(void);
 int32_t tracea_last_split_k(void);
 
 /* tracea_gemm for callers that cannot allocate device memory: code whose stream is being

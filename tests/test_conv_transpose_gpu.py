@@ -226,3 +226,42 @@ def test_formulation_by_output_phase_against_the_oracle_and_the_other_formulatio
     # the two differ by the order of fp32 additions and one output rounding at most
     ulp = 2.0 ** -7 if dtype == "bf16" else 2.0 ** -10
     assert np.abs(got[1] - got[0]).max() <= ulp * max(1.0, np.abs(ref).max())
+
+
+def test_filter_cache_reuses_the_regrouped_bank_until_it_is_cleared(tracea_gpu):
+    """With the filter cache on, the first call builds the regrouped bank and later calls allocate nothing
+    and give the same bits as without the cache; filters changed in place are seen after a clear."""
+    from tracea_amd import capi
+    n, h, w, c, k, r, s, stride, pad = 2, 16, 16, 32, 24, 4, 4, 2, 1
+    rng = np.random.default_rng(77)
+    x = _dev(round_f16(rng.uniform(-1, 1, (n, h, w, c))), torch.float16)
+    wt = _dev(round_f16(rng.uniform(-0.5, 0.5, (c, r, s, k))), torch.float16)
+    run = lambda: tracea_gpu.conv_transpose2d(x, wt, stride=stride, padding=pad)
+    plain = run().clone()
+    assert capi.last_variant("conv2d") is not None  # the by-phase formulation
+    try:
+        capi.lib().tracea_set_conv_transpose_filter_cache(1)
+        first = run().clone()
+        torch.cuda.synchronize()
+        out = torch.empty_like(first)
+        free0 = torch.cuda.mem_get_info()[0]
+        for _ in range(3):
+            tracea_gpu.conv_transpose2d(x, wt, stride=stride, padding=pad, out=out)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0
+        assert torch.equal(first, plain) and torch.equal(out, plain)
+        # another stride / padding of the same filters is another bank
+        other = tracea_gpu.conv_transpose2d(x, wt, stride=stride, padding=0)
+        capi.lib().tracea_set_conv_transpose_filter_cache(0)
+        assert torch.equal(other, tracea_gpu.conv_transpose2d(x, wt, stride=stride, padding=0))
+        capi.lib().tracea_set_conv_transpose_filter_cache(1)
+        # filters changed in place: the cached bank is the old one until the cache is cleared
+        wt.mul_(2.0)
+        stale = run().clone()
+        assert torch.equal(stale, plain)
+        capi.lib().tracea_conv_transpose_filter_cache_clear()
+        fresh = run()
+        assert torch.allclose(fresh.float(), 2.0 * plain.float(), atol=2e-2, rtol=2e-3) and not torch.equal(fresh, plain)
+    finally:
+        capi.lib().tracea_set_conv_transpose_filter_cache(0)
+        capi.lib().tracea_conv_transpose_filter_cache_clear()

@@ -140,6 +140,8 @@ SIGNATURES = {
                                      C.POINTER(EpilogueOp), C.c_uint32, C.c_void_p]),
     "tracea_set_split_k": (None, [C.c_int32]),
     "tracea_set_conv_transpose_by_phase": (None, [C.c_int32]),
+    "tracea_set_conv_transpose_filter_cache": (None, [C.c_int32]),
+    "tracea_conv_transpose_filter_cache_clear": (None, []),
     "tracea_last_split_k": (C.c_int32, []),
     "tracea_variant_count": (C.c_int32, [C.c_char_p]),
     "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),

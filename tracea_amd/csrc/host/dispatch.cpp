@@ -264,6 +264,37 @@ TraceaStatus hip_status(const char *what, int e) {
 
 void set_split_k_enabled(bool on) { g_split_k_enabled.store(on); }
 void set_conv_transpose_by_phase(bool on) { g_conv_transpose_by_phase.store(on); }
+
+// Regrouped filter banks of the by-phase transposed convolution, kept between calls when the caller
+// has switched the cache on (tracea_set_conv_transpose_filter_cache).
+namespace {
+std::atomic<bool> g_ct_filter_cache{false};
+struct CtFilterKey {
+  int device;
+  const void *w;
+  long long dims[4], strides[4];
+  int dtype, sh, sw, pad_h, pad_w;
+  long long ho, wo;
+  bool operator<(const CtFilterKey &o) const { return memcmp(this, &o, sizeof(*this)) < 0; }
+};
+std::mutex g_ct_filter_mu;
+std::map<CtFilterKey, void *> g_ct_filters;
+}  // namespace
+void set_conv_transpose_filter_cache(bool on) { g_ct_filter_cache.store(on); }
+void conv_transpose_filter_cache_clear() {
+  std::lock_guard<std::mutex> lk(g_ct_filter_mu);
+  if (g_ct_filters.empty()) return;
+  int prev = 0;
+  const bool have_prev = hipGetDevice(&prev) == hipSuccess;
+  for (auto &kv : g_ct_filters) {
+    if (hipSetDevice(kv.first.device) == hipSuccess) {
+      (void)hipDeviceSynchronize();  // a launch that reads the copy may still be in flight
+      (void)hipFree(kv.second);
+    }
+  }
+  g_ct_filters.clear();
+  if (have_prev) (void)hipSetDevice(prev);
+}
 int last_split_k() { return t_last_splits; }
 
 void set_forced_variant(const char *op, int index) {
@@ -1650,14 +1681,49 @@ TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const Ep
   // (no launch of this path splits K, and work on one stream is ordered); a bank beyond its 64 MiB
   // cap, or a first use while the stream is being captured, takes a stream-ordered allocation.
   hipError_t e = hipSuccess;
-  void *filt = splitk_scratch(out.device, stream, (size_t)total * 2 + 256);
-  const bool pooled = filt != nullptr;
-  if (!pooled) {
-    e = hipMallocAsync(&filt, (size_t)total * 2 + 256, stream);
-    if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+  void *filt = nullptr;
+  bool pooled = true, regroup = true;
+  if (g_ct_filter_cache.load()) {
+    // cached copy of this bank: built once (the stream is drained before the copy is published, so that
+    // calls on other streams may read it), then no helper launch and no allocation per call
+    CtFilterKey key;
+    memset(&key, 0, sizeof(key));
+    key.device = out.device; key.w = w.ptr; key.dtype = w.dtype;
+    for (int i = 0; i < 4; ++i) { key.dims[i] = w.shape[i]; key.strides[i] = w.stride[i]; }
+    key.sh = sh; key.sw = sw; key.pad_h = plan.pad_h; key.pad_w = plan.pad_w; key.ho = Ho; key.wo = Wo;
+    std::lock_guard<std::mutex> lk(g_ct_filter_mu);
+    auto it = g_ct_filters.find(key);
+    if (it != g_ct_filters.end()) {
+      filt = it->second;
+      regroup = false;
+    } else {
+      hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+      if (g_ct_filters.size() < 64 && hipStreamIsCapturing(stream, &cap) == hipSuccess && cap == hipStreamCaptureStatusNone &&
+          hipMalloc(&filt, (size_t)total * 2 + 256) == hipSuccess) {
+        f.out = filt;
+        TraceaStatus fs = hip_status("phase filter launch", launch_phase_filters(f, stream));
+        if (fs == TRACEA_SUCCESS && hipStreamSynchronize(stream) != hipSuccess) fs = TRACEA_UNKNOWN_ERROR;
+        if (fs != TRACEA_SUCCESS) {
+          (void)hipFree(filt);
+          return fs == TRACEA_UNKNOWN_ERROR ? fail(TRACEA_UNKNOWN_ERROR, "tracea_conv_transpose2d: regrouping the filters failed") : fs;
+        }
+        g_ct_filters[key] = filt;
+        regroup = false;
+      } else {
+        filt = nullptr;  // (cache full, stream under capture or out of memory: per-call regrouping below)
+      }
+    }
+  }
+  if (filt == nullptr) {
+    filt = splitk_scratch(out.device, stream, (size_t)total * 2 + 256);
+    pooled = filt != nullptr;
+    if (!pooled) {
+      e = hipMallocAsync(&filt, (size_t)total * 2 + 256, stream);
+      if (e != hipSuccess) return hip_status("tracea_conv_transpose2d: workspace allocation", (int)e);
+    }
   }
   f.out = filt;
-  TraceaStatus st = hip_status("phase filter launch", launch_phase_filters(f, stream));
+  TraceaStatus st = regroup ? hip_status("phase filter launch", launch_phase_filters(f, stream)) : TRACEA_SUCCESS;
   const long long x_extent = (long long)N * H * W * C * 2;
   // Phases that are alike but for their padding (even filter extents divided by the stride: the 4x4
   // stride-2 decoder layer) go out as one launch with the phase in blockIdx.z.

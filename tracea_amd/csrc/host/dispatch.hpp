@@ -48,6 +48,8 @@ void set_split_k_enabled(bool on);
 // Transposed convolutions as one stride-1 convolution per output phase where that applies (on by
 // default); off: always the GEMM to partial products followed by the gather.
 void set_conv_transpose_by_phase(bool on);
+void set_conv_transpose_filter_cache(bool on);
+void conv_transpose_filter_cache_clear();
 int last_split_k();
 
 TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorView &b,
