@@ -297,8 +297,20 @@ TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaT
  * scratch buffer the library keeps per (device, stream) (grown on demand up to 64 MiB, never
  * while the stream is being captured, never freed) and a second kernel sums them and applies
  * the operator chain.  On by default; tracea_set_split_k(0) turns it off.
- * tracea_last_split_k: K ranges of the calling thread's latest gemm / conv2d launch (1: not split). */
+ * tracea_last_split_k: K ranges of the calling thread's latest gemm / conv2d launch (1: not split).
+ * Half-precision launches on tiles up to 128x128 that are split at most four ways need no second kernel: every workgroup leaves its partial
+ * product in the scratch buffer and takes a ticket from a per-tile counter (4 bytes per tile, per (device,
+ * stream), zero between launches); the workgroup that draws a tile's last ticket sums the partial products in
+ * K order, applies the operator chain and writes the tile.  Results equal those of the two-kernel form bit for
+ * bit (same order of summation).  tracea_set_split_k_one_launch(0) goes back to two kernels everywhere (the
+ * fp32 GEMM, the larger tiles, finer splits and tracea_gemm_noalloc always use two: with many K ranges the
+ * reduction kernel, which spreads the sum over the device, is faster than one workgroup per tile);
+ * tracea_last_split_k_launches says which
+ * form the calling thread's latest gemm / conv2d launch took (1 or 2).  (The reference has no split along K:
+ * its GEMM grid is one block per output tile, src/emitter/cuda/gemm.rs:92-207.) */
 void tracea_set_split_k(int32_t enabled);
+void tracea_set_split_k_one_launch(int32_t enabled);
+int32_t tracea_last_split_k_launches(void);
 /* tracea_conv_transpose2d runs as one stride-1 convolution per output phase (stride_h * stride_w
  * launches on a regrouped copy of the filter bank, the outputs written in place) when every phase
  * has taps and no negative padding and the input is dense half-precision NHWC with a multiple of 8

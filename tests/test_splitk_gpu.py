@@ -106,6 +106,112 @@ def test_conv_split_matches_oracle(tracea_gpu, split_switch, shape):
         assert_close_scaled(got.float().cpu().numpy(), want, tol_half(r * s * c, "f16"), "%s %s" % (shape, layout))
 
 
+@pytest.fixture
+def launch_switch(split_switch):
+    capi = split_switch
+    capi.lib().tracea_set_split_k_one_launch(1)
+    yield capi
+    capi.lib().tracea_set_split_k_one_launch(1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_one_launch_split_equals_the_two_launch_form_bit_for_bit(tracea_gpu, launch_switch, dtype):
+    """The tile's last workgroup sums the partial products in K order, whoever it is: the result is that of
+    the reduction kernel bit for bit, on repeated calls (the counters are back at zero after each) and for
+    every variant that can take the one-launch form."""
+    capi = launch_switch
+    tdt, rnd = (torch.float16, round_f16) if dtype == "f16" else (torch.bfloat16, round_bf16)
+    one_launch = 0
+    # (two, four and four K ranges on the default variants, a K tail, ragged M and N; the last two are split
+    # more finely and stay with two launches)
+    for (m, n, k) in [(3136, 64, 576), (784, 128, 1152), (512, 512, 1024), (300, 200, 1096), (96, 136, 1096), (49, 512, 4608),
+                      (100, 72, 2056)]:
+        rng = np.random.default_rng(m + n + k)
+        a = _dev(rnd(rng.standard_normal((m, k)) / np.sqrt(k)), tdt)
+        bt = _dev(rnd(rng.standard_normal((n, k))), tdt)
+        bias = _dev((rng.standard_normal(n) * 0.2).astype(np.float32))
+        res = _dev(rnd(rng.standard_normal((m, n))), tdt)
+        ops = [(capi.OP_BIAS_ADD, bias), (capi.OP_RESIDUAL_ADD, res), (capi.OP_RELU,)]
+        for b in (bt.t(), bt.t().contiguous()):
+            capi.lib().tracea_set_split_k_one_launch(0)
+            two = tracea_gpu.gemm_ex(a, b, ops)
+            assert capi.lib().tracea_last_split_k() >= 2 and capi.lib().tracea_last_split_k_launches() == 2
+            capi.lib().tracea_set_split_k_one_launch(1)
+            for rep in range(3):
+                one = tracea_gpu.gemm_ex(a, b, ops)
+                assert capi.lib().tracea_last_split_k() >= 2
+                one_launch += capi.lib().tracea_last_split_k_launches() == 1
+                assert torch.equal(one, two), "(%d, %d, %d) call %d" % (m, n, k, rep)
+    assert one_launch >= 3 * 2 * 3
+
+
+def test_one_launch_split_on_every_variant_that_takes_it(tracea_gpu, launch_switch):
+    capi = launch_switch
+    m, n, k = 96, 136, 1096                                  # 18 K tiles of 64 (the last one 8 wide): at most 4 ranges
+    rng = np.random.default_rng(5)
+    a = _dev(round_f16(rng.standard_normal((m, k)) / np.sqrt(k)), torch.float16)
+    bt = _dev(round_f16(rng.standard_normal((n, k))), torch.float16)
+    names = capi.variants("gemm")
+    took = 0
+    try:
+        for i, nm in enumerate(names):
+            capi.force_variant("gemm", i)
+            for b in (bt.t(), bt.t().contiguous()):
+                capi.lib().tracea_set_split_k_one_launch(0)
+                two = tracea_gpu.gemm(a, b, out_dtype=torch.float32)
+                capi.lib().tracea_set_split_k_one_launch(1)
+                one = tracea_gpu.gemm(a, b, out_dtype=torch.float32)
+                took += capi.lib().tracea_last_split_k_launches() == 1
+                assert torch.equal(one, two), nm
+    finally:
+        capi.force_variant("gemm", -1)
+    assert took >= 6
+
+
+def test_one_launch_conv_split_and_graph_replay(tracea_gpu, launch_switch):
+    """ResNet-18's 28x28x128 stage at batch 1 on a streamed variant (784 pixels, K = 1152, four K ranges): one
+    kernel, the same bits as two, also when the launch is replayed from a HIP graph with other split launches
+    between the replays."""
+    capi = launch_switch
+    rng = np.random.default_rng(11)
+    x = _dev(round_f16(rng.standard_normal((1, 28, 28, 128))), torch.float16)
+    w = _dev(round_f16(rng.standard_normal((128, 3, 3, 128)) * np.sqrt(2.0 / 1152)), torch.float16)
+    bias = _dev((rng.standard_normal(128) * 0.1).astype(np.float32))
+    ops = [(capi.OP_BIAS_ADD, bias), (capi.OP_RELU,)]
+    capi.force_variant("conv2d", "t128x64x64_w4x1_p2")
+    try:
+        _conv_one_and_two_launches(tracea_gpu, capi, x, w, ops)
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
+def _conv_one_and_two_launches(tracea_gpu, capi, x, w, ops):
+    capi.lib().tracea_set_split_k_one_launch(0)
+    two = tracea_gpu.conv2d_ex(x, w, ops, stride=1, padding=1, weight_layout="krsc")
+    assert capi.lib().tracea_last_split_k_launches() == 2
+    capi.lib().tracea_set_split_k_one_launch(1)
+    one = tracea_gpu.conv2d_ex(x, w, ops, stride=1, padding=1, weight_layout="krsc")
+    assert capi.lib().tracea_last_split_k() >= 2 and capi.lib().tracea_last_split_k_launches() == 1
+    assert torch.equal(one, two)
+    out = torch.empty_like(one)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        tracea_gpu.conv2d_ex(x, w, ops, stride=1, padding=1, weight_layout="krsc", out=out)   # buffers of this stream
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):
+        tracea_gpu.conv2d_ex(x, w, ops, stride=1, padding=1, weight_layout="krsc", out=out)
+    a = torch.randn(512, 1024, device="cuda").half()
+    b = torch.randn(1024, 512, device="cuda").half()
+    for rep in range(3):
+        out.zero_()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, two), "replay %d" % rep
+        tracea_gpu.gemm(a, b)                                 # eager work between the replays
+        torch.cuda.synchronize()
+
+
 def test_large_problems_are_not_split(tracea_gpu, split_switch):
     capi = split_switch
     a = torch.randn(2048, 1024, device="cuda").half()

@@ -139,6 +139,8 @@ SIGNATURES = {
     "tracea_gemm_ttg_ex": (C.c_int, [TensorView, TensorView, C.POINTER(TensorView), GemmParams,
                                      C.POINTER(EpilogueOp), C.c_uint32, C.c_void_p]),
     "tracea_set_split_k": (None, [C.c_int32]),
+    "tracea_set_split_k_one_launch": (None, [C.c_int32]),
+    "tracea_last_split_k_launches": (C.c_int32, []),
     "tracea_set_conv_transpose_by_phase": (None, [C.c_int32]),
     "tracea_set_conv_transpose_filter_cache": (None, [C.c_int32]),
     "tracea_conv_transpose_filter_cache_clear": (None, []),

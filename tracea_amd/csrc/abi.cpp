@@ -156,6 +156,8 @@ TraceaStatus tracea_attention(TraceaTensorView q, TraceaTensorView k, TraceaTens
 }
 
 void tracea_set_split_k(int32_t enabled) { set_split_k_enabled(enabled != 0); }
+void tracea_set_split_k_one_launch(int32_t enabled) { set_split_k_one_launch(enabled != 0); }
+int32_t tracea_last_split_k_launches(void) { return last_split_k_launches(); }
 void tracea_set_conv_transpose_by_phase(int32_t enabled) { set_conv_transpose_by_phase(enabled != 0); }
 void tracea_set_conv_transpose_filter_cache(int32_t enabled) { set_conv_transpose_filter_cache(enabled != 0); }
 void tracea_conv_transpose_filter_cache_clear(void) { conv_transpose_filter_cache_clear(); }

@@ -40,6 +40,12 @@ struct ContractionArgs {
   int grid_m, grid_n;  // tiles along M and N
   int k_split;         // 0: one workgroup per tile runs all of K; else the K extent of one split (a multiple
                        // of the variant's BK): grid.y = ceil(K / k_split), C is the [splits][M][ldc] workspace
+  // One-launch split (k_split > 0 and fuse_ws set): C, out_dtype and epi are the call's own; every workgroup
+  // leaves its fp32 partial product, in accumulator order, in block (blockIdx.x*splits + blockIdx.y) of fuse_ws
+  // and takes a ticket from fuse_count[blockIdx.x]; the last one of a tile sums the blocks in split order, runs
+  // the operator chain, writes C and puts the counter back to zero.
+  float *fuse_ws;
+  unsigned *fuse_count;
   int group_m;         // tile-order group height
   // GEMM over a tile list (null: the dense grid_m x grid_n grid): workgroup p of the
   // launch (grid.x = list length) runs record tile_list[p]; a record is 5 words

@@ -575,7 +575,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   int tile_m, tile_n;
   int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
   int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
-  long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
+  // (tiles above 128x128 are never split in one launch: their kernels do not carry that code)
+  constexpr bool FUSE_OK = BM * BN <= 128 * 128;
+  const bool fused = FUSE_OK && args.k_split > 0 && args.fuse_ws != nullptr;
+  long long zrow = args.k_split > 0 && !fused ? (long long)blockIdx.y * M : 0ll;
   if (!CONV && args.tile_list != nullptr) {
     // Tile list (the reference's two-level tile table, src/core/ttg.rs:3-11 and
     // src/emitter/cuda/low_rank.rs:69-76): workgroup p runs record tile_list[p] =
@@ -1189,6 +1192,68 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     __builtin_amdgcn_s_waitcnt(0x0f70);  // clamped repeats must not land on the epilogue staging
   }
   __syncthreads();
+
+  // ---- one-launch split: leave the partial product, take a ticket; the tile's last workgroup sums ----
+  // Every wave's accumulators go out as they lie in registers (block (i, j), group g: one 16-byte piece per
+  // lane, 1 KB per store instruction) and come back the same way, so the layout needs no name.  The K
+  // ranges of a tile may run on different XCDs, whose L2 caches do not see each other's lines.  Device-
+  // scope fences would settle that (write the L2 back, invalidate it) but cost more than the second kernel
+  // they save: several microseconds each, one after the other on an L2.  Instead the partial products
+  // travel with device scope themselves: stores that write through to memory, loads that do not trust a
+  // line of another L2, and a device-scope counter.  Order of events: the workgroup's stores are
+  // acknowledged (vmcnt(0)), barrier, one thread takes the ticket; whoever draws the last ticket of the
+  // tile reads every partial product.  Nobody waits for anybody.  The sum runs over the K ranges in order,
+  // this workgroup's own included, whichever of them comes last: the result does not depend on the
+  // order of arrival and equals that of the two-launch reduction.
+  if constexpr (FUSE_OK) {
+    if (fused) {
+      __shared__ unsigned s_ticket;
+      constexpr int DEVICE_SCOPE = 16;  // the sc1 bit of a buffer instruction
+      const unsigned splits = gridDim.y;
+      constexpr unsigned TILE_BYTES = BM * BN * 4, WAVE_BYTES = TM * TN * 4;
+      __amdgpu_buffer_rsrc_t rsrc_ws = __builtin_amdgcn_make_buffer_rsrc((void *)args.fuse_ws, 0, 0x7fffffff, 0x00020000);
+      const unsigned first = blockIdx.x * splits * TILE_BYTES + wave * WAVE_BYTES + lane * 16;
+      const unsigned mine = first + blockIdx.y * TILE_BYTES;
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_ws, (int)(mine + ((i * FN + j) * 4 + g) * 1024), 0,
+                                                   DEVICE_SCOPE);
+          }
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+      __syncthreads();
+      if (tid == 0) s_ticket = __hip_atomic_fetch_add(args.fuse_count + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();
+      if (s_ticket != splits - 1) return;
+      // (back to zero for the next launch on this stream)
+      if (tid == 0) __hip_atomic_store(args.fuse_count + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+#pragma unroll 2
+      for (unsigned z = 0; z < splits; ++z) {
+        const unsigned src = first + z * TILE_BYTES;
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const f32x4 v = __builtin_bit_cast(
+                  f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_ws, (int)(src + ((i * FN + j) * 4 + g) * 1024), 0, DEVICE_SCOPE));
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] += v[e];
+            }
+      }
+    }
+  }
 
   // ---- epilogue ----
   // The MFMA leaves lane l with row (l&31) and channels 8g + 4*(l>>5) + 0..3 of

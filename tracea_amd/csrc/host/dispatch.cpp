@@ -249,11 +249,13 @@ std::atomic<int> g_forced_contraction{-1};
 std::atomic<int> g_forced_conv{-1};
 std::atomic<int> g_forced_attention{-1};
 std::atomic<bool> g_split_k_enabled{true};
+std::atomic<bool> g_split_k_one_launch{true};
 std::atomic<bool> g_conv_transpose_by_phase{true};
 // variant the calling thread's latest launch of each operator used (-1: none,
 // or a kernel outside the variant tables)
 thread_local int t_last_contraction = -1, t_last_conv = -1, t_last_attention = -1;
 thread_local int t_last_splits = 1;  // K ranges of the calling thread's latest gemm / conv2d launch
+thread_local int t_last_split_launches = 1;  // kernels that launch took: 2 when a reduction kernel followed
 
 TraceaStatus hip_status(const char *what, int e) {
   if (e == 0) return TRACEA_SUCCESS;
@@ -263,6 +265,8 @@ TraceaStatus hip_status(const char *what, int e) {
 }  // namespace
 
 void set_split_k_enabled(bool on) { g_split_k_enabled.store(on); }
+void set_split_k_one_launch(bool on) { g_split_k_one_launch.store(on); }
+int last_split_k_launches() { return t_last_split_launches; }
 void set_conv_transpose_by_phase(bool on) { g_conv_transpose_by_phase.store(on); }
 
 // Regrouped filter banks of the by-phase transposed convolution, kept between calls when the caller
@@ -412,6 +416,8 @@ namespace {
 // convolution geometry (plan_conv_patch / plan_conv_filter_resident), never split K and run no GEMM.
 inline bool conv_only(const ContractionVariant &v) { return v.pipeline >= 4; }
 
+constexpr int kOneLaunchMaxSplits = 4;  // finest split that runs as one launch (see launch_maybe_split)
+
 int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split, int min_tiles = 4) {
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
@@ -473,7 +479,9 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
       if (waves < 8.0) prior *= std::sqrt(std::sqrt(waves / 8.0));
     }
     double cost = rounds * (double)v.bm * (double)v.bn * k_per / (slot_rate * prior);
-    if (splits > 1) cost += 4.0 + (double)splits * m * n * 4.0 / 3.0e6;
+    // (a coarse split on a tile up to 128x128 runs as one launch, see launch_maybe_split: about a microsecond less)
+    const bool one_launch = splits <= kOneLaunchMaxSplits && v.bm * v.bn <= 128 * 128 && g_split_k_one_launch.load();
+    if (splits > 1) cost += (one_launch ? 3.0 : 4.0) + (double)splits * m * n * 4.0 / 3.0e6;
     if (best < 0 || cost < best_cost) {
       best_cost = cost;
       best = i;
@@ -569,6 +577,29 @@ void *splitk_scratch(int device, hipStream_t stream, size_t bytes) {
   return p;
 }
 
+// Ticket counters of the one-launch split, one per tile, kept per (device, stream) like the scratch
+// buffer: zero when allocated, and every launch leaves them at zero again.  Null while the stream is
+// being captured and the counters do not exist yet.
+constexpr int kFuseTiles = 16384;
+std::map<std::pair<int, void *>, unsigned *> g_fuse_counters;
+unsigned *fuse_counters(int device, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  auto &slot = g_fuse_counters[{device, (void *)stream}];
+  if (slot != nullptr) return slot;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  void *p = nullptr;
+  if (hipMalloc(&p, kFuseTiles * sizeof(unsigned)) != hipSuccess || hipMemset(p, 0, kFuseTiles * sizeof(unsigned)) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  slot = (unsigned *)p;
+  return slot;
+}
+
 // Launches `args` on variant v, split along K when that pays; `chain` is the operator chain
 // of the call (args.epi is ignored).
 // The workspace of a launch split `splits` ways: the per-stream buffer (null when it cannot be had:
@@ -597,6 +628,28 @@ TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, C
                                 hipStream_t stream, bool static_only = false) {
   int k_split = 0;
   const int splits = g_split_k_enabled.load() ? choose_split(v, args.M, args.N, args.K, &k_split) : 1;
+  t_last_split_launches = 1;
+  // One launch: the tile's last workgroup sums the partial products and runs the chain (tiles up to
+  // 128x128: the larger kernels do not carry the code; never for the entry point that must not allocate).
+  // Up to kOneLaunchMaxSplits K ranges only: one workgroup reads all of a tile's partial products through
+  // one CU, where the reduction kernel spreads them over the device.  Measured, 20 launches in a graph:
+  // 2 ranges 6.6 us against 7.6, 4 ranges 7.2-7.8 against 8.0-9.3, 9 ranges 8.9 against 7.7, 18 ranges
+  // 12.8 against 8.5.
+  const long long tiles = (long long)args.grid_m * args.grid_n;
+  if (splits > 1 && splits <= kOneLaunchMaxSplits && g_split_k_one_launch.load() && !static_only && v.bm * v.bn <= 128 * 128 && args.phases <= 1 &&
+      args.out_map == 0 && args.tile_list == nullptr && tiles <= kFuseTiles) {
+    const size_t bytes = (size_t)tiles * (size_t)splits * (size_t)(v.bm * v.bn) * 4;
+    void *fws = splitk_scratch(device, stream, bytes);
+    unsigned *cnt = fws != nullptr ? fuse_counters(device, stream) : nullptr;
+    if (cnt != nullptr) {
+      args.epi = chain;
+      args.k_split = k_split;
+      args.fuse_ws = (float *)fws;
+      args.fuse_count = cnt;
+      t_last_splits = splits;
+      return hip_status(what, v.launch(args, conv, dtype, b_ncontig, stream));
+    }
+  }
   TraceaStatus ws = TRACEA_SUCCESS;
   void *scratch = split_workspace(what, static_only, device, stream, splits, args.M, args.N, &ws);
   if (ws != TRACEA_SUCCESS) return ws;
@@ -618,6 +671,7 @@ TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, C
   args.k_split = k_split;
   TraceaStatus st = hip_status(what, v.launch(args, conv, dtype, b_ncontig, stream));
   if (st != TRACEA_SUCCESS) return st;
+  t_last_split_launches = 2;
   return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
 }
 

@@ -45,6 +45,8 @@ int last_variant(const char *op);
 // Split-K of launches with few output tiles and a long K (on by default), and the number of
 // K ranges the calling thread's latest gemm / conv2d launch was split into (1: not split).
 void set_split_k_enabled(bool on);
+void set_split_k_one_launch(bool on);  // default on: the tile's last workgroup reduces, no second kernel
+int last_split_k_launches();            // 1 or 2: kernels the calling thread's latest gemm / conv2d launch took
 // Transposed convolutions as one stride-1 convolution per output phase where that applies (on by
 // default); off: always the GEMM to partial products followed by the gather.
 void set_conv_transpose_by_phase(bool on);
