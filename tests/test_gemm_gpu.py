@@ -66,7 +66,7 @@ def test_reference_known_answer_16cubed_f16(tracea_gpu):
 HALF_SHAPES = [(256, 256, 128), (300, 200, 136), (512, 384, 1024), (64, 72, 8), (1000, 24, 72)]
 
 
-@pytest.mark.parametrize("variant", range(24))
+@pytest.mark.parametrize("variant", range(32))
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_half_every_variant_both_b_layouts(tracea_gpu, variant, dtype):
     from tracea_amd import capi
@@ -88,6 +88,43 @@ def test_half_every_variant_both_b_layouts(tracea_gpu, variant, dtype):
             assert_close_scaled(c2, ref, tol_half(k, dtype), "%s %s NN %s" % (names[variant], dtype, (m, n, k)))
     finally:
         capi.force_variant("gemm", -1)
+
+
+def test_members_on_16x16x32_mfmas_run_themselves_or_their_twin(tracea_gpu):
+    """The MFMA shape is an axis of the family: the _m16 members multiply with v_mfma_f32_16x16x32 and give
+    the same bits as their 32x32x16 twins (same K order of the partial sums inside a K tile is not
+    promised, so the bar is the operator's tolerance; in practice the results are equal).  A call they
+    cannot take (N-contiguous B) runs on the twin."""
+    from tracea_amd import capi
+    names = capi.variants("gemm")
+    m16 = [nm for nm in names if nm.endswith("_m16")]
+    assert len(m16) >= 3
+    rng = np.random.default_rng(16)
+    m, n, k = 520, 392, 1088                                   # ragged M and N, 17 K tiles
+    a = round_f16(rng.standard_normal((m, k)) / np.sqrt(k))
+    bt = round_f16(rng.standard_normal((n, k)))
+    ref = oracle.gemm_f64(a, bt.T)
+    da, dbt = _dev(a, torch.float16), _dev(bt, torch.float16)
+    try:
+        for nm in m16:
+            twin = nm[: -len("_m16")]
+            assert twin in names
+            capi.force_variant("gemm", nm)
+            c = tracea_gpu.gemm(da, dbt.t())
+            assert capi.last_variant("gemm") == nm
+            assert_close_scaled(c.float().cpu().numpy(), ref, tol_half(k, "f16"), nm)
+            c_n = tracea_gpu.gemm(da, dbt.t().contiguous())
+            assert capi.last_variant("gemm") == twin
+            capi.force_variant("gemm", twin)
+            c_t = tracea_gpu.gemm(da, dbt.t())
+            assert_close_scaled(c.float().cpu().numpy(), c_t.float().cpu().numpy(), 2.0 ** -10, nm + " vs twin")
+            assert torch.equal(c_n, tracea_gpu.gemm(da, dbt.t().contiguous()))
+    finally:
+        capi.force_variant("gemm", -1)
+    # the default for a large product with a K-contiguous B is a 16x16x32 member
+    big = torch.randn(4096, 512, device="cuda").half()
+    tracea_gpu.gemm(big, torch.randn(4096, 512, device="cuda").half().t())
+    assert capi.last_variant("gemm").endswith("_m16")
 
 
 def test_epilogue_kinds_match_oracle_chain(tracea_gpu):

@@ -112,11 +112,13 @@ struct ContractionVariant {
                  //    and fetched with transposing LDS reads);
                  // 3: ring of `stages` LDS buffers, direct-to-LDS loads stages-1 tiles ahead
                  // 4: convolution only: input patch resident in LDS, filter tiles through a ring of `stages`
+                 // (the build's mode 6 is pipeline 2 with mfma = 16)
                  // 5: convolution only: input patch and filter bank both resident in LDS
                  //    (conv_resident_kernel.hpp); bm = most pixels per workgroup, K = 16 * stages exactly
   size_t lds_bytes;
   // launch: returns hipError_t as int
   int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);
+  int mfma;  // MFMA shape of the half-precision kernels: 32 (32x32x16) or 16 (16x16x32: GEMM on pipeline 2, K-contiguous B only)
 };
 
 int contraction_variant_count();

@@ -66,6 +66,24 @@ struct Mfma32<DT_BF16> {
   }
 };
 
+// The 16x16x32 shape: four times the blocks of a quarter the size, 16 cycles each.  A fragment is 16 rows
+// by 32 k (lane l: row l & 15, k = 8 * (l >> 4) .. + 7), the result a column of 4 per lane (lane l: column
+// l & 15 of the second operand, rows 4 * (l >> 4) .. + 3 of the first).
+template <int DT>
+struct Mfma16;
+template <>
+struct Mfma16<DT_F16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma16<DT_BF16> {
+  static __device__ __forceinline__ f32x4 run(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+
 // q = n / d, r = n % d through a precomputed reciprocal: m = ceil(2^(32+s)/d),
 // or m == 0 for a power-of-two d with s = log2(d).  Same arithmetic as the
 // reference's device fast_divmod (src/emitter/cuda/conv.rs:144-151).
@@ -545,8 +563,11 @@ struct Sequenced {
 };
 
 // ---- the kernel -----------------------------------------------------------------
-template <int DT, int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, bool CONV, bool B_NCONTIG>
+// MS: the MFMA shape, 32 (v_mfma_f32_32x32x16) or 16 (v_mfma_f32_16x16x32; GEMM on pipeline 2 with a K-contiguous B only).
+template <int DT, int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, int MS, bool CONV, bool B_NCONTIG>
 __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const ContractionArgs args) {
+  static_assert(MS == 32 || (MS == 16 && PIPE == 2 && !CONV && !B_NCONTIG && BK % 32 == 0),
+                "the 16x16x32 form exists for a GEMM on pipeline 2 with a K-contiguous B");
   constexpr int NT = WM * WN * 64;
   constexpr int CH = BK / 8;       // 16-byte pieces per tile row
   constexpr int ROW_BYTES = BK * 2;
@@ -576,8 +597,9 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
   int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
   // (tiles above 128x128 are never split in one launch: their kernels do not carry that code)
-  constexpr bool FUSE_OK = BM * BN <= 128 * 128;
+  constexpr bool FUSE_OK = BM * BN <= 128 * 128 && MS == 32;
   const bool fused = FUSE_OK && args.k_split > 0 && args.fuse_ws != nullptr;
+  if (!FUSE_OK && args.k_split > 0 && args.fuse_ws != nullptr) return;  // (a launch the dispatcher never makes: C is not a workspace)
   long long zrow = args.k_split > 0 && !fused ? (long long)blockIdx.y * M : 0ll;
   if (!CONV && args.tile_list != nullptr) {
     // Tile list (the reference's two-level tile table, src/core/ttg.rs:3-11 and
@@ -908,6 +930,14 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     for (int j = 0; j < FN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+  // (MS == 16: 16x16 blocks, block (i, j) = rows 16 i .., channels 16 j .. of the wave tile; the other set is unused)
+  f32x4 acc16[MS == 16 ? 2 * FM : 1][MS == 16 ? 2 * FN : 1];
+#pragma unroll
+  for (int i = 0; i < (MS == 16 ? 2 * FM : 1); ++i)
+#pragma unroll
+    for (int j = 0; j < (MS == 16 ? 2 * FN : 1); ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc16[i][j][e] = 0.0f;
 
   const int lrow = lane & 31;
   const int lhalf = lane >> 5;
@@ -1033,27 +1063,52 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // that frees its buffer, a whole tile of MFMAs before the barrier that
     // publishes it; the only wait on global memory is the one in front of that
     // barrier.
-    constexpr int KS = BK / 16;
+    // A k-step is one MFMA deep: 16 k with 32-row fragments, 32 k with the 16-row fragments of the
+    // 16x16x32 shape (XF fragments per 32 rows; same bytes per fragment, same bytes per K tile).
+    constexpr int KSTEP = MS == 16 ? 32 : 16, XF = MS == 16 ? 2 : 1;
+    constexpr int KS = BK / KSTEP;
     static_assert(KS >= 2 && KS % 2 == 0, "pipelined loop needs an even number of k-steps");
-    constexpr int R = FM * FN, D = FM + (B_NCONTIG ? 2 * FN : FN), L = NA + NB;
-    u32x4 fa[2][FM], fb[2][FN];
+    constexpr int R = XF * FM * XF * FN, D = XF * FM + (B_NCONTIG ? 2 * FN : XF * FN), L = NA + NB;
+    u32x4 fa[2][XF * FM], fb[2][XF * FN];
+    // (16-row fragments: row lane & 15, 16-byte piece 4 ks + (lane >> 4); the piece swizzle has a period
+    // of 16 rows, so every fragment of the wave sees the same one)
+    const int row16 = lane & 15, q16 = lane >> 4;
+    const int swz16 = (row16 / RP) & (CH - 1);
     auto read_operands = [&](int set, const unsigned char *sA, const unsigned char *sB, int ks) {
-      const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
-      const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
-      const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+      if constexpr (MS == 16) {
+        static_assert(16 % (RP * CH) == 0, "the piece swizzle must repeat every 16 rows");
+        const unsigned char *pa = sA + (wm * TM + row16) * ROW_BYTES;
+        const unsigned char *pb = sB + (wn * TN + row16) * ROW_BYTES;
+        const int coff = ((ks * 4 + q16) ^ swz16) << 4;
 #pragma unroll
-      for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
+        for (int i = 0; i < 2 * FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 16 * ROW_BYTES + coff);
 #pragma unroll
-      for (int j = 0; j < FN; ++j) {
-        if constexpr (B_NCONTIG) fb[set][j] = read_b_tr(sB, j, ks);
-        else fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+        for (int j = 0; j < 2 * FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 16 * ROW_BYTES + coff);
+      } else {
+        const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
+        const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
+        const int coff = ((ks * 2 + lhalf) ^ lswz) << 4;
+#pragma unroll
+        for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+          if constexpr (B_NCONTIG) fb[set][j] = read_b_tr(sB, j, ks);
+          else fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
+        }
       }
     };
     auto mma = [&](int set) {
+      if constexpr (MS == 16) {
 #pragma unroll
-      for (int i = 0; i < FM; ++i)
+        for (int i = 0; i < 2 * FM; ++i)
 #pragma unroll
-        for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(fb[set][j], fa[set][i], acc[i][j]);
+          for (int j = 0; j < 2 * FN; ++j) acc16[i][j] = Mfma16<DT>::run(fb[set][j], fa[set][i], acc16[i][j]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+          for (int j = 0; j < FN; ++j) acc[i][j] = Mfma32<DT>::run(fb[set][j], fa[set][i], acc[i][j]);
+      }
     };
     // The L requests of a tile are issued in SPREAD consecutive k-step regions,
     // the first of which is the one right after the barrier that freed the
@@ -1237,7 +1292,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         for (int j = 0; j < FN; ++j)
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
-#pragma unroll 2
+      // (one K range at a time: with two in flight the loads' registers cost the 128x128 tile its second wave per SIMD)
+#pragma unroll 1
       for (unsigned z = 0; z < splits; ++z) {
         const unsigned src = first + z * TILE_BYTES;
 #pragma unroll
@@ -1286,11 +1342,23 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     constexpr int i = decltype(blk)::value;
     static_for<0, FN>([&](auto col) {
       constexpr int j = decltype(col)::value;
+      if constexpr (MS == 16) {
+        // lane: row lane & 15 of each 16x16 block, channels 4 * (lane >> 4) .. + 3
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
-                   acc[i][j][g * 4 + 3]};
-        *(f32x4 *)(stage + lrow * EP_PITCH + j * 32 + g * 8 + lhalf * 4) = v;
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int jj = 0; jj < 2; ++jj) {
+            const f32x4 a4 = acc16[2 * i + h][2 * j + jj];
+            f32x4 v = {a4[0], a4[1], a4[2], a4[3]};
+            *(f32x4 *)(stage + ((lane & 15) + 16 * h) * EP_PITCH + j * 32 + jj * 16 + (lane >> 4) * 4) = v;
+          }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2],
+                     acc[i][j][g * 4 + 3]};
+          *(f32x4 *)(stage + lrow * EP_PITCH + j * 32 + g * 8 + lhalf * 4) = v;
+        }
       }
     });
     // The staging area is private to the wave and a wave's LDS operations
@@ -1347,9 +1415,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   });
 }
 
-template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE>
+template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, int MS = 32>
 int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
                        hipStream_t stream) {
+  if (MS == 16 && (b_ncontig || conv)) return (int)hipErrorInvalidValue;  // (the dispatcher sends such calls to the 32x32x16 twin)
   constexpr size_t lds = (size_t)NS * (BM + BN) * BK * 2;
   const bool listed = !conv && a.tile_list != nullptr;  // one workgroup per record, no split grid
   const dim3 grid((unsigned)(listed ? a.tile_count : a.grid_m * a.grid_n),
@@ -1358,7 +1427,7 @@ int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_nc
       block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \
-    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, NS, PIPE, CONVV, NCV>;                      \
+    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, NS, PIPE, MS, (CONVV) && MS == 32, (NCV) && MS == 32>; \
     static bool attr_done = false;                                                           \
     if (!attr_done) {                                                                        \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                  \

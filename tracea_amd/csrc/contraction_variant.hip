@@ -14,16 +14,19 @@ namespace tracea_amd {
 // Host-side accessor (a function, so that nothing here is emitted for the device).
 const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
   static const ContractionVariant v = {
-      TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT,
+      TRACEA_STR(V_NAME), V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, (V_DIRECT == 6 ? 2 : V_DIRECT),
 #if V_DIRECT == 4
       (size_t)V_STAGES * V_BN * V_BK * 2,  // filter ring only; the patch size depends on the problem
-      &launch_conv_patch<V_BM, V_BN, V_WM, V_WN, V_STAGES>};
+      &launch_conv_patch<V_BM, V_BN, V_WM, V_WN, V_STAGES>, 32};
 #elif V_DIRECT == 5
       (size_t)rs_filter_bytes(V_STAGES) + RS_TABLE_BYTES,  // the patch, sized by the problem, comes on top
-      &launch_conv_resident<V_STAGES, 4>};  // 64 input channels: 4 k-steps per tap
+      &launch_conv_resident<V_STAGES, 4>, 32};  // 64 input channels: 4 k-steps per tap
+#elif V_DIRECT == 6
+      (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
+      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, 2, 16>, 16};  // pipeline 2 on 16x16x32 MFMAs
 #else
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
-      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT>};
+      &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, V_DIRECT>, 32};
 #endif
   return v;
 }

@@ -273,13 +273,15 @@ void set_conv_transpose_by_phase(bool on) { g_conv_transpose_by_phase.store(on);
 // has switched the cache on (tracea_set_conv_transpose_filter_cache).
 namespace {
 std::atomic<bool> g_ct_filter_cache{false};
+// (one array of equal words: a struct of mixed members has padding bytes, which a copy into the map need
+// not preserve and a bytewise comparison would read)
 struct CtFilterKey {
-  int device;
-  const void *w;
-  long long dims[4], strides[4];
-  int dtype, sh, sw, pad_h, pad_w;
-  long long ho, wo;
-  bool operator<(const CtFilterKey &o) const { return memcmp(this, &o, sizeof(*this)) < 0; }
+  long long v[17];  // device, filter pointer, dims[4], strides[4], dtype, stride h/w, padding h/w, output h/w
+  bool operator<(const CtFilterKey &o) const {
+    for (int i = 0; i < 17; ++i)
+      if (v[i] != o.v[i]) return v[i] < o.v[i];
+    return false;
+  }
 };
 std::mutex g_ct_filter_mu;
 std::map<CtFilterKey, void *> g_ct_filters;
@@ -291,7 +293,7 @@ void conv_transpose_filter_cache_clear() {
   int prev = 0;
   const bool have_prev = hipGetDevice(&prev) == hipSuccess;
   for (auto &kv : g_ct_filters) {
-    if (hipSetDevice(kv.first.device) == hipSuccess) {
+    if (hipSetDevice((int)kv.first.v[0]) == hipSuccess) {
       (void)hipDeviceSynchronize();  // a launch that reads the copy may still be in flight
       (void)hipFree(kv.second);
     }
@@ -465,6 +467,11 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
     // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
+    // The same loop on 16x16x32 MFMAs.  Measured against the 32x32x16 twin (replayed graphs, same box):
+    // 256x256 tiles 110.8-112.7 us against 116.1-119.6 at 4096^3 and 210 against 222 at 8192x2048x8192;
+    // 128x128 tiles 5 % faster at 4096^3, 8 % slower at 2048^3, 27 % slower at 1024^3; 128x64 tiles slower
+    // everywhere.  (Convolutions and calls with an N-contiguous B or operands of 2 GiB run on the twin: resolve_variant.)
+    if (v.mfma == 16) prior *= v.bm * v.bn >= 256 * 256 ? 1.04 : 0.9;
     {
       // A CU with fewer than 8 resident waves (one 4-wave workgroup, the launch too small or
       // the tile's LDS too large for a second) hides less latency.  The fourth root is fitted
@@ -480,7 +487,7 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
     }
     double cost = rounds * (double)v.bm * (double)v.bn * k_per / (slot_rate * prior);
     // (a coarse split on a tile up to 128x128 runs as one launch, see launch_maybe_split: about a microsecond less)
-    const bool one_launch = splits <= kOneLaunchMaxSplits && v.bm * v.bn <= 128 * 128 && g_split_k_one_launch.load();
+    const bool one_launch = splits <= kOneLaunchMaxSplits && v.bm * v.bn <= 128 * 128 && v.mfma == 32 && g_split_k_one_launch.load();
     if (splits > 1) cost += (one_launch ? 3.0 : 4.0) + (double)splits * m * n * 4.0 / 3.0e6;
     if (best < 0 || cost < best_cost) {
       best_cost = cost;
@@ -500,12 +507,12 @@ int pick_contraction(const char *op, const std::string &cache_key, int m, int n,
   return select_contraction_variant(m, n, k, conv);
 }
 
-// The variant with the same tile shape and the given pipeline mode, or -1.
+// The variant (on 32x32x16 MFMAs) with the same tile shape and the given pipeline mode, or -1.
 int twin(int vi, int pipeline) {
   const ContractionVariant &p = contraction_variant(vi);
   for (int i = 0; i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
-    if (v.pipeline == pipeline && v.bm == p.bm && v.bn == p.bn && v.bk == p.bk &&
+    if (v.pipeline == pipeline && v.mfma == 32 && v.bm == p.bm && v.bn == p.bn && v.bk == p.bk &&
         v.waves_m == p.waves_m && v.waves_n == p.waves_n)
       return i;
   }
@@ -515,8 +522,14 @@ int twin(int vi, int pipeline) {
 // Replaces a variant that cannot run the problem by the nearest one that can:
 // direct-to-LDS loads (pipelines 2 and 3) address operands with 32-bit byte
 // offsets, so operands of 2 GiB and more go through registers (`staged`); the
-// register-staged pipelined loop (pipeline 1) has no K-tail masking for a GEMM.
-int resolve_variant(int vi, bool conv, bool staged, bool k_exact) {
+// register-staged pipelined loop (pipeline 1) has no K-tail masking for a GEMM; the members on 16x16x32
+// MFMAs exist for a GEMM on pipeline 2 with a K-contiguous B.
+int resolve_variant(int vi, bool conv, bool staged, bool k_exact, bool b_ncontig) {
+  if (contraction_variant(vi).mfma == 16 && (conv || b_ncontig || staged)) {
+    const int t = twin(vi, 2);
+    if (t >= 0) vi = t;
+    else return select_contraction_variant(1024, 1024, 1024, conv);  // (every such member has a twin; not reached)
+  }
   int pipe = contraction_variant(vi).pipeline;
   if (pipe >= 4) pipe = 2;  // a convolution-only kernel asked for a GEMM: same tile with streamed operands, if any
   if (pipe >= 2 && staged) pipe = 1;
@@ -636,7 +649,7 @@ TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, C
   // 2 ranges 6.6 us against 7.6, 4 ranges 7.2-7.8 against 8.0-9.3, 9 ranges 8.9 against 7.7, 18 ranges
   // 12.8 against 8.5.
   const long long tiles = (long long)args.grid_m * args.grid_n;
-  if (splits > 1 && splits <= kOneLaunchMaxSplits && g_split_k_one_launch.load() && !static_only && v.bm * v.bn <= 128 * 128 && args.phases <= 1 &&
+  if (splits > 1 && splits <= kOneLaunchMaxSplits && g_split_k_one_launch.load() && !static_only && v.bm * v.bn <= 128 * 128 && v.mfma == 32 && args.phases <= 1 &&
       args.out_map == 0 && args.tile_list == nullptr && tiles <= kFuseTiles) {
     const size_t bytes = (size_t)tiles * (size_t)splits * (size_t)(v.bm * v.bn) * 4;
     void *fws = splitk_scratch(device, stream, bytes);
@@ -706,7 +719,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       const long long a_extent = ((M - 1) * a.stride[0] + K) * 2;
       const long long b_extent = b_kcontig ? ((N - 1) * b.stride[1] + K) * 2 : ((K - 1) * b.stride[0] + N) * 2;
       const bool small = a_extent < (1ll << 31) && b_extent < (1ll << 31);
-      vi = resolve_variant(vi, false, !small, K % contraction_variant(vi).bk == 0);
+      vi = resolve_variant(vi, false, !small, K % contraction_variant(vi).bk == 0, !b_kcontig);
       const ContractionVariant &v = contraction_variant(vi);
       args.a_bytes = (unsigned)(small ? a_extent : 0);
       args.b_bytes = (unsigned)(small ? b_extent : 0);
@@ -735,8 +748,8 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     // finishes first is taken.  Measured, 128 / 64, in us: 1024^3 32.5 / 27.0, 1536^3 104 / 79,
     // 2304x2048x512 70 / 49, 3072^3 539 / 454, 2048^3 138 / 135, 4096^3 972 / 1027.
     // Both split along K by the rule of the half kernels.
-    static const ContractionVariant f32_tile128 = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr};
-    static const ContractionVariant f32_tile64 = {"f32_64x64x16", 64, 64, 16, 2, 2, 1, 0, 0, nullptr};
+    static const ContractionVariant f32_tile128 = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr, 32};
+    static const ContractionVariant f32_tile64 = {"f32_64x64x16", 64, 64, 16, 2, 2, 1, 0, 0, nullptr, 32};
     const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
     const long long ncu = device_limits().cus;
     const int tile = args.a_bytes != 0 && (double)((tiles64 + ncu - 1) / ncu) * 1.06 < (double)((tiles128 + ncu - 1) / ncu) * 4.0 ? 64 : 128;
@@ -889,7 +902,7 @@ TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &ta, const TraceaTensorV
   const bool use_forced = vi >= 0;
   for (int i = 0; !use_forced && i < contraction_variant_count(); ++i) {
     const ContractionVariant &v = contraction_variant(i);
-    if (conv_only(v) || v.bm != (int)layout.mt || v.bn != (int)layout.nt) continue;
+    if (conv_only(v) || v.mfma != 32 || v.bm != (int)layout.mt || v.bn != (int)layout.nt) continue;
     if (vi < 0) { vi = i; continue; }
     const ContractionVariant &best = contraction_variant(vi);
     const int r = rank_of_pipeline[v.pipeline], rb = rank_of_pipeline[best.pipeline];
@@ -898,7 +911,7 @@ TraceaStatus dispatch_gemm_tiles(const TraceaTensorView &ta, const TraceaTensorV
   if (vi < 0)
     return fail(TRACEA_UNSUPPORTED_CONFIG, "%s: no kernel with a %ux%u macro-tile (compiled: 64x64, 128x64, 128x128, "
                 "256x64, 256x128, 256x256)", what, layout.mt, layout.nt);
-  vi = resolve_variant(vi, false, !small, tables.k_gcd % contraction_variant(vi).bk == 0);
+  vi = resolve_variant(vi, false, !small, tables.k_gcd % contraction_variant(vi).bk == 0, !b_kcontig);
   const ContractionVariant &v = contraction_variant(vi);
 
   DeviceScope scope(c.device);
@@ -1505,7 +1518,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
     vi = select_contraction_variant(a.M, a.N, a.K, true);
     if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
   }
-  vi = resolve_variant(vi, true, !small, true);
+  vi = resolve_variant(vi, true, !small, true, plan.w_ncontig);
   const ContractionVariant &v = contraction_variant(vi);
   a.a_bytes = (unsigned)(small ? x_extent : 0);
   a.b_bytes = (unsigned)(small ? w_extent : 0);
@@ -1741,10 +1754,9 @@ TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const Ep
     // cached copy of this bank: built once (the stream is drained before the copy is published, so that
     // calls on other streams may read it), then no helper launch and no allocation per call
     CtFilterKey key;
-    memset(&key, 0, sizeof(key));
-    key.device = out.device; key.w = w.ptr; key.dtype = w.dtype;
-    for (int i = 0; i < 4; ++i) { key.dims[i] = w.shape[i]; key.strides[i] = w.stride[i]; }
-    key.sh = sh; key.sw = sw; key.pad_h = plan.pad_h; key.pad_w = plan.pad_w; key.ho = Ho; key.wo = Wo;
+    key.v[0] = out.device; key.v[1] = (long long)(uintptr_t)w.ptr; key.v[10] = w.dtype;
+    for (int i = 0; i < 4; ++i) { key.v[2 + i] = w.shape[i]; key.v[6 + i] = w.stride[i]; }
+    key.v[11] = sh; key.v[12] = sw; key.v[13] = plan.pad_h; key.v[14] = plan.pad_w; key.v[15] = Ho; key.v[16] = Wo;
     std::lock_guard<std::mutex> lk(g_ct_filter_mu);
     auto it = g_ct_filters.find(key);
     if (it != g_ct_filters.end()) {
@@ -1831,7 +1843,7 @@ TraceaStatus run_conv_transpose_by_phase(const ConvTransposePlan &plan, const Ep
       if (vi < 0) { st = fail(TRACEA_UNKNOWN_ERROR, "tracea_conv_transpose2d: no kernel variant available"); break; }
       const long long w_extent = (long long)K * kg * 2;
       const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
-      vi = resolve_variant(vi, true, !small, true);
+      vi = resolve_variant(vi, true, !small, true, false);
       const ContractionVariant &v = contraction_variant(vi);
       c.a_bytes = (unsigned)(small ? x_extent : 0);
       c.b_bytes = (unsigned)(small ? w_extent : 0);

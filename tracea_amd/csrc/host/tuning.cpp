@@ -201,10 +201,9 @@ PipelineConfig config_for_contraction_variant(int index) {
   c.force_num_warps = (uint32_t)(v.waves_m * v.waves_n);
   c.micro_m = (uint32_t)(v.bm / v.waves_m);
   c.micro_n = (uint32_t)(v.bn / v.waves_n);
-  // every half-precision kernel of the family multiplies with v_mfma_f32_32x32x16 (the 16x16x32 shape
-  // sustained two thirds of its rate in these loops), under the reference's name for a 32x32 MFMA block
-  // (src/core/config.rs:166-181)
-  c.intrinsic_shape = "M32N32K2";
+  // v_mfma_f32_32x32x16 or v_mfma_f32_16x16x32 under the reference's names for a 32x32 and a 16x16 MFMA
+  // block (src/core/config.rs:166-181)
+  c.intrinsic_shape = v.mfma == 16 ? "M16N16K4" : "M32N32K2";
   c.gemm_variant = "Simd";
   c.double_buffer = true;
   c.cp_async_distance = (uint32_t)v.pipeline;  // operand prefetch distance in k-steps
@@ -220,7 +219,7 @@ int contraction_variant_for_config(const PipelineConfig &c) {
     if (c.has_force_num_warps && (uint32_t)(v.waves_m * v.waves_n) != c.force_num_warps) continue;
     if (c.micro_m > 1 && (uint32_t)(v.bm / v.waves_m) != c.micro_m) continue;
     if (c.cp_async_distance != (uint32_t)v.pipeline) continue;
-    if (c.intrinsic_shape == "M16N16K4") continue;  // no member with 16x16 MFMA blocks
+    if ((c.intrinsic_shape == "M16N16K4") != (v.mfma == 16)) continue;
     return i;
   }
   return -1;
