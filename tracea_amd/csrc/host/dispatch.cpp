@@ -468,10 +468,12 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
     // The same loop on 16x16x32 MFMAs.  Measured against the 32x32x16 twin (replayed graphs, same box):
-    // 256x256 tiles 110.8-112.7 us against 116.1-119.6 at 4096^3 and 210 against 222 at 8192x2048x8192;
+    // 256x256 tiles on four waves 104.2-108.7 us, on eight 107.7-110.3, against 116.1-119.6 at 4096^3;
     // 128x128 tiles 5 % faster at 4096^3, 8 % slower at 2048^3, 27 % slower at 1024^3; 128x64 tiles slower
     // everywhere.  (Convolutions and calls with an N-contiguous B or operands of 2 GiB run on the twin: resolve_variant.)
-    if (v.mfma == 16) prior *= v.bm * v.bn >= 256 * 256 ? 1.04 : 0.9;
+    // Four waves against eight on 16x16x32: 781 against 836 us at 8192^3, 198 against 203 at 8192x2048x8192,
+    // 36.3 against 35.0 at 4096x4096x1024 (the four-wave factor also undoes the few-waves penalty below).
+    if (v.mfma == 16) prior *= v.bm * v.bn >= 256 * 256 ? (v.waves_m * v.waves_n == 4 ? (k >= 2048 ? 1.35 : 1.2) : 1.06) : 0.9;
     {
       // A CU with fewer than 8 resident waves (one 4-wave workgroup, the launch too small or
       // the tile's LDS too large for a second) hides less latency.  The fourth root is fitted
@@ -526,7 +528,16 @@ int twin(int vi, int pipeline) {
 // MFMAs exist for a GEMM on pipeline 2 with a K-contiguous B.
 int resolve_variant(int vi, bool conv, bool staged, bool k_exact, bool b_ncontig) {
   if (contraction_variant(vi).mfma == 16 && (conv || b_ncontig || staged)) {
-    const int t = twin(vi, 2);
+    // the member with the same tile on 32x32x16 MFMAs; of several wave layouts the one with the most waves
+    // (with an N-contiguous B, 4096^3: eight waves 117 us, four 131)
+    const ContractionVariant &p = contraction_variant(vi);
+    int t = twin(vi, 2);
+    for (int i = 0; i < contraction_variant_count(); ++i) {
+      const ContractionVariant &v = contraction_variant(i);
+      if (v.pipeline == 2 && v.mfma == 32 && v.bm == p.bm && v.bn == p.bn && v.bk == p.bk &&
+          (t < 0 || v.waves_m * v.waves_n > contraction_variant(t).waves_m * contraction_variant(t).waves_n))
+        t = i;
+    }
     if (t >= 0) vi = t;
     else return select_contraction_variant(1024, 1024, 1024, conv);  // (every such member has a twin; not reached)
   }
