@@ -90,42 +90,39 @@ def test_half_every_variant_both_b_layouts(tracea_gpu, variant, dtype):
         capi.force_variant("gemm", -1)
 
 
-def test_members_on_16x16x32_mfmas_run_themselves_or_their_twin(tracea_gpu):
-    """The MFMA shape is an axis of the family: the _m16 members multiply with v_mfma_f32_16x16x32 and give
-    the same bits as their 32x32x16 twins (same K order of the partial sums inside a K tile is not
-    promised, so the bar is the operator's tolerance; in practice the results are equal).  A call they
-    cannot take (N-contiguous B) runs on the twin."""
+def test_members_on_16x16x32_mfmas(tracea_gpu):
+    """The MFMA shape is an axis of the family: the _m16 members multiply with v_mfma_f32_16x16x32, for both
+    layouts of B, and agree with the oracle and with their 32x32x16 twins (in practice bit for bit)."""
     from tracea_amd import capi
     names = capi.variants("gemm")
     m16 = [nm for nm in names if nm.endswith("_m16")]
     assert len(m16) >= 3
     rng = np.random.default_rng(16)
-    m, n, k = 520, 392, 1088                                   # ragged M and N, 17 K tiles
-    a = round_f16(rng.standard_normal((m, k)) / np.sqrt(k))
-    bt = round_f16(rng.standard_normal((n, k)))
-    ref = oracle.gemm_f64(a, bt.T)
-    da, dbt = _dev(a, torch.float16), _dev(bt, torch.float16)
     try:
-        for nm in m16:
-            twin = nm[: -len("_m16")]
-            assert twin in names
-            capi.force_variant("gemm", nm)
-            c = tracea_gpu.gemm(da, dbt.t())
-            assert capi.last_variant("gemm") == nm
-            assert_close_scaled(c.float().cpu().numpy(), ref, tol_half(k, "f16"), nm)
-            c_n = tracea_gpu.gemm(da, dbt.t().contiguous())
-            ran = capi.last_variant("gemm")                    # same tile on 32x32x16, whatever its wave layout
-            assert not ran.endswith("_m16") and ran.split("_")[0] == nm.split("_")[0]
-            capi.force_variant("gemm", twin)
-            c_t = tracea_gpu.gemm(da, dbt.t())
-            assert_close_scaled(c.float().cpu().numpy(), c_t.float().cpu().numpy(), 2.0 ** -10, nm + " vs twin")
-            capi.force_variant("gemm", ran)
-            assert torch.equal(c_n, tracea_gpu.gemm(da, dbt.t().contiguous()))
+        for (m, n, k) in [(520, 392, 1088), (256, 512, 192), (100, 72, 2048)]:   # ragged M and N, 17 / 3 / 32 K tiles
+            a = round_f16(rng.standard_normal((m, k)) / np.sqrt(k))
+            bt = round_f16(rng.standard_normal((n, k)))
+            ref = oracle.gemm_f64(a, bt.T)
+            da, dbt = _dev(a, torch.float16), _dev(bt, torch.float16)
+            for nm in m16:
+                twin = nm[: -len("_m16")]
+                assert twin in names
+                for b in (dbt.t(), dbt.t().contiguous()):          # K-contiguous and N-contiguous B
+                    capi.force_variant("gemm", nm)
+                    c = tracea_gpu.gemm(da, b)
+                    assert capi.last_variant("gemm") == nm
+                    assert_close_scaled(c.float().cpu().numpy(), ref, tol_half(k, "f16"), "%s %s" % (nm, (m, n, k)))
+                    capi.force_variant("gemm", twin)
+                    c_t = tracea_gpu.gemm(da, b)
+                    assert_close_scaled(c.float().cpu().numpy(), c_t.float().cpu().numpy(), 2.0 ** -10, nm + " vs twin")
     finally:
         capi.force_variant("gemm", -1)
-    # the default for a large product with a K-contiguous B is a 16x16x32 member
+    # the default for a large product is a 16x16x32 member, whichever way B lies
     big = torch.randn(4096, 512, device="cuda").half()
-    tracea_gpu.gemm(big, torch.randn(4096, 512, device="cuda").half().t())
+    wide = torch.randn(4096, 512, device="cuda").half()
+    tracea_gpu.gemm(big, wide.t())
+    assert capi.last_variant("gemm").endswith("_m16")
+    tracea_gpu.gemm(big, wide.t().contiguous())
     assert capi.last_variant("gemm").endswith("_m16")
 
 

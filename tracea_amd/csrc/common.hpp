@@ -118,7 +118,7 @@ struct ContractionVariant {
   size_t lds_bytes;
   // launch: returns hipError_t as int
   int (*launch)(const ContractionArgs &, bool conv, int dtype, bool b_ncontig, hipStream_t);
-  int mfma;  // MFMA shape of the half-precision kernels: 32 (32x32x16) or 16 (16x16x32: GEMM on pipeline 2, K-contiguous B only)
+  int mfma;  // MFMA shape of the half-precision kernels: 32 (32x32x16) or 16 (16x16x32: GEMM on pipeline 2 only)
 };
 
 int contraction_variant_count();

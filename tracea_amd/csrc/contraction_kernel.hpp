@@ -563,11 +563,10 @@ struct Sequenced {
 };
 
 // ---- the kernel -----------------------------------------------------------------
-// MS: the MFMA shape, 32 (v_mfma_f32_32x32x16) or 16 (v_mfma_f32_16x16x32; GEMM on pipeline 2 with a K-contiguous B only).
+// MS: the MFMA shape, 32 (v_mfma_f32_32x32x16) or 16 (v_mfma_f32_16x16x32; GEMM on pipeline 2 only).
 template <int DT, int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, int MS, bool CONV, bool B_NCONTIG>
 __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const ContractionArgs args) {
-  static_assert(MS == 32 || (MS == 16 && PIPE == 2 && !CONV && !B_NCONTIG && BK % 32 == 0),
-                "the 16x16x32 form exists for a GEMM on pipeline 2 with a K-contiguous B");
+  static_assert(MS == 32 || (MS == 16 && PIPE == 2 && !CONV && BK % 32 == 0), "the 16x16x32 form exists for a GEMM on pipeline 2");
   constexpr int NT = WM * WN * 64;
   constexpr int CH = BK / 8;       // 16-byte pieces per tile row
   constexpr int ROW_BYTES = BK * 2;
@@ -682,7 +681,11 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // 16-byte column is XORed with a function of the row so that those four land in the four
   // different 64-byte bank groups.
   constexpr int NB_ROWB = BN * 2, NB_CH = BN / 8;
-  auto nb_swz = [](int krow) -> int { return NB_ROWB >= 256 ? ((krow & 3) << 2) : (((krow >> 1) & 1) << 2); };
+  // (16x16x32: the two 16-lane groups of a half-wave read k rows 8 apart at the same channels; the second
+  // XOR moves one of them to the other 32 bytes of the bank group)
+  auto nb_swz = [](int krow) -> int {
+    return (NB_ROWB >= 256 ? ((krow & 3) << 2) : (((krow >> 1) & 1) << 2)) ^ (MS == 16 ? ((krow >> 3) & 1) << 1 : 0);
+  };
 
   u32x4 ra[NA], rb[NB];
 
@@ -867,6 +870,29 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   }
   auto read_b_tr = [&](const unsigned char *sB, int j, int ks) -> u32x4 {
     const unsigned char *p = sB + tr_off[j] + ks * 16 * NB_ROWB;
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
+    const s16x4 hi =
+        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p + 4 * NB_ROWB));
+    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+    u32x4 v;
+    v[0] = lo2[0]; v[1] = lo2[1]; v[2] = hi2[0]; v[3] = hi2[1];
+    return v;
+  };
+
+  // The same for the 16x16x32 operand (16 channels by 32 k): 16-lane group g takes k 8g .. 8g+7 of the
+  // 32-wide k-step for the block's 16 channels.
+  int tr_off16[B_NCONTIG && MS == 16 ? 2 * FN : 1];
+  if constexpr (B_NCONTIG && MS == 16) {
+    const int r = lane & 15;
+    const int row = (lane >> 4) * 8 + (r >> 2);
+#pragma unroll
+    for (int j = 0; j < 2 * FN; ++j) {
+      const int col = wn * TN + j * 16 + (r & 3) * 4;
+      tr_off16[j] = row * NB_ROWB + (((col >> 3) ^ nb_swz(row)) << 4) + (col & 7) * 2;
+    }
+  }
+  auto read_b_tr16 = [&](const unsigned char *sB, int j, int ks) -> u32x4 {
+    const unsigned char *p = sB + tr_off16[j] + ks * 32 * NB_ROWB;
     const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
     const s16x4 hi =
         __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p + 4 * NB_ROWB));
@@ -1068,7 +1094,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     constexpr int KSTEP = MS == 16 ? 32 : 16, XF = MS == 16 ? 2 : 1;
     constexpr int KS = BK / KSTEP;
     static_assert(KS >= 2 && KS % 2 == 0, "pipelined loop needs an even number of k-steps");
-    constexpr int R = XF * FM * XF * FN, D = XF * FM + (B_NCONTIG ? 2 * FN : XF * FN), L = NA + NB;
+    constexpr int R = XF * FM * XF * FN, D = XF * FM + (B_NCONTIG ? 2 * XF * FN : XF * FN), L = NA + NB;
     u32x4 fa[2][XF * FM], fb[2][XF * FN];
     // (16-row fragments: row lane & 15, 16-byte piece 4 ks + (lane >> 4); the piece swizzle has a period
     // of 16 rows, so every fragment of the wave sees the same one)
@@ -1083,7 +1109,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 #pragma unroll
         for (int i = 0; i < 2 * FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 16 * ROW_BYTES + coff);
 #pragma unroll
-        for (int j = 0; j < 2 * FN; ++j) fb[set][j] = *(const u32x4 *)(pb + j * 16 * ROW_BYTES + coff);
+        for (int j = 0; j < 2 * FN; ++j) {
+          if constexpr (B_NCONTIG) fb[set][j] = read_b_tr16(sB, j, ks);
+          else fb[set][j] = *(const u32x4 *)(pb + j * 16 * ROW_BYTES + coff);
+        }
       } else {
         const unsigned char *pa = sA + (wm * TM + lrow) * ROW_BYTES;
         const unsigned char *pb = sB + (wn * TN + lrow) * ROW_BYTES;
@@ -1438,7 +1467,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
 template <int BM, int BN, int BK, int WM, int WN, int NS, int PIPE, int MS = 32>
 int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig,
                        hipStream_t stream) {
-  if (MS == 16 && (b_ncontig || conv)) return (int)hipErrorInvalidValue;  // (the dispatcher sends such calls to the 32x32x16 twin)
+  if (MS == 16 && conv) return (int)hipErrorInvalidValue;  // (the dispatcher sends convolutions to the 32x32x16 twin)
   constexpr size_t lds = (size_t)NS * (BM + BN) * BK * 2;
   const bool listed = !conv && a.tile_list != nullptr;  // one workgroup per record, no split grid
   const dim3 grid((unsigned)(listed ? a.tile_count : a.grid_m * a.grid_n),
@@ -1447,7 +1476,7 @@ int launch_contraction(const ContractionArgs &a, bool conv, int dtype, bool b_nc
       block(WM * WN * 64);
 #define TRACEA_LAUNCH(DTV, CONVV, NCV)                                                       \
   do {                                                                                       \
-    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, NS, PIPE, MS, (CONVV) && MS == 32, (NCV) && MS == 32>; \
+    auto kfn = contraction_kernel<DTV, BM, BN, BK, WM, WN, NS, PIPE, MS, (CONVV) && MS == 32, NCV>; \
     static bool attr_done = false;                                                           \
     if (!attr_done) {                                                                        \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                  \

@@ -442,7 +442,7 @@ int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split,
 // The slot rate is calibrated on the 4096^3 GEMM (256x256 tiles, one round, 120 us);
 // the estimate then reads 52.8 / 25.9 us for a 3x3 convolution on N32 7x7x512 with
 // unsplit 64x64 tiles / 128x128 tiles split four ways, where 53.7 / 29.6 us were measured.
-int select_contraction_variant(int m, int n, int k, bool conv) {
+int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig) {
   (void)conv;
   const DeviceLimits &dev = device_limits();
   const double cus = (double)dev.cus, slot_rate = dev.slot_rate;  // multiply-accumulates per microsecond and CU at efficiency 1
@@ -470,10 +470,14 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
     // The same loop on 16x16x32 MFMAs.  Measured against the 32x32x16 twin (replayed graphs, same box):
     // 256x256 tiles on four waves 104.2-108.7 us, on eight 107.7-110.3, against 116.1-119.6 at 4096^3;
     // 128x128 tiles 5 % faster at 4096^3, 8 % slower at 2048^3, 27 % slower at 1024^3; 128x64 tiles slower
-    // everywhere.  (Convolutions and calls with an N-contiguous B or operands of 2 GiB run on the twin: resolve_variant.)
+    // everywhere.  (Convolutions and calls with operands of 2 GiB run on the twin: resolve_variant.)
     // Four waves against eight on 16x16x32: 781 against 836 us at 8192^3, 198 against 203 at 8192x2048x8192,
     // 36.3 against 35.0 at 4096x4096x1024 (the four-wave factor also undoes the few-waves penalty below).
     if (v.mfma == 16) prior *= v.bm * v.bn >= 256 * 256 ? (v.waves_m * v.waves_n == 4 ? (k >= 2048 ? 1.35 : 1.2) : 1.06) : 0.9;
+    // An N-contiguous B is fetched with two transposing LDS reads per fragment, and four waves have twice the
+    // B fragments of eight: 4096^3 123-136 us on four waves against 117-119 on eight, either MFMA shape
+    // (the library GEMM itself takes 113 us with this layout).
+    if (b_ncontig && !conv && v.bm * v.bn >= 256 * 256 && v.waves_m * v.waves_n == 4) prior *= 0.8;
     {
       // A CU with fewer than 8 resident waves (one 4-wave workgroup, the launch too small or
       // the tile's LDS too large for a second) hides less latency.  The fourth root is fitted
@@ -501,12 +505,12 @@ int select_contraction_variant(int m, int n, int k, bool conv) {
 
 namespace {
 
-int pick_contraction(const char *op, const std::string &cache_key, int m, int n, int k, bool conv) {
+int pick_contraction(const char *op, const std::string &cache_key, int m, int n, int k, bool conv, bool b_ncontig = false) {
   const int forced = forced_variant(op);
   if (forced >= 0) return forced;
   int cached = tuning_cache_lookup_variant(cache_key);
   if (cached >= 0) return cached;
-  return select_contraction_variant(m, n, k, conv);
+  return select_contraction_variant(m, n, k, conv, b_ncontig);
 }
 
 // The variant (on 32x32x16 MFMAs) with the same tile shape and the given pipeline mode, or -1.
@@ -525,19 +529,11 @@ int twin(int vi, int pipeline) {
 // direct-to-LDS loads (pipelines 2 and 3) address operands with 32-bit byte
 // offsets, so operands of 2 GiB and more go through registers (`staged`); the
 // register-staged pipelined loop (pipeline 1) has no K-tail masking for a GEMM; the members on 16x16x32
-// MFMAs exist for a GEMM on pipeline 2 with a K-contiguous B.
+// MFMAs exist for a GEMM on pipeline 2.
 int resolve_variant(int vi, bool conv, bool staged, bool k_exact, bool b_ncontig) {
-  if (contraction_variant(vi).mfma == 16 && (conv || b_ncontig || staged)) {
-    // the member with the same tile on 32x32x16 MFMAs; of several wave layouts the one with the most waves
-    // (with an N-contiguous B, 4096^3: eight waves 117 us, four 131)
-    const ContractionVariant &p = contraction_variant(vi);
-    int t = twin(vi, 2);
-    for (int i = 0; i < contraction_variant_count(); ++i) {
-      const ContractionVariant &v = contraction_variant(i);
-      if (v.pipeline == 2 && v.mfma == 32 && v.bm == p.bm && v.bn == p.bn && v.bk == p.bk &&
-          (t < 0 || v.waves_m * v.waves_n > contraction_variant(t).waves_m * contraction_variant(t).waves_n))
-        t = i;
-    }
+  (void)b_ncontig;
+  if (contraction_variant(vi).mfma == 16 && (conv || staged)) {
+    const int t = twin(vi, 2);  // the member with the same tile on 32x32x16 MFMAs
     if (t >= 0) vi = t;
     else return select_contraction_variant(1024, 1024, 1024, conv);  // (every such member has a twin; not reached)
   }
@@ -724,7 +720,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.epi = chain;
       char key[160];
       snprintf(key, sizeof(key), "gemm_%lld_%lld_%lld_%s", M, N, K, tuning_device_name());
-      int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false);
+      int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false, !b_kcontig);
       if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "gemm: no kernel variant available");
       // direct-to-LDS variants address operands with 32-bit byte offsets below 2 GiB
       const long long a_extent = ((M - 1) * a.stride[0] + K) * 2;

@@ -108,7 +108,7 @@ TraceaStatus dispatch_attention(const TraceaTensorView &q, const TraceaTensorVie
 
 // Heuristic choice among the feasible contraction variants (used when neither a
 // forced variant nor a tuning-cache entry decides).  Returns -1 if none fits.
-int select_contraction_variant(int m, int n, int k, bool conv);
+int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig = false);
 
 // TraceaResult builders: strings are malloc'ed, released by tracea_free_string.
 struct PipelineConfig;
