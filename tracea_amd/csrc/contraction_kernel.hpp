@@ -1126,6 +1126,28 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         }
       }
     };
+    // (16x16x32) fragment u of the k-step: A fragments first, then B
+    auto read_one = [&](int set, const unsigned char *sA, const unsigned char *sB, int ks, int u) {
+      const int coff = ((ks * 4 + q16) ^ swz16) << 4;
+      if (u < 2 * FM) {
+        fa[set][u] = *(const u32x4 *)(sA + (wm * TM + row16) * ROW_BYTES + u * 16 * ROW_BYTES + coff);
+      } else {
+        const int j = u - 2 * FM;
+        if constexpr (B_NCONTIG) fb[set][j] = read_b_tr16(sB, j, ks);
+        else fb[set][j] = *(const u32x4 *)(sB + (wn * TN + row16) * ROW_BYTES + j * 16 * ROW_BYTES + coff);
+      }
+    };
+    // requests [lo, hi) of a tile and the operand reads of a k-step in alternation, in program order
+    auto mixed = [&](unsigned char *dA, unsigned char *dB, int k0, int lo, int hi, int set, const unsigned char *sA,
+                     const unsigned char *sB, int ks) {
+      constexpr int NR = XF * FM + XF * FN;
+#pragma unroll
+      for (int u = 0; u < NR; ++u) {
+        const int p0 = lo + (u * (hi - lo)) / NR, p1 = lo + ((u + 1) * (hi - lo)) / NR;
+        if (p1 > p0) dma(dA, dB, k0, p0, p1);
+        read_one(set, sA, sB, ks, u);
+      }
+    };
     auto mma = [&](int set) {
       if constexpr (MS == 16) {
 #pragma unroll
@@ -1147,7 +1169,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     // requested in front of the barrier has only that one k-step to arrive in: three quarters go out behind
     // the barrier, and in both k-steps the requests are issued ahead of the operand reads.  Measured at
     // 4096^3 on four waves (same box): shares of 8/10/12/14/16 of 16 requests behind the barrier 123 / 107.7 /
-    // 108.5 / 127 / 119 us; reads first, halves: 113-116 us.
+    // 108.5 / 127 / 119 us; reads first, halves: 113-116 us.  (With the alternation behind the barrier the
+    // shares from 10 to 16 are within a percent of each other.)
     constexpr bool DMA_FIRST = MS == 16;
     constexpr int CUT1 = MS == 16 ? (L * 3) / 4 : L / SPREAD, CUT2 = SPREAD == 3 ? 2 * L / SPREAD : L;
     dma(smem, smem + A_STAGE, 0, 0, L);
@@ -1187,10 +1210,12 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       // kt+2 into it (clamped to the last tile, whose second copy is never read)
       // while the last k-step of tile kt runs from registers
       if constexpr (DMA_FIRST) {
-        dma(cur, cur + A_STAGE, (kt + 2 < nk ? kt + 2 : nk - 1) * BK, 0, CUT1);
-        read_operands(0, nxt, nxt + A_STAGE, 0);
+        // (behind the barrier requests and operand reads alternate, one group of either kind per MFMA slot:
+        // a block of twelve requests in front of the reads held the MFMAs up, 105.8-106.2 against 103.8-104.7 us;
+        // in front of the barrier the same alternation delays the requests and costs 5 %)
+        mixed(cur, cur + A_STAGE, (kt + 2 < nk ? kt + 2 : nk - 1) * BK, 0, CUT1, 0, nxt, nxt + A_STAGE, 0);
         mma((KS - 1) & 1);
-        Sequenced<0, R, 0x020, CUT1, 0x100, D>::run();
+        Interleave<0, R, 0x120, CUT1 + D, 0x100, 0>::run();
       } else {
         read_operands(0, nxt, nxt + A_STAGE, 0);
         dma(cur, cur + A_STAGE, (kt + 2 < nk ? kt + 2 : nk - 1) * BK, 0, CUT1);
