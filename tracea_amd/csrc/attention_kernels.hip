@@ -63,6 +63,18 @@ struct MfmaValu {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
+// max(x, x of lane l ^ 32) without a trip through LDS: v_permlane32_swap exchanges the upper half of its
+// first operand with the lower half of its second; given the same value twice, the two results are a
+// lane's own value and its partner's, in one order or the other.  (Written as an instruction: the
+// compiler's builtin for the swap hands back its first result twice, and the maximum of the two would be
+// folded away.  The s_nop covers the wait the hardware asks for between a vector-ALU write of an operand
+// and the swap, which the compiler cannot see to insert.)
+__device__ __forceinline__ float max_with_lane_xor32(float x) {
+  float a0 = x, a1 = x;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a0), "+v"(a1));
+  return fmaxf(a0, a1);
+}
+
 template <int DT>
 __device__ __forceinline__ u32x4 pack8(const float (&p)[8]) {
   if constexpr (DT == DT_F16) {
@@ -531,7 +543,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           }
           mx = fmaxf(mx, s[qi][blk][e]);
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_with_lane_xor32(mx);
       const float m_new = fmaxf(m_run[qi], mx * a.scale_log2);
       moved |= m_new > m_run[qi];
       alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - m_new);
@@ -714,7 +726,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       bool moved = false;
 #pragma unroll
       for (int qi = 0; qi < QB; ++qi) {
-        const float mw = fmaxf(mx[qi], __shfl_xor(mx[qi], 32, 64));
+        const float mw = max_with_lane_xor32(mx[qi]);
         const float m_new = fmaxf(m_run[qi], mw * a.scale_log2);
         moved |= m_new > m_run[qi];
         alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - m_new);
@@ -824,6 +836,10 @@ static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream
 #undef TRACEA_FA_LAUNCH
 }
 
+}  // namespace tracea_amd
+#include "attention_m16_kernel.hpp"
+namespace tracea_amd {
+
 // The buffer loads address a (batch, head) slice with 32-bit byte offsets.
 static bool slice_fits(const AttentionArgs &a) {
   const long long k_ext = ((long long)(a.S - 1 + 4 * FA_BKV) * a.k_ss + a.D) * 2;  // (tiles up to 3 past the end are requested)
@@ -860,27 +876,32 @@ static int launch_fa2(const AttentionArgs &a, int dtype, hipStream_t stream) {
 static bool feasible_d128(const AttentionArgs &a) { return a.D == 128; }
 static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 
-// The kernel family: queries per workgroup (32 per wave, 4 or 8 waves), K/V ring depth (2 or 3 stages per
+// The kernel family: MFMA shape (m16: v_mfma_f32_16x16x32, attention_m16_kernel.hpp; the others 32x32x16),
+// queries per workgroup (32 per wave, 4 or 8 waves), K/V ring depth (2 or 3 stages per
 // tensor), head dimension, and the three kernel forms (pipe2 / pipe: direct-to-LDS tiles, maximum taken
 // under the P.V MFMAs or in a phase of its own; tr / u16: the register-staged cross-check).  The tuner
-// measures every feasible member (tracea_tune_fa2); the first feasible entry is the default.  (Head
+// measures every feasible member (tracea_tune_fa2); the first feasible entry is the default.  (The m16
+// members need 13 % more cycles than pipe2 and get a higher clock from the power limit: at B4 H32 S4096 D128
+// 1055-1062 us against 1070 dense, 629-639 against 625 causal, so they are not the default.)  (Head
 // dimension 128 has no 3-stage member: the third set of per-lane tile addresses does not fit the 256
 // registers of two waves per SIMD and the kernel spills.)
 static const AttentionVariant kAttentionVariants[] = {
-    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128},
-    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64},
-    {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128},
-    {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64},
-    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128},
-    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64},
-    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64},
-    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3>, &feasible_pipe_d64},
-    {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128},
-    {"fa2_q128_kv64_d64_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, false, 4, 2>, &feasible_pipe_d64},
-    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, true>, &feasible_d128},
-    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, false>, &feasible_d128},
-    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, true>, &feasible_d64},
-    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, false>, &feasible_d64},
+    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128, 32},
+    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64, 32},
+    {"fa2_q128_kv64_d128_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<128, 4>, &feasible_pipe_d128, 16},
+    {"fa2_q128_kv64_d64_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<64, 4>, &feasible_pipe_d64, 16},
+    {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128, 32},
+    {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64, 32},
+    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128, 32},
+    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64, 32},
+    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64, 32},
+    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3>, &feasible_pipe_d64, 32},
+    {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128, 32},
+    {"fa2_q128_kv64_d64_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, false, 4, 2>, &feasible_pipe_d64, 32},
+    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, true>, &feasible_d128, 32},
+    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, false>, &feasible_d128, 32},
+    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, true>, &feasible_d64, 32},
+    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, false>, &feasible_d64, 32},
 };
 
 int attention_variant_count() { return (int)(sizeof(kAttentionVariants) / sizeof(kAttentionVariants[0])); }

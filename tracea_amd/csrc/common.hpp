@@ -226,6 +226,7 @@ struct AttentionVariant {
   int stages;  // LDS stages per K and per V ring
   int (*launch)(const AttentionArgs &, int dtype, hipStream_t);
   bool (*feasible)(const AttentionArgs &);
+  int mfma;  // MFMA shape: 32 (32x32x16) or 16 (16x16x32)
 };
 int attention_variant_count();
 const AttentionVariant &attention_variant(int i);

@@ -232,7 +232,7 @@ PipelineConfig config_for_attention_variant(int index) {
   c.swizzle_mode = "Xor8";
   c.has_force_num_warps = true;
   c.force_num_warps = (uint32_t)v.waves;
-  c.intrinsic_shape = "M32N32K2";
+  c.intrinsic_shape = v.mfma == 16 ? "M16N16K4" : "M32N32K2";
   c.attention_variant = "FlashV2";
   c.softmax_granularity = "PerTile";
   c.double_buffer = true;
