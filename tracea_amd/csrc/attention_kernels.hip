@@ -88,6 +88,23 @@ __device__ __forceinline__ u32x4 pack8(const float (&p)[8]) {
   }
 }
 
+// The running maximum follows the scores lazily: it moves (and O and the row sum are rescaled) only when a
+// tile's maximum exceeds it by more than FA_RESCALE_TAU in the exponent's log2 units.  Softmax needs ONE
+// reference value per query for all its keys, not the true maximum: with a reference up to TAU below it the
+// probabilities of a tile reach 2^TAU instead of 1, far inside the range of fp32 sums and 16-bit operands,
+// and the final division by the row sum takes the factor out again.  With the exact maximum a wave of 32
+// queries rescales in about 54 of the 64 tiles of a 4096-key sequence (some query's maximum moves in a tile
+// with probability min(1, 32/t)), 64 multiplies each on a vector ALU that is the busiest unit of the kernel;
+// lazily it rescales once or twice.  (A dominant key still moves the reference at once.)
+constexpr float FA_RESCALE_TAU = 8.0f;
+__device__ __forceinline__ bool lazy_running_max(float &m_run, float candidate, float &alpha) {
+  const bool moved = candidate > m_run + FA_RESCALE_TAU;
+  const float m_new = moved ? candidate : m_run;
+  alpha = __builtin_amdgcn_exp2f(m_run - m_new);  // exactly 1 where the reference stays
+  m_run = m_new;
+  return moved;
+}
+
 constexpr int FA_BQ = 128;   // query rows per workgroup
 constexpr int FA_BKV = 64;   // keys per tile
 constexpr int FA_WAVES = 4;
@@ -544,10 +561,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           mx = fmaxf(mx, s[qi][blk][e]);
         }
       mx = max_with_lane_xor32(mx);
-      const float m_new = fmaxf(m_run[qi], mx * a.scale_log2);
-      moved |= m_new > m_run[qi];
-      alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - m_new);
-      m_run[qi] = m_new;
+      moved |= lazy_running_max(m_run[qi], mx * a.scale_log2, alpha[qi]);
     }
     return moved;
   };
@@ -643,12 +657,6 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       constexpr int EPC = 32 * QB / KS;  // exponentials per chunk
       static_assert((32 * QB) % KS == 0 && (EPC == 4 || EPC == 8 || EPC == 16), "exponentials must divide over the k-steps");
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int qi = 0; qi < QB; ++qi)
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-          for (int e = 0; e < 16; ++e) s_nxt[qi][blk][e] = 0.0f;
       u32x4 kf0 = *(const u32x4 *)(sKn + k_piece(lrow, g));
       u32x4 kf1 = *(const u32x4 *)(sKn + k_piece(32 + lrow, g));
       float lsum[QB];
@@ -664,8 +672,10 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         }
 #pragma unroll
         for (int qi = 0; qi < QB; ++qi) {
-          s_nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], s_nxt[qi][0]);
-          s_nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], s_nxt[qi][1]);
+          // (the first k-step starts from the MFMA's constant zero: no 32 registers to clear per tile)
+          const f32x16 zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+          s_nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], ks == 0 ? zero16 : s_nxt[qi][0]);
+          s_nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], ks == 0 ? zero16 : s_nxt[qi][1]);
         }
 #pragma unroll
         for (int j = 0; j < EPC; ++j) {
@@ -727,10 +737,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
       for (int qi = 0; qi < QB; ++qi) {
         const float mw = max_with_lane_xor32(mx[qi]);
-        const float m_new = fmaxf(m_run[qi], mw * a.scale_log2);
-        moved |= m_new > m_run[qi];
-        alpha[qi] = __builtin_amdgcn_exp2f(m_run[qi] - m_new);
-        m_run[qi] = m_new;
+        moved |= lazy_running_max(m_run[qi], mw * a.scale_log2, alpha[qi]);
       }
       rescale(moved);
     }

@@ -193,10 +193,7 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
       const float mw = row_max(mx[qb]);
-      const float m_new = fmaxf(m_run[qb], mw * a.scale_log2);
-      moved |= m_new > m_run[qb];
-      alpha[qb] = __builtin_amdgcn_exp2f(m_run[qb] - m_new);
-      m_run[qb] = m_new;
+      moved |= lazy_running_max(m_run[qb], mw * a.scale_log2, alpha[qb]);
     }
     return moved;
   };
