@@ -96,6 +96,40 @@ def test_dominant_key_needs_the_true_running_maximum(tracea_gpu, variant, dom_mo
         capi.force_variant("attention", -1)
 
 
+@pytest.mark.parametrize("variant", [("q128", "pipe2"), ("q128", "m16"), ("q256", "s2_pipe2"), ("q128", "pipe")], ids=lambda v: "_".join(v))
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+@pytest.mark.parametrize("step", [0.05, 0.11, 0.3])
+def test_scores_that_climb_along_the_sequence(tracea_gpu, variant, dtype, step):
+    """The kernels' reference value for the softmax moves only when a tile's maximum is more than 2^8 above
+    it.  Here every query's score grows linearly with the key index, by step * 64 per tile in the exponent's
+    log2 units (3.2, 7, 19): below the threshold (the reference lags by several tiles and probabilities
+    reach 2^8), just under it, and above it (it moves at every tile).  The output must be the oracle's in all
+    three regimes, dense and causal, and at a sequence end inside a tile."""
+    from tracea_amd import capi
+    tdt, rnd = (torch.bfloat16, round_bf16) if dtype == "bf16" else (torch.float16, round_f16)
+    b, h, s, d = 1, 2, 600, 128
+    rng = np.random.default_rng(int(step * 100))
+    # q = (c, 0, 0, ...) + noise, k_j = (j * u, ...) + noise: q.k_j / sqrt(d) * log2(e) = step * j + O(1)
+    c = 8.0
+    u = step * np.sqrt(d) / (c * np.log2(np.e))
+    q = rng.standard_normal((b, h, s, d)) * 0.3
+    k = rng.standard_normal((b, h, s, d)) * 0.3
+    q[..., 0] = c
+    k[..., 0] = np.arange(s) * u
+    v = rng.standard_normal((b, h, s, d))
+    q, k, v = rnd(q), rnd(k), rnd(v)
+    name = _member(capi, variant, d)
+    capi.force_variant("attention", name)
+    try:
+        for causal in (False, True):
+            ref = oracle.attention_bhsd(q, k, v, 1.0 / np.sqrt(d), causal)
+            got = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal).float().cpu().numpy()
+            assert np.isfinite(got).all()
+            assert_close_scaled(got, ref, _tol(d, dtype), "%s step %.2f causal=%s" % (name, step, causal))
+    finally:
+        capi.force_variant("attention", -1)
+
+
 def test_reference_gpu_check_shape(tracea_gpu):
     # examples/verify_fa2_gpu.rs:67-162: B1 H4 S512 D64 causal, inputs U[0,0.2), tolerance 2e-3
     rng = np.random.default_rng(42)
