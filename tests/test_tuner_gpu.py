@@ -90,6 +90,18 @@ def test_tune_fa2_returns_a_flash_variant(tracea_gpu, cache_file):
     assert cfg["attention_variant"] == "FlashV2" and score > 0.0
     ok, _, _, err = capi.take_result(capi.lib().tracea_tune_fa2(1, 2, 256, 96, True))
     assert not ok and "D 64 or 128" in err
+    # the record decides which member of the family later calls on this problem run
+    q, k, v = [torch.randn(1, 2, 256, 64, device="cuda").bfloat16() for _ in range(3)]
+    tracea_gpu.attention(q, k, v, causal=True)
+    ran = capi.last_variant("attention")
+    shape = "M16N16K4" if ran.endswith("_m16") else "M32N32K2"
+    assert ("q%d_" % cfg["m_tile"]) in ran and cfg["intrinsic_shape"] == shape
+    # without a record: dense attention over a long sequence takes 256 queries on eight waves, causal the 128-query member
+    q, k, v = [torch.randn(4, 32, 2048, 128, device="cuda").bfloat16() for _ in range(3)]
+    tracea_gpu.attention(q, k, v, causal=False)
+    assert capi.last_variant("attention") == "fa2_q256_kv64_d128_s2_pipe2"
+    tracea_gpu.attention(q, k, v, causal=True)
+    assert capi.last_variant("attention") == "fa2_q128_kv64_d128_pipe2"
 
 
 def test_tuner_cli_writes_the_reference_record(tracea_gpu, cache_file, tmp_path):

@@ -2037,8 +2037,22 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
   a.scale_log2 = scale * 1.4426950408889634f;
   a.causal = params.causal ? 1 : 0;
 
+  // Choice of the family member: a forced one, else the tuner's record of this problem, else by rule.
   int vi = forced_variant("attention");
   if (vi >= 0 && !attention_variant(vi).feasible(a)) vi = -1;
+  if (vi < 0) vi = tuning_cache_lookup_attention(a);
+  if (vi < 0 && !a.causal && S >= 2048 && B * H * ((S + 255) / 256) >= 2 * device_limits().cus) {
+    // Dense attention over a long sequence with enough workgroups to go round: 256 queries on eight waves share
+    // every K/V tile (B4 H32 S4096 D128: 997-999 us against 1013 for 128 queries on four).  Under a causal mask
+    // the smaller block wins (584 against 624 us: less masked work on the diagonal, finer load balance).
+    for (int i = 0; i < attention_variant_count(); ++i) {
+      const AttentionVariant &v = attention_variant(i);
+      if (v.block_q == 256 && v.waves == 8 && v.stages == 2 && v.mfma == 32 && v.feasible(a)) {
+        vi = i;
+        break;
+      }
+    }
+  }
   if (vi < 0) {
     for (int i = 0; i < attention_variant_count(); ++i)
       if (attention_variant(i).feasible(a)) {

@@ -240,6 +240,29 @@ PipelineConfig config_for_attention_variant(int index) {
   return c;
 }
 
+int attention_variant_for_config(const PipelineConfig &c, const AttentionArgs &a) {
+  for (int i = 0; i < attention_variant_count(); ++i) {
+    const AttentionVariant &v = attention_variant(i);
+    if ((uint32_t)v.block_q != c.m_tile || (uint32_t)v.stages != c.num_stages) continue;
+    if (c.has_force_num_warps && (uint32_t)v.waves != c.force_num_warps) continue;
+    if ((c.intrinsic_shape == "M16N16K4") != (v.mfma == 16)) continue;
+    if (v.feasible(a)) return i;
+  }
+  return -1;
+}
+
+std::string attention_cache_key(size_t b, size_t s, size_t h, size_t d, bool causal) {
+  char key[200];
+  snprintf(key, sizeof(key), "fa2_kernel:b%zu_s%zu_h%zu_d%zu_%s", b, s, h, d, causal ? "causal" : "dense");
+  return key;
+}
+
+int tuning_cache_lookup_attention(const AttentionArgs &a) {
+  CacheEntry e;
+  if (!tuning_cache_get(attention_cache_key((size_t)a.B, (size_t)a.S, (size_t)a.H, (size_t)a.D, a.causal != 0), &e)) return -1;
+  return attention_variant_for_config(e.config, a);
+}
+
 char *dup_cstr(const std::string &s) {
   char *p = (char *)malloc(s.size() + 1);
   if (p) memcpy(p, s.c_str(), s.size() + 1);
@@ -639,8 +662,7 @@ TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
   e.score = (float)best_tflops;
   e.timestamp = now_seconds();
   // key of the reference's attention adapter (src/kernels/attention/cuda_adapter.rs)
-  char key[200];
-  snprintf(key, sizeof(key), "fa2_kernel:b%zu_s%zu_h%zu_d%zu_%s", b, s, h, d, causal ? "causal" : "dense");
+  const std::string key = attention_cache_key(b, s, h, d, causal);
   tuning_cache_put(key, e, true);
   record_history(key, e, "BF16");
   return success(e.config, e.score);

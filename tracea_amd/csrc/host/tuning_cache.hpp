@@ -4,6 +4,7 @@
 #pragma once
 #include <string>
 
+#include "../common.hpp"
 #include "pipeline_config.hpp"
 
 namespace tracea_amd {
@@ -47,5 +48,11 @@ int tuning_cache_lookup_variant(const std::string &key);
 PipelineConfig config_for_contraction_variant(int index);
 int contraction_variant_for_config(const PipelineConfig &c);
 PipelineConfig config_for_attention_variant(int index);
+// First attention variant with the config's queries per workgroup, wave count, ring depth and MFMA shape that is
+// feasible for `a`, or -1; and the variant a cached record of the problem names (key of the reference's attention
+// adapter, src/kernels/attention/cuda_adapter.rs), or -1.
+int attention_variant_for_config(const PipelineConfig &c, const AttentionArgs &a);
+int tuning_cache_lookup_attention(const AttentionArgs &a);
+std::string attention_cache_key(size_t b, size_t s, size_t h, size_t d, bool causal);
 
 }  // namespace tracea_amd
