@@ -897,6 +897,8 @@ static const AttentionVariant kAttentionVariants[] = {
     {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64, 32},
     {"fa2_q128_kv64_d128_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<128, 4>, &feasible_pipe_d128, 16},
     {"fa2_q128_kv64_d64_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<64, 4>, &feasible_pipe_d64, 16},
+    {"fa2_q256_kv64_d128_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<128, 8>, &feasible_pipe_d128, 16},
+    {"fa2_q256_kv64_d64_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<64, 8>, &feasible_pipe_d64, 16},
     {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128, 32},
     {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64, 32},
     {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128, 32},
