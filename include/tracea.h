@@ -292,18 +292,19 @@ TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaT
 
 
 /* Split-K.  A gemm / conv2d launch with few output tiles and a long K (tiles * 2 <= 256 CUs,
- * at least 8 K tiles; 32 K tiles of 16 for the 64x64 tile of the fp32 GEMM) is split along K
+ * at least 8 K tiles; the 64x64 tile of the fp32 GEMM: up to about four workgroups per CU, ranges of at least
+ * 16 K tiles of 16) is split along K
  * over more workgroups; fp32 partial products go to a
  * scratch buffer the library keeps per (device, stream) (grown on demand up to 64 MiB, never
  * while the stream is being captured, never freed) and a second kernel sums them and applies
  * the operator chain.  On by default; tracea_set_split_k(0) turns it off.
  * tracea_last_split_k: K ranges of the calling thread's latest gemm / conv2d launch (1: not split).
- * Half-precision launches on tiles up to 128x128 that are split at most four ways need no second kernel: every workgroup leaves its partial
+ * Half-precision launches on tiles up to 128x128 and fp32 launches that are split at most four ways need no second kernel: every workgroup leaves its partial
  * product in the scratch buffer and takes a ticket from a per-tile counter (4 bytes per tile, per (device,
  * stream), zero between launches); the workgroup that draws a tile's last ticket sums the partial products in
  * K order, applies the operator chain and writes the tile.  Results equal those of the two-kernel form bit for
  * bit (same order of summation).  tracea_set_split_k_one_launch(0) goes back to two kernels everywhere (the
- * fp32 GEMM, the larger tiles, finer splits and tracea_gemm_noalloc always use two: with many K ranges the
+ * larger half-precision tiles, finer splits and tracea_gemm_noalloc always use two: with many K ranges the
  * reduction kernel, which spreads the sum over the device, is faster than one workgroup per tile);
  * tracea_last_split_k_launches says which
  * form the calling thread's latest gemm / conv2d launch took (1 or 2).  (The reference has no split along K:

@@ -212,6 +212,29 @@ def _conv_one_and_two_launches(tracea_gpu, capi, x, w, ops):
         torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("shape", [(1024, 1024, 1024), (512, 512, 1024), (100, 36, 2052), (768, 1024, 512)])
+def test_fp32_one_launch_split_equals_the_two_launch_form(tracea_gpu, launch_switch, shape):
+    """The fp32 GEMM on 64x64 tiles: K ranges summed by the tile's last workgroup or by the reduction kernel,
+    the same ranges in the same order, hence the same bits; and the float64 product within 1e-4 sqrt(K)."""
+    capi = launch_switch
+    m, n, k = shape
+    rng = np.random.default_rng(m + n + k)
+    a = _dev(rng.uniform(-1, 1, (m, k)).astype(np.float32))
+    b = _dev(rng.uniform(-1, 1, (k, n)).astype(np.float32))
+    bias = _dev(rng.standard_normal(n).astype(np.float32))
+    capi.lib().tracea_set_split_k_one_launch(0)
+    two = tracea_gpu.gemm(a, b, bias=bias, epilogue="bias")
+    splits = capi.lib().tracea_last_split_k()
+    assert splits >= 2 and capi.lib().tracea_last_split_k_launches() == 2
+    capi.lib().tracea_set_split_k_one_launch(1)
+    for rep in range(3):
+        one = tracea_gpu.gemm(a, b, bias=bias, epilogue="bias")
+        assert capi.lib().tracea_last_split_k() == splits and capi.lib().tracea_last_split_k_launches() == 1
+        assert torch.equal(one, two), "call %d" % rep
+    want = a.double().cpu().numpy() @ b.double().cpu().numpy() + bias.double().cpu().numpy()
+    np.testing.assert_allclose(one.cpu().numpy(), want, rtol=0, atol=1e-4 * np.sqrt(k))
+
+
 def test_large_problems_are_not_split(tracea_gpu, split_switch):
     capi = split_switch
     a = torch.randn(2048, 1024, device="cuda").half()

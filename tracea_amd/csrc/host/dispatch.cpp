@@ -761,9 +761,43 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
     const long long ncu = device_limits().cus;
     const int tile = args.a_bytes != 0 && (double)((tiles64 + ncu - 1) / ncu) * 1.06 < (double)((tiles128 + ncu - 1) / ncu) * 4.0 ? 64 : 128;
-    const ContractionVariant &f32_tile = tile == 64 ? f32_tile64 : f32_tile128;
-    int k_split = 0;
-    const int splits = g_split_k_enabled.load() ? choose_split(f32_tile, (int)M, (int)N, (int)K, &k_split, tile == 64 ? 16 : 4) : 1;
+    int k_split = 0, splits = 1;
+    t_last_split_launches = 1;
+    const bool can_fuse = args.a_bytes != 0 && !static_only && g_split_k_enabled.load() && g_split_k_one_launch.load();
+    const int nk = (int)((K + 15) / 16);
+    if (tile == 64 && args.a_bytes != 0 && g_split_k_enabled.load()) {
+      // (the same K ranges whether the sum then runs in the launch or, for the entry point that must not
+      // allocate or with one-launch splits switched off, in a reduction kernel: the results are the same bits)
+      // The 64x64 tile splits in one launch (the tile's last workgroup sums, see the kernel), and it wants about
+      // four workgroups per CU: a workgroup is one wave per SIMD walking K alone, and the others' MFMAs run
+      // under its waits.  Ranges of at least 16 K tiles, at most four.  Measured (us, replayed graphs,
+      // unsplit -> split): 1024^3 30.3 -> 26.0, 1024x1024x2048 79.5 -> 44.4, 768x1024x1024 28.1 -> 22.6,
+      // 2048x1024x1024 55.5 -> 44.7, 1536^3 98.2 -> 95.3; 2048^3 (four tiles per CU as it is) stays unsplit.
+      long long want = (4 * ncu + tiles64 / 2) / tiles64;
+      if (want > kOneLaunchMaxSplits) want = kOneLaunchMaxSplits;
+      if (want > nk / 16) want = nk / 16;
+      if (want >= 2) {
+        const int per = (int)((nk + want - 1) / want);
+        k_split = per * 16;
+        splits = (nk + per - 1) / per;
+      }
+    } else {
+      const ContractionVariant &f32_tile0 = tile == 64 ? f32_tile64 : f32_tile128;
+      splits = g_split_k_enabled.load() ? choose_split(f32_tile0, (int)M, (int)N, (int)K, &k_split, tile == 64 ? 16 : 4) : 1;
+    }
+    const long long tiles = tile == 64 ? tiles64 : tiles128;
+    if (can_fuse && splits > 1 && splits <= kOneLaunchMaxSplits && tiles <= kFuseTiles) {
+      void *fws = splitk_scratch(c.device, stream, (size_t)tiles * (size_t)splits * (size_t)(tile * tile) * 4);
+      unsigned *cnt = fws != nullptr ? fuse_counters(c.device, stream) : nullptr;
+      if (cnt != nullptr) {
+        args.epi = chain;
+        args.k_split = k_split;
+        args.fuse_ws = (float *)fws;
+        args.fuse_count = cnt;
+        t_last_splits = splits;
+        return hip_status("gemm_f32 launch", launch_gemm_f32(args, tile, stream));
+      }
+    }
     TraceaStatus ws = TRACEA_SUCCESS;
     void *scratch = split_workspace("gemm_f32 launch", static_only, c.device, stream, splits, M, N, &ws);
     if (ws != TRACEA_SUCCESS) return ws;
@@ -782,6 +816,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     args.k_split = k_split;
     TraceaStatus st = hip_status("gemm_f32 launch", launch_gemm_f32(args, tile, stream));
     if (st != TRACEA_SUCCESS) return st;
+    t_last_split_launches = 2;
     return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
   }
   GenericGemmArgs g{};

@@ -199,7 +199,9 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   const int M = args.M, N = args.N;
   const int kb = args.k_split > 0 ? (int)blockIdx.y * args.k_split : 0;
   const int K = args.k_split > 0 ? min(args.K, kb + args.k_split) : args.K;
-  const long long zrow = args.k_split > 0 ? (long long)blockIdx.y * M : 0ll;
+  // one-launch split: see the block in front of the epilogue
+  const bool fused = args.k_split > 0 && args.fuse_ws != nullptr;
+  const long long zrow = args.k_split > 0 && !fused ? (long long)blockIdx.y * M : 0ll;
 
   constexpr unsigned OOB = 0x80000000u;
   __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)args.A, 0, (int)args.a_bytes, 0x00020000);
@@ -252,6 +254,13 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
+  // With one 32x32 block per wave (T = 1) every MFMA would wait for the one before it, the same accumulator
+  // being its input: the odd k pairs of a tile go to a second accumulator, added in once at the end, and
+  // the matrix pipe always has an independent MFMA to start.
+  f32x16 acc_odd;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc_odd[e] = 0.0f;
+
   const int lrow = lane & 31, lhalf = lane >> 5;
   // A: row wm*32T + i*32 + lrow, 16-byte columns 2h and 2h+1 (k = 8h .. 8h+7)
   int a_off[T][2];
@@ -294,11 +303,16 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
     // kt+1 spread between the MFMAs of the second half: with one wave per SIMD whatever is issued
     // between two barriers without an MFMA in flight is time the matrix pipe stands still
     auto mfma = [&](int u, int t) {
+      if constexpr (T == 1) {
+        if (t & 1) acc_odd = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][0][t], af[u][0][t >> 2][t & 3], acc_odd, 0, 0, 0);
+        else acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][0][t], af[u][0][t >> 2][t & 3], acc[0][0], 0, 0, 0);
+      } else {
 #pragma unroll
-      for (int i = 0; i < T; ++i)
+        for (int i = 0; i < T; ++i)
 #pragma unroll
-        for (int j = 0; j < T; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < T; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+      }
     };
 #pragma unroll
     for (int u = 0; u < KSUB; ++u)
@@ -334,7 +348,61 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   // requests past the end of K may still be writing zeros where the epilogue stages
   __builtin_amdgcn_s_waitcnt(0x0f70);
   __syncthreads();
+  if constexpr (T == 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[0][0][e] += acc_odd[e];
+  }
 
+  // One-launch split along K, as in the half-precision kernels: every workgroup leaves its partial product in
+  // block (tile, K range) of a workspace, in accumulator order, with device-scope stores (the K ranges of a
+  // tile may run on XCDs whose L2s do not see each other's lines), and takes a ticket; the workgroup that draws
+  // the tile's last ticket sums the blocks in K order, its own included, and runs the epilogue.  Nobody waits.
+  if (fused) {
+    __shared__ unsigned s_ticket;
+    constexpr int DEVICE_SCOPE = 16;  // the sc1 bit of a buffer instruction
+    const unsigned splits = gridDim.y;
+    constexpr unsigned TILE_BYTES = BM * BN * 4, WAVE_BYTES = TILE_BYTES / 4;
+    __amdgpu_buffer_rsrc_t rsrc_ws = __builtin_amdgcn_make_buffer_rsrc((void *)args.fuse_ws, 0, 0x7fffffff, 0x00020000);
+    const unsigned first = blockIdx.x * splits * TILE_BYTES + wave_u * WAVE_BYTES + lane * 16;
+    const unsigned mine = first + blockIdx.y * TILE_BYTES;
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+      for (int j = 0; j < T; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_ws, (int)(mine + ((i * T + j) * 4 + g) * 1024), 0,
+                                                 DEVICE_SCOPE);
+        }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stores are acknowledged
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(args.fuse_count + blockIdx.x, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != splits - 1) return;
+    if (tid == 0) __hip_atomic_store(args.fuse_count + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int i = 0; i < T; ++i)
+#pragma unroll
+      for (int j = 0; j < T; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+#pragma unroll 1
+    for (unsigned z = 0; z < splits; ++z) {
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int j = 0; j < T; ++j)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 v = __builtin_bit_cast(
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_ws, (int)(first + z * TILE_BYTES + ((i * T + j) * 4 + g) * 1024), 0,
+                                                           DEVICE_SCOPE));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] += v[e];
+          }
+    }
+  }
   f32_tile_epilogue<32, T, T>(acc, (float *)smem + wave_u * (32 * 32 * T), args, m0 + wm * (32 * T), n0 + wn * (32 * T),
                               zrow, lane);
 }
