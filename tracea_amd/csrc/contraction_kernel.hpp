@@ -703,11 +703,17 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   // requested here so that they arrive under the main loop.
   constexpr int TAB_ENTRIES = TRACEA_MAX_EPILOGUE_OPS * 2 * BN;
   constexpr int TPT = (TAB_ENTRIES + NT - 1) / NT;
+  // (An empty chain branches round all of it: the entries are some 1600 instructions with scalar loads
+  // between them, 4000 cycles in front of the first tile request of a launch that needs none of them.)
   float tabr[TPT];
 #pragma unroll
-  for (int i = 0; i < TPT; ++i) {
-    const int idx = tid + i * NT;
-    tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;
+  for (int i = 0; i < TPT; ++i) tabr[i] = 0.0f;
+  if (plan.n_ops > 0) {
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int idx = tid + i * NT;
+      tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;
+    }
   }
 
   // Every load is issued unconditionally from an address that is always
