@@ -28,7 +28,8 @@ def _tol(d, dtype):
 # members of the kernel family: (queries per workgroup, form); w4 = four waves of 64 queries, otherwise
 # 32 queries per wave; a member that a head dimension does not have (3-stage rings at D = 128) is skipped
 FAMILY = [("q128", "pipe"), ("q128", "pipe2"), ("q128", "tr"), ("q128", "u16"), ("q256", "s2_pipe2"),
-          ("q256", "s3_pipe2"), ("q128", "s3_pipe2"), ("q256", "w4_pipe2"), ("q128", "m16"), ("q256", "s2_m16")]
+          ("q256", "s3_pipe2"), ("q128", "s3_pipe2"), ("q256", "w4_pipe2"), ("q128", "m16"), ("q256", "s2_m16"),
+          ("q128", "pipe2_x2"), ("q256", "s2_pipe2_x2")]
 
 
 def _member(capi, variant, d):
@@ -126,6 +127,46 @@ def test_scores_that_climb_along_the_sequence(tracea_gpu, variant, dtype, step):
             got = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal).float().cpu().numpy()
             assert np.isfinite(got).all()
             assert_close_scaled(got, ref, _tol(d, dtype), "%s step %.2f causal=%s" % (name, step, causal))
+    finally:
+        capi.force_variant("attention", -1)
+
+
+@pytest.mark.parametrize("variant", [("q128", "pipe2"), ("q256", "s2_pipe2")], ids=lambda v: "_".join(v))
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_two_query_blocks_per_workgroup(tracea_gpu, variant, d, dtype):
+    """The _x2 members give a workgroup two query blocks (a heavy and a light one under a causal mask), the
+    second on K/V tiles and queries requested during the first.  Every query still sees its keys in the same
+    order with the same arithmetic: the output must equal the one-block member's bit for bit, on lengths that
+    end inside a tile, on scores that climb along the sequence and with a dominant key; the one-block member
+    is checked against the oracle on the same inputs.  A length with an odd number of blocks has no pairs: a
+    forced _x2 member is then not the one that runs."""
+    from tracea_amd import capi
+    tdt, rnd = (torch.bfloat16, round_bf16) if dtype == "bf16" else (torch.float16, round_f16)
+    bq = int(variant[0][1:])
+    single, paired = _member(capi, variant, d), _member(capi, (variant[0], variant[1] + "_x2"), d)
+    try:
+        for (b, h, s) in [(1, 2, 2 * bq), (2, 3, 4 * bq - 37), (1, 2, 8 * bq), (1, 1, 6 * bq - bq // 2 - 1)]:
+            rng = np.random.default_rng(s + d)
+            q, k, v = [rng.standard_normal((b, h, s, d)) * 0.5 for _ in range(3)]
+            q[..., 0] = 6.0
+            k[0, 0, :, 0] = np.arange(s) * (0.11 * np.sqrt(d) / (6.0 * np.log2(np.e)))  # climbing scores in one head
+            k[0, -1, s // 3, :] = 3.0                                                     # a dominant key in another
+            q, k, v = rnd(q), rnd(k), rnd(v)
+            for causal in (False, True):
+                capi.force_variant("attention", single)
+                one = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal)
+                assert capi.last_variant("attention") == single
+                capi.force_variant("attention", paired)
+                two = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal)
+                assert capi.last_variant("attention") == paired, (s, causal)
+                assert torch.equal(one, two), "%s S=%d causal=%s: differs from %s" % (paired, s, causal, single)
+                want = oracle.attention_bhsd(q, k, v, 1.0 / np.sqrt(d), causal)
+                assert_close_scaled(one.float().cpu().numpy(), want, _tol(d, dtype), "%s S=%d causal=%s" % (single, s, causal))
+        q, k, v = [_dev(rnd(np.random.default_rng(3).standard_normal((1, 2, 3 * bq, d))), tdt) for _ in range(3)]
+        capi.force_variant("attention", paired)
+        tracea_gpu.attention(q, k, v, causal=True)
+        assert capi.last_variant("attention") != paired
     finally:
         capi.force_variant("attention", -1)
 

@@ -96,10 +96,19 @@ def test_tune_fa2_returns_a_flash_variant(tracea_gpu, cache_file):
     ran = capi.last_variant("attention")
     shape = "M16N16K4" if ran.endswith("_m16") else "M32N32K2"
     assert ("q%d_" % cfg["m_tile"]) in ran and cfg["intrinsic_shape"] == shape
-    # without a record: dense attention over a long sequence takes 256 queries on eight waves, causal the 128-query member
+    assert cfg["fusion_count"] == (2 if ran.endswith("_x2") else 1)  # query blocks per workgroup
+    # without a record, with a pair of query blocks per CU or more: dense attention takes 256 queries on eight
+    # waves, causal 128 on four, two blocks per workgroup each
     q, k, v = [torch.randn(4, 32, 2048, 128, device="cuda").bfloat16() for _ in range(3)]
     tracea_gpu.attention(q, k, v, causal=False)
+    assert capi.last_variant("attention") == "fa2_q256_kv64_d128_s2_pipe2_x2"
+    tracea_gpu.attention(q, k, v, causal=True)
+    assert capi.last_variant("attention") == "fa2_q128_kv64_d128_pipe2_x2"
+    # an odd number of blocks has no pairs; few pairs leave CUs idle
+    q, k, v = [torch.randn(4, 32, 2048 + 256, 128, device="cuda").bfloat16() for _ in range(3)]
+    tracea_gpu.attention(q, k, v, causal=False)
     assert capi.last_variant("attention") == "fa2_q256_kv64_d128_s2_pipe2"
+    q, k, v = [torch.randn(1, 32, 1024, 128, device="cuda").bfloat16() for _ in range(3)]
     tracea_gpu.attention(q, k, v, causal=True)
     assert capi.last_variant("attention") == "fa2_q128_kv64_d128_pipe2"
 

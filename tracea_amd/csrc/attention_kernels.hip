@@ -384,10 +384,20 @@ fa2_fwd_kernel(const AttentionArgs a) {
 // ---------------------------------------------------------------------------
 // WAVES: waves of 32 queries per workgroup (4 or 8: 128 or 256 queries share every K/V tile);
 // NSTG: LDS stages per K and per V ring (2: tiles requested one iteration ahead, 3: two).
-template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB>
+// ITEMS: query blocks a workgroup takes one after the other (1 or 2; the reference's fusion_count,
+// src/optimizer/benchmark.rs:131-132).  With 2 the K/V rings run on across the two: the look-ahead requests
+// of the first block's last iterations fetch the second block's first tiles, its queries are fetched together
+// with the first block's, and O leaves from registers (the staging area in LDS would lie under those tiles)
+// -- the second block starts without a load to wait for.  Under a causal mask the pair is block j and block
+// nqb-1-j: every workgroup then has the same number of tiles.  Same bits as one block per workgroup.
+// Measured at B4 H32 S4096 D128 (replayed graphs, one box): dense 1002 -> 980 us on 8 waves, causal 585 -> 553
+// on 4.  (Four blocks per workgroup: the third set of queries in flight spills at head dimension 128, and the
+// coarser units balance worse: 999 and 572 us.)
+template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB, int ITEMS = 1>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 fa2_fwd_pipe_kernel(const AttentionArgs a) {
   static_assert(QB == 1 || (QB == 2 && EARLY_MAX), "two query blocks per wave exist in the two-phase form only");
+  static_assert(ITEMS == 1 || (ITEMS == 2 && EARLY_MAX), "pairs of query blocks exist in the two-phase form only");
   constexpr int WQ = 32 * QB;  // queries per wave
   constexpr int BQ = WQ * WAVES;
   constexpr int ROW_BYTES = D * 2;
@@ -411,13 +421,20 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   const int lrow = lane & 31, g = lane >> 5;
 
   const int nqb = (a.S + BQ - 1) / BQ;
-  const int total = nqb * a.B * a.H;
+  const int per_bh = nqb / ITEMS;  // workgroups per (batch, head); the host launches pairs for an even nqb only
+  const int total = per_bh * a.B * a.H;
   int vid = blockIdx.x;
   if ((total & 7) == 0) vid = (vid & 7) * (total >> 3) + (vid >> 3);
-  const int bh = vid / nqb;
-  const int qb = nqb - 1 - (vid - bh * nqb);
+  const int bh = vid / per_bh;
+  const int slot = vid - bh * per_bh;
+  // the query block of item i: alone, from the last block to the first; in pairs, a heavy and a light one
+  // under a causal mask and two neighbours otherwise
+  auto item_block = [&](int i) __attribute__((always_inline)) -> int {
+    if constexpr (ITEMS == 1) return nqb - 1 - slot;
+    else return a.causal ? (i == 0 ? nqb - 1 - slot : slot) : 2 * slot + i;
+  };
   const int b = bh / a.H, h = bh - b * a.H;
-  const int q0 = qb * BQ;
+  int q0 = item_block(0) * BQ;
   const int S = a.S;
 
   const unsigned short *Qg = (const unsigned short *)a.Q + (long long)b * a.q_sb + (long long)h * a.q_sh;
@@ -425,17 +442,22 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   const unsigned short *Vg = (const unsigned short *)a.V + (long long)b * a.v_sb + (long long)h * a.v_sh;
   unsigned short *Og = (unsigned short *)a.O + (long long)b * a.o_sb + (long long)h * a.o_sh;
 
-  const int q_wave0 = q0 + wave * WQ;
+  int q_wave0 = q0 + wave * WQ;
   int q_mine[QB];  // this lane's query in each of the wave's blocks of 32
   u32x4 qf[QB][KS];
+  auto load_q = [&](int first_query, u32x4 (&dst)[QB][KS]) __attribute__((always_inline)) {
 #pragma unroll
-  for (int qi = 0; qi < QB; ++qi) {
-    q_mine[qi] = q_wave0 + qi * 32 + lrow;
-    const int qr = q_mine[qi] < S ? q_mine[qi] : S - 1;
-    const unsigned short *qp = Qg + (long long)qr * a.q_ss + g * 8;
+    for (int qi = 0; qi < QB; ++qi) {
+      const int mine = first_query + wave * WQ + qi * 32 + lrow;
+      const int qr = mine < S ? mine : S - 1;
+      const unsigned short *qp = Qg + (long long)qr * a.q_ss + g * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[qi][ks] = *(const u32x4 *)(qp + ks * 16);
-  }
+      for (int ks = 0; ks < KS; ++ks) dst[qi][ks] = *(const u32x4 *)(qp + ks * 16);
+    }
+  };
+#pragma unroll
+  for (int qi = 0; qi < QB; ++qi) q_mine[qi] = q_wave0 + qi * 32 + lrow;
+  load_q(q0, qf);
 
   auto k_piece = [&](int row, int c) __attribute__((always_inline)) -> int {
     return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
@@ -477,12 +499,23 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           16, (int)(v_voff[i] + adv), 0, 0, 0);
   };
 
-  int ntiles = (S + FA_BKV - 1) / FA_BKV;
-  if (a.causal) {
-    const int last_q = (q0 + BQ - 1 < S ? q0 + BQ - 1 : S - 1);
-    const int need = last_q / FA_BKV + 1;
-    ntiles = need < ntiles ? need : ntiles;
-  }
+  auto tiles_of = [&](int first_query) __attribute__((always_inline)) -> int {
+    int n = (S + FA_BKV - 1) / FA_BKV;
+    if (a.causal) {
+      const int last_q = (first_query + BQ - 1 < S ? first_query + BQ - 1 : S - 1);
+      const int need = last_q / FA_BKV + 1;
+      n = need < n ? need : n;
+    }
+    return n;
+  };
+  int ntiles = tiles_of(q0);
+  // tb: K/V tiles of the items before the current one.  Tile t of an item lives in ring stage (tb + t) % NSTG,
+  // and a look-ahead request past the item's last tile fetches the next item's tiles (same batch and head).
+  int tb = 0, item = 0;
+  auto ahead = [&](int f) __attribute__((always_inline)) -> int {
+    if constexpr (ITEMS == 1) return f;
+    else return (f >= ntiles && item + 1 < ITEMS) ? f - ntiles : f;
+  };
 
   // (a key fragment read from LDS serves all QB query blocks of the wave: with one block every MFMA
   // needs 1 KB of LDS, which is all that LDS delivers while the four matrix pipes of the CU run)
@@ -504,18 +537,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   };
 
   f32x16 o[QB][DB];
-#pragma unroll
-  for (int qi = 0; qi < QB; ++qi)
-#pragma unroll
-    for (int d = 0; d < DB; ++d)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) o[qi][d][e] = 0.0f;
   float m_run[QB], l_run[QB];
-#pragma unroll
-  for (int qi = 0; qi < QB; ++qi) {
-    m_run[qi] = -1.0e30f;
-    l_run[qi] = 0.0f;
-  }
 
   // tiles at or beyond the end of the sequence lie outside the buffers and load as zeros
   // requests of a wave that may stay in flight where an iteration waits for its tiles: those of the
@@ -529,10 +551,9 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     load_v(1, sVbase + TILE_BYTES);
     load_k(2, sKbase + 2 * TILE_BYTES);
   }
-  __builtin_amdgcn_s_waitcnt(WAIT_TILES);
-  __syncthreads();
+  u32x4 qf_next[ITEMS > 1 ? QB : 1][KS];  // the second item's queries travel with the first tiles
+  if constexpr (ITEMS > 1) load_q(item_block(1) * BQ, qf_next);
   f32x16 s_cur[QB][2], s_nxt[QB][2];
-  scores(sKbase, s_cur);
 
   // Masks tile `tile`'s scores in s (EDGE only) and folds them into the running
   // maximum.  The maximum is taken over the raw scores (the scale is positive);
@@ -582,7 +603,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // the vector ALU.
   u32x4 pf[QB][4];
   auto softmax_and_next_scores = [&](int t) __attribute__((always_inline)) {  // (one query block per wave)
-    const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
+    const unsigned char *sKn = sKbase + ((tb + t + 1) % NSTG) * TILE_BYTES;
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -633,7 +654,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // interleaved instruction by instruction.  For EARLY_MAX the tag describes
   // tile t+1, the one whose maximum the iteration takes.
   auto iteration = [&](int t, auto edge_tag) __attribute__((always_inline)) {
-    const unsigned char *sV = sVbase + (t % NSTG) * TILE_BYTES;
+    const unsigned char *sV = sVbase + ((tb + t) % NSTG) * TILE_BYTES;
     if constexpr (!EARLY_MAX) {
       const bool moved = take_max(t, edge_tag, s_cur);
       rescale(moved);
@@ -650,7 +671,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       // matrix pipe works on its MFMAs, whatever order the compiler gives them
       // inside the chunk.
       constexpr bool EDGE = decltype(edge_tag)::value;
-      const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
+      const unsigned char *sKn = sKbase + ((tb + t + 1) % NSTG) * TILE_BYTES;
       // ---- phase A: S^T(t+1) = K(t+1) Q^T  with  P(t) = exp2(S(t)*scale - m), row sums ----
       // chunk ks: the 2*QB MFMAs of k-step ks (operands read one chunk ahead) and
       // 32*QB/KS of the 32*QB exponentials
@@ -747,6 +768,36 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       for (int blk = 0; blk < 2; ++blk) s_cur[qi][blk] = s_nxt[qi][blk];
   };
 
+#pragma unroll 1
+  for (item = 0; item < ITEMS; ++item) {
+  if constexpr (ITEMS > 1) {
+    if (item > 0) {
+      q0 = item_block(item) * BQ;
+      q_wave0 = q0 + wave * WQ;
+      ntiles = tiles_of(q0);
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) {
+        q_mine[qi] = q_wave0 + qi * 32 + lrow;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) qf[qi][ks] = qf_next[qi][ks];
+      }
+    }
+  }
+#pragma unroll
+  for (int qi = 0; qi < QB; ++qi) {
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) o[qi][d][e] = 0.0f;
+    m_run[qi] = -1.0e30f;
+    l_run[qi] = 0.0f;
+    alpha[qi] = 1.0f;
+  }
+  // (a later item finds its first tiles requested by the item before it, and published by that item's last barrier)
+  __builtin_amdgcn_s_waitcnt(WAIT_TILES);
+  __syncthreads();
+  scores(sKbase + (tb % NSTG) * TILE_BYTES, s_cur);
+
   // Interior tiles first, then the edge tiles (they are the last ones: the tail of
   // the sequence and, under a causal mask, the tiles that reach the diagonal of
   // this wave's queries), each in a loop of its own with a single body.
@@ -771,17 +822,52 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   for (; t < interior_end; ++t) {
     __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(t+1) and V(t), requested NSTG-1 iterations ago
     __syncthreads();
-    load_k(t + NSTG, sKbase + (t % NSTG) * TILE_BYTES);
-    load_v(t + NSTG - 1, sVbase + ((t + NSTG - 1) % NSTG) * TILE_BYTES);
+    load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
+    load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
     iteration(t, std::false_type{});
   }
   for (; t < ntiles; ++t) {
     __builtin_amdgcn_s_waitcnt(WAIT_TILES);
     __syncthreads();
-    load_k(t + NSTG, sKbase + (t % NSTG) * TILE_BYTES);
-    load_v(t + NSTG - 1, sVbase + ((t + NSTG - 1) % NSTG) * TILE_BYTES);
+    load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
+    load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
     iteration(t, std::true_type{});
   }
+  if constexpr (ITEMS > 1) {
+    // O from registers: the lanes of the two halves of the wave hold head-dim values 0..3 and 4..7 of a group
+    // of 8; one swap per register between the halves gives every lane 16 bytes of one row.
+#pragma unroll
+    for (int qi = 0; qi < QB; ++qi) {
+      const float l_tot = l_run[qi] + __shfl_xor(l_run[qi], 32, 64);
+      const float inv_l = 1.0f / l_tot;
+      unsigned short *orow = Og + (long long)q_mine[qi] * a.o_ss;
+#pragma unroll
+      for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int vp = 0; vp < 2; ++vp) {
+          u32x2 w[2];
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            float x[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = o[qi][d][(vp * 2 + half) * 4 + e] * inv_l;
+            if constexpr (DT == DT_F16) {
+              f16x4 hq = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
+              w[half] = __builtin_bit_cast(u32x2, hq);
+            } else {
+              bf16x4 hq = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
+              w[half] = __builtin_bit_cast(u32x2, hq);
+            }
+          }
+          unsigned e0 = w[0][0], e1 = w[0][1], o0 = w[1][0], o1 = w[1][1];
+          asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(e0), "+v"(o0));
+          asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(e1), "+v"(o1));
+          const u32x4 row16 = {e0, e1, o0, o1};
+          if (q_mine[qi] < S) *(u32x4 *)(orow + d * 32 + (vp * 2 + g) * 8) = row16;
+        }
+    }
+    tb += ntiles;
+  } else {
   __builtin_amdgcn_s_waitcnt(0x0f70);  // look-ahead loads must not land on the output staging
   __syncthreads();
 
@@ -817,17 +903,22 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     if (q < S)
       *(u32x4 *)(Og + (long long)q * a.o_ss + c * 8) = *(const u32x4 *)(so + row * ROW_BYTES + c * 16);
   }
+  }
+  }  // items
+  // (the last item's look-ahead requests write LDS: they must have landed before the workgroup gives it up)
+  if constexpr (ITEMS > 1) __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 
-template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1>
+template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1, int ITEMS = 1>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
-  constexpr size_t ring = 2 * (size_t)NSTG * FA_BKV * D * 2, staging = (size_t)WAVES * 32 * QB * D * 2;
+  constexpr size_t ring = 2 * (size_t)NSTG * FA_BKV * D * 2, staging = ITEMS > 1 ? 0 : (size_t)WAVES * 32 * QB * D * 2;
   constexpr size_t lds = ring > staging ? ring : staging;
   const int nqb = (a.S + 32 * QB * WAVES - 1) / (32 * QB * WAVES);
-  const dim3 grid((unsigned)(nqb * a.B * a.H)), block(WAVES * 64);
+  if (nqb % ITEMS != 0) return (int)hipErrorInvalidValue;  // (feasible_pairs keeps such a call away)
+  const dim3 grid((unsigned)(nqb / ITEMS * a.B * a.H)), block(WAVES * 64);
 #define TRACEA_FA_LAUNCH(DTV)                                                                  \
   do {                                                                                         \
-    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB>;                        \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB, ITEMS>;                 \
     static bool attr_done = false;                                                             \
     if (!attr_done) {                                                                          \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
@@ -856,6 +947,12 @@ static bool slice_fits(const AttentionArgs &a) {
 // (the running maximum is taken over raw scores, which needs a positive scale)
 static bool feasible_pipe_d128(const AttentionArgs &a) { return a.D == 128 && a.scale_log2 > 0.0f && slice_fits(a); }
 static bool feasible_pipe_d64(const AttentionArgs &a) { return a.D == 64 && a.scale_log2 > 0.0f && slice_fits(a); }
+// Two query blocks per workgroup: an even number of blocks, and at least two K/V tiles in the lightest one.
+template <int D, int BQ>
+static bool feasible_pairs(const AttentionArgs &a) {
+  const int nqb = (a.S + BQ - 1) / BQ;
+  return a.D == D && a.scale_log2 > 0.0f && slice_fits(a) && nqb % 2 == 0 && a.S >= 2 * FA_BKV;
+}
 
 template <int D, bool V_TR>
 static int launch_fa2(const AttentionArgs &a, int dtype, hipStream_t stream) {
@@ -893,24 +990,28 @@ static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 // dimension 128 has no 3-stage member: the third set of per-lane tile addresses does not fit the 256
 // registers of two waves per SIMD and the kernel spills.)
 static const AttentionVariant kAttentionVariants[] = {
-    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128, 32},
-    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64, 32},
-    {"fa2_q128_kv64_d128_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<128, 4>, &feasible_pipe_d128, 16},
-    {"fa2_q128_kv64_d64_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<64, 4>, &feasible_pipe_d64, 16},
-    {"fa2_q256_kv64_d128_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<128, 8>, &feasible_pipe_d128, 16},
-    {"fa2_q256_kv64_d64_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<64, 8>, &feasible_pipe_d64, 16},
-    {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128, 32},
-    {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64, 32},
-    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128, 32},
-    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64, 32},
-    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64, 32},
-    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3>, &feasible_pipe_d64, 32},
-    {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128, 32},
-    {"fa2_q128_kv64_d64_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, false, 4, 2>, &feasible_pipe_d64, 32},
-    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, true>, &feasible_d128, 32},
-    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, false>, &feasible_d128, 32},
-    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, true>, &feasible_d64, 32},
-    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, false>, &feasible_d64, 32},
+    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d128_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<128, 4>, &feasible_pipe_d128, 16, 1},
+    {"fa2_q128_kv64_d64_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<64, 4>, &feasible_pipe_d64, 16, 1},
+    {"fa2_q256_kv64_d128_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<128, 8>, &feasible_pipe_d128, 16, 1},
+    {"fa2_q256_kv64_d64_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<64, 8>, &feasible_pipe_d64, 16, 1},
+    {"fa2_q128_kv64_d128_pipe2_x2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 1, 2>, &feasible_pairs<128, 128>, 32, 2},
+    {"fa2_q128_kv64_d64_pipe2_x2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 1, 2>, &feasible_pairs<64, 128>, 32, 2},
+    {"fa2_q256_kv64_d128_s2_pipe2_x2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2, 1, 2>, &feasible_pairs<128, 256>, 32, 2},
+    {"fa2_q256_kv64_d64_s2_pipe2_x2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2, 1, 2>, &feasible_pairs<64, 256>, 32, 2},
+    {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q128_kv64_d64_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, false, 4, 2>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, true>, &feasible_d128, 32, 1},
+    {"fa2_q128_kv64_d128_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, false>, &feasible_d128, 32, 1},
+    {"fa2_q128_kv64_d64_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, true>, &feasible_d64, 32, 1},
+    {"fa2_q128_kv64_d64_u16", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<64, false>, &feasible_d64, 32, 1},
 };
 
 int attention_variant_count() { return (int)(sizeof(kAttentionVariants) / sizeof(kAttentionVariants[0])); }

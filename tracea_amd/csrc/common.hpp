@@ -226,7 +226,8 @@ struct AttentionVariant {
   int stages;  // LDS stages per K and per V ring
   int (*launch)(const AttentionArgs &, int dtype, hipStream_t);
   bool (*feasible)(const AttentionArgs &);
-  int mfma;  // MFMA shape: 32 (32x32x16) or 16 (16x16x32)
+  int mfma;   // MFMA shape: 32 (32x32x16) or 16 (16x16x32)
+  int items;  // query blocks a workgroup takes one after the other (1 or 2)
 };
 int attention_variant_count();
 const AttentionVariant &attention_variant(int i);

@@ -424,6 +424,8 @@ int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split,
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
   const long long cus = device_limits().cus;
+  static const int exp_min = getenv("TRACEA_EXP_MIN") ? atoi(getenv("TRACEA_EXP_MIN")) : 0;
+  if (exp_min > 0) min_tiles = exp_min;
   if (conv_only(v) || tiles * 2 > cus || nk < 2 * min_tiles) return 1;
   long long splits = cus / tiles;
   if (splits > nk / min_tiles) splits = nk / min_tiles;  // at least min_tiles K tiles per range
@@ -2076,18 +2078,25 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
   int vi = forced_variant("attention");
   if (vi >= 0 && !attention_variant(vi).feasible(a)) vi = -1;
   if (vi < 0) vi = tuning_cache_lookup_attention(a);
-  if (vi < 0 && !a.causal && S >= 2048 && B * H * ((S + 255) / 256) >= 2 * device_limits().cus) {
-    // Dense attention over a long sequence with enough workgroups to go round: 256 queries on eight waves share
-    // every K/V tile (B4 H32 S4096 D128: 997-999 us against 1013 for 128 queries on four).  Under a causal mask
-    // the smaller block wins (584 against 624 us: less masked work on the diagonal, finer load balance).
+  auto member = [&](int block_q, int waves, int items) {
     for (int i = 0; i < attention_variant_count(); ++i) {
       const AttentionVariant &v = attention_variant(i);
-      if (v.block_q == 256 && v.waves == 8 && v.stages == 2 && v.mfma == 32 && v.feasible(a)) {
-        vi = i;
-        break;
-      }
+      if (v.block_q == block_q && v.waves == waves && v.stages == 2 && v.mfma == 32 && v.items == items && v.feasible(a)) return i;
     }
-  }
+    return -1;
+  };
+  const long long cus = device_limits().cus, bh = (long long)(B * H);
+  // Two query blocks per workgroup where the pairs alone fill the device: the second block starts on tiles and
+  // queries already requested, and under a causal mask a heavy block is paired with a light one.  Sweep over
+  // B*H in {8, 32, 128, 512} and S in {512 ... 8192}, replayed graphs: with at least one pair per CU the paired
+  // member wins or ties (causal B4 H32 S4096 D128 585 -> 553 us, B1 H32 S2048 63.8 -> 52.2; dense B4 H32 S4096
+  // 1002 -> 980 on eight waves), with fewer it loses (causal B1 H32 S1024 26.2 -> 30.1).
+  if (vi < 0 && a.causal && bh * (((S + 127) / 128) / 2) >= cus) vi = member(128, 4, 2);
+  if (vi < 0 && !a.causal && bh * (((S + 255) / 256) / 2) >= cus) vi = member(256, 8, 2);
+  // Dense attention over a long sequence with enough workgroups to go round: 256 queries on eight waves share
+  // every K/V tile (B4 H32 S4096 D128: 997-999 us against 1013 for 128 queries on four).  Under a causal mask
+  // the smaller block wins (584 against 624 us: less masked work on the diagonal, finer load balance).
+  if (vi < 0 && !a.causal && S >= 2048 && bh * ((S + 255) / 256) >= 2 * cus) vi = member(256, 8, 1);
   if (vi < 0) {
     for (int i = 0; i < attention_variant_count(); ++i)
       if (attention_variant(i).feasible(a)) {

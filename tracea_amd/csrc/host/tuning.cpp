@@ -237,6 +237,7 @@ PipelineConfig config_for_attention_variant(int index) {
   c.softmax_granularity = "PerTile";
   c.double_buffer = true;
   c.bank_conflict_padding = 0;
+  c.fusion_count = (uint32_t)v.items;  // tiles of the output a workgroup takes (src/optimizer/benchmark.rs:131-132)
   return c;
 }
 
@@ -246,6 +247,7 @@ int attention_variant_for_config(const PipelineConfig &c, const AttentionArgs &a
     if ((uint32_t)v.block_q != c.m_tile || (uint32_t)v.stages != c.num_stages) continue;
     if (c.has_force_num_warps && (uint32_t)v.waves != c.force_num_warps) continue;
     if ((c.intrinsic_shape == "M16N16K4") != (v.mfma == 16)) continue;
+    if ((uint32_t)v.items != (c.fusion_count > 1 ? c.fusion_count : 1u)) continue;
     if (v.feasible(a)) return i;
   }
   return -1;
