@@ -424,8 +424,6 @@ int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split,
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
   const long long cus = device_limits().cus;
-  static const int exp_min = getenv("TRACEA_EXP_MIN") ? atoi(getenv("TRACEA_EXP_MIN")) : 0;
-  if (exp_min > 0) min_tiles = exp_min;
   if (conv_only(v) || tiles * 2 > cus || nk < 2 * min_tiles) return 1;
   long long splits = cus / tiles;
   if (splits > nk / min_tiles) splits = nk / min_tiles;  // at least min_tiles K tiles per range
