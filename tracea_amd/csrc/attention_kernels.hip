@@ -444,6 +444,12 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 
   int q_wave0 = q0 + wave * WQ;
   int q_mine[QB];  // this lane's query in each of the wave's blocks of 32
+  // The last key this lane's scores may keep (the query itself under a causal mask, else the end of the
+  // sequence), less the lane half's offset inside a group of 8 keys: an edge tile then masks element e with one
+  // comparison of a constant against last_key - kv0 (two comparisons, index arithmetic and their scalar
+  // combination per element cost an edge tile 1.55 times the vector instructions of an interior one).
+  int last_key[QB];
+  int wave_last_key;  // (wave-uniform) the last key any query of the wave may keep
   u32x4 qf[QB][KS];
   auto load_q = [&](int first_query, u32x4 (&dst)[QB][KS]) __attribute__((always_inline)) {
 #pragma unroll
@@ -456,7 +462,11 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     }
   };
 #pragma unroll
-  for (int qi = 0; qi < QB; ++qi) q_mine[qi] = q_wave0 + qi * 32 + lrow;
+  for (int qi = 0; qi < QB; ++qi) {
+    q_mine[qi] = q_wave0 + qi * 32 + lrow;
+    last_key[qi] = (a.causal && q_mine[qi] < S - 1 ? q_mine[qi] : S - 1) - g * 4;
+  }
+  wave_last_key = a.causal && q0 + (wave_u + 1) * WQ - 1 < S - 1 ? q0 + (wave_u + 1) * WQ - 1 : S - 1;
   load_q(q0, qf);
 
   auto k_piece = [&](int row, int c) __attribute__((always_inline)) -> int {
@@ -574,11 +584,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
-          if constexpr (EDGE) {
-            const int kv = kv0 + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-            const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine[qi]));
-            s[qi][blk][e] = dead ? -INFINITY : s[qi][blk][e];
-          }
+          if constexpr (EDGE) s[qi][blk][e] = blk * 32 + (e >> 2) * 8 + (e & 3) > last_key[qi] - kv0 ? -INFINITY : s[qi][blk][e];
           mx = fmaxf(mx, s[qi][blk][e]);
         }
       mx = max_with_lane_xor32(mx);
@@ -744,11 +750,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int idx = kk * 8 + j, blk = idx >> 4, e = idx & 15;
-            if constexpr (EDGE) {
-              const int kv = kv0n + blk * 32 + (e >> 2) * 8 + g * 4 + (e & 3);
-              const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine[qi]));
-              s_nxt[qi][blk][e] = dead ? -INFINITY : s_nxt[qi][blk][e];
-            }
+            if constexpr (EDGE) s_nxt[qi][blk][e] = blk * 32 + (e >> 2) * 8 + (e & 3) > last_key[qi] - kv0n ? -INFINITY : s_nxt[qi][blk][e];
             mx[qi] = fmaxf(mx[qi], s_nxt[qi][blk][e]);
           }
         if constexpr (QB > 1) MfmaValu<0, DB * QB, (8 * QB * (EDGE ? 4 : 1) + DB * QB - 1) / (DB * QB), 2 * DB>::run();
@@ -768,16 +770,46 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       for (int blk = 0; blk < 2; ++blk) s_cur[qi][blk] = s_nxt[qi][blk];
   };
 
+  // The iteration of the last tile any query of the wave may keep: its exponentials and its P.V product.
+  // The tile after it has no key for this wave: no score product and no maximum.
+  auto last_live_iteration = [&](int t) __attribute__((always_inline)) {
+    const unsigned char *sV = sVbase + ((tb + t) % NSTG) * TILE_BYTES;
+#pragma unroll
+    for (int qi = 0; qi < QB; ++qi) {
+      float lsum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        float p[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[qi][w >> 1][(w & 1) * 8 + j], a.scale_log2, -m_run[qi]));
+          lsum += p[j];
+        }
+        pf[qi][w] = pack8<DT>(p);
+      }
+      l_run[qi] = l_run[qi] * alpha[qi] + lsum;
+    }
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int d = 0; d < DB; ++d) {
+        const u32x4 vf = read_v(sV, kk, d);
+#pragma unroll
+        for (int qi = 0; qi < QB; ++qi) o[qi][d] = Mfma32<DT>::run(vf, pf[qi][kk], o[qi][d]);
+      }
+  };
 #pragma unroll 1
   for (item = 0; item < ITEMS; ++item) {
   if constexpr (ITEMS > 1) {
     if (item > 0) {
       q0 = item_block(item) * BQ;
       q_wave0 = q0 + wave * WQ;
+      wave_last_key = a.causal && q0 + (wave_u + 1) * WQ - 1 < S - 1 ? q0 + (wave_u + 1) * WQ - 1 : S - 1;
       ntiles = tiles_of(q0);
 #pragma unroll
       for (int qi = 0; qi < QB; ++qi) {
         q_mine[qi] = q_wave0 + qi * 32 + lrow;
+        last_key[qi] = (a.causal && q_mine[qi] < S - 1 ? q_mine[qi] : S - 1) - g * 4;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) qf[qi][ks] = qf_next[qi][ks];
       }
@@ -826,12 +858,39 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
     iteration(t, std::false_type{});
   }
-  for (; t < ntiles; ++t) {
+  if constexpr (EARLY_MAX) {
+    // A tile none of whose keys any query of this wave may keep -- the one after the last, and under a causal
+    // mask the tiles past the wave's diagonal -- gets no score product, no maximum, no exponentials and no P.V
+    // product: full iterations while tile t+1 has a key for the wave, the softmax and P.V of the last such
+    // tile, and then only the workgroup's barriers and tile requests.  (Per block of 128 queries under a
+    // causal mask that is one and a half iterations of two of the four waves and half an iteration of the others.)
+    const int last_live = wave_last_key / FA_BKV;
+    for (; t < last_live; ++t) {
+      __builtin_amdgcn_s_waitcnt(WAIT_TILES);
+      __syncthreads();
+      load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
+      load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
+      iteration(t, std::true_type{});
+    }
     __builtin_amdgcn_s_waitcnt(WAIT_TILES);
     __syncthreads();
     load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
     load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
-    iteration(t, std::true_type{});
+    last_live_iteration(t);
+    for (++t; t < ntiles; ++t) {
+      __builtin_amdgcn_s_waitcnt(WAIT_TILES);
+      __syncthreads();
+      load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
+      load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
+    }
+  } else {
+    for (; t < ntiles; ++t) {
+      __builtin_amdgcn_s_waitcnt(WAIT_TILES);
+      __syncthreads();
+      load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
+      load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
+      iteration(t, std::true_type{});
+    }
   }
   if constexpr (ITEMS > 1) {
     // O from registers: the lanes of the two halves of the wave hold head-dim values 0..3 and 4..7 of a group
