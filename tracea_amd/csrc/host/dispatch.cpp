@@ -424,6 +424,7 @@ int choose_split(const ContractionVariant &v, int M, int N, int K, int *k_split,
   const long long tiles = (long long)((M + v.bm - 1) / v.bm) * ((N + v.bn - 1) / v.bn);
   const int nk = (K + v.bk - 1) / v.bk;
   const long long cus = device_limits().cus;
+  if (v.bk >= 128 && min_tiles == 4) min_tiles = 2;  // (a range is at least 256 deep, whatever the K tile)
   if (conv_only(v) || tiles * 2 > cus || nk < 2 * min_tiles) return 1;
   long long splits = cus / tiles;
   if (splits > nk / min_tiles) splits = nk / min_tiles;  // at least min_tiles K tiles per range
@@ -467,6 +468,11 @@ int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig) {
     // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
+    // K tiles of 128: a row of an operand tile is 256 contiguous bytes instead of 128, which memory beyond the L2
+    // delivers better.  Replayed graphs, K-tile 64 -> 128: M 6272 N 256 K 2304 (ResNet's 14x14 stage at batch 32)
+    // 22.3-23.4 -> 17.8-18.4 us, M 1568 N 512 K 4608 (the 7x7 stage) 37.8-40.3 -> 26.3-31.3; from K = 1152 up
+    // the deeper tile wins on 64x64 and 128x64 tiles, from 2304 up on 128x128; below it is level or 3 % behind.
+    if (v.bk == 128) prior *= k >= (v.bm * v.bn >= 128 * 128 ? 2048 : 1024) ? 1.2 : 0.95;
     // The same loop on 16x16x32 MFMAs.  Measured against the 32x32x16 twin (replayed graphs, same box):
     // 256x256 tiles on four waves 104.2-108.7 us, on eight 107.7-110.3, against 116.1-119.6 at 4096^3;
     // 128x128 tiles 5 % faster at 4096^3, 8 % slower at 2048^3, 27 % slower at 1024^3; 128x64 tiles slower
