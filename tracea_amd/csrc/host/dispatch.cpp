@@ -468,11 +468,17 @@ int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig) {
     // one, direct-to-LDS loads a further ~10 %, eight waves ~4 % over four
     prior *= v.pipeline == 2 ? 1.5 : (v.pipeline == 1 ? 1.35 : (v.pipeline == 3 ? 1.25 : 1.0));
     if (v.waves_m * v.waves_n == 8) prior *= 1.04;
+    // (256x64 tiles on four waves of 64x64: never the best member in the sweeps over GEMM and ResNet layer shapes,
+    // and 74.5 us against 47.2 for 128x64 tiles where the reuse term preferred it: N32 224x224 8->64 7x7 s2)
+    if (v.bm == 256 && v.bn == 64 && v.waves_m * v.waves_n == 4) prior *= 0.85;
     // K tiles of 128: a row of an operand tile is 256 contiguous bytes instead of 128, which memory beyond the L2
     // delivers better.  Replayed graphs, K-tile 64 -> 128: M 6272 N 256 K 2304 (ResNet's 14x14 stage at batch 32)
     // 22.3-23.4 -> 17.8-18.4 us, M 1568 N 512 K 4608 (the 7x7 stage) 37.8-40.3 -> 26.3-31.3; from K = 1152 up
     // the deeper tile wins on 64x64 and 128x64 tiles, from 2304 up on 128x128; below it is level or 3 % behind.
-    if (v.bk == 128) prior *= k >= (v.bm * v.bn >= 128 * 128 ? 2048 : 1024) ? 1.2 : 0.95;
+    // Only where a CU has one workgroup anyway: with more workgroups than CUs the doubled LDS footprint costs
+    // the co-resident workgroups that hide each other's waits (2048^3 on 128x64 tiles 33.4 us against 23.4-24,
+    // 1024x4096x1024 17.9 against 13.1).
+    if (v.bk == 128) prior *= units <= cus && k >= (v.bm * v.bn >= 128 * 128 ? 2048 : 1024) ? 1.2 : 0.85;
     // The same loop on 16x16x32 MFMAs.  Measured against the 32x32x16 twin (replayed graphs, same box):
     // 256x256 tiles on four waves 104.2-108.7 us, on eight 107.7-110.3, against 116.1-119.6 at 4096^3;
     // 128x128 tiles 5 % faster at 4096^3, 8 % slower at 2048^3, 27 % slower at 1024^3; 128x64 tiles slower
