@@ -35,6 +35,8 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
@@ -1402,6 +1404,17 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int RPI = 64 / LPR;                    // rows per pass
   constexpr int STAGING_FLOATS = WM * WN * 32 * EP_PITCH;
   static_assert((size_t)(STAGING_FLOATS + TAB_ENTRIES) * 4 <= (size_t)NS * STAGE, "staging and operand table must fit");
+  // A 16x16x32 tile with nothing to apply leaves from registers.  A lane holds channels 4q .. 4q+3 (q = lane >> 4)
+  // of row lane & 15 of each 16x16 block; one v_permlane16_swap per packed register between two neighbouring
+  // blocks gives every lane 8 consecutive channels of its row (the lanes of 16-lane group q end up with
+  // channels 0-7, 16-23, 8-15, 24-31 of the 32-column pair), i.e. one 16-byte store, with the same
+  // round-to-nearest conversion as the staged rows.  Staging the whole tile in fp32 moves 512 KB through
+  // LDS at 128 bytes per clock on a CU that has nothing else to run: 8.1 k cycles from the last barrier to
+  // the end of the kernel with the stores taken out, 11.2 k with them.  (Decided per block of 32 rows, inside
+  // the loop below: as a path of its own in front of the loop it cost the register allocation a hundred spills.)
+  // (four-wave kernels: the eight-wave 256x256 member has 256 registers and spills 16 with this path in it)
+  constexpr bool REG_EPILOGUE = MS == 16 && !CONV && WM * WN == 4;
+  const bool from_registers = REG_EPILOGUE && simple && plan.n_ops == 0 && args.out_dtype == DT;
   float *stage = (float *)smem + wave * (32 * EP_PITCH);
   float *table = (float *)smem + STAGING_FLOATS;
   const int er = lane / LPR, ec = (lane % LPR) * 8;
@@ -1420,6 +1433,39 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   const long long om_img = args.o_img;
   static_for<0, FM>([&](auto blk) {
     constexpr int i = decltype(blk)::value;
+    if constexpr (REG_EPILOGUE) {
+      if (from_registers) {
+        const int q = lane >> 4;
+        unsigned short *cbase = (unsigned short *)args.C + n0 + wn * TN + (q & 1) * 16 + (q >> 1) * 8;
+        auto pack2 = [](float x, float y) __attribute__((always_inline)) -> unsigned {
+          if constexpr (DT == DT_F16) {
+            const f16x2 h = {(_Float16)x, (_Float16)y};
+            return __builtin_bit_cast(unsigned, h);
+          } else {
+            const bf16x2 h = {(__bf16)x, (__bf16)y};
+            return __builtin_bit_cast(unsigned, h);
+          }
+        };
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          const int m = m0 + wm * TM + i * 32 + h * 16 + (lane & 15);
+          unsigned short *crow = cbase + (zrow + m) * args.ldc;
+#pragma unroll
+          for (int j = 0; j < FN; ++j) {
+            const f32x4 a4 = acc16[2 * i + h][2 * j], b4 = acc16[2 * i + h][2 * j + 1];
+            unsigned a_lo = pack2(a4[0], a4[1]), a_hi = pack2(a4[2], a4[3]);
+            unsigned b_lo = pack2(b4[0], b4[1]), b_hi = pack2(b4[2], b4[3]);
+            // (as instructions: the compiler's builtin for the swap returns its first result twice; the s_nop
+            // is the wait the hardware asks for between a vector-ALU write of an operand and the swap)
+            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a_lo), "+v"(b_lo));
+            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a_hi), "+v"(b_hi));
+            const u32x4 row8 = {a_lo, a_hi, b_lo, b_hi};
+            if (m < M) *(u32x4 *)(crow + j * 32) = row8;
+          }
+        }
+        return;
+      }
+    }
     static_for<0, FN>([&](auto col) {
       constexpr int j = decltype(col)::value;
       if constexpr (MS == 16) {
