@@ -892,9 +892,11 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       iteration(t, std::true_type{});
     }
   }
-  if constexpr (ITEMS > 1) {
+  {
     // O from registers: the lanes of the two halves of the wave hold head-dim values 0..3 and 4..7 of a group
-    // of 8; one swap per register between the halves gives every lane 16 bytes of one row.
+    // of 8; one swap per register between the halves gives every lane 16 bytes of one row.  (No staging in
+    // LDS: it would lie under the tiles a later item has in flight, it cost a wait, two barriers and the bank
+    // conflicts of 8-byte writes at a row pitch -- 10 to 18 % of the kernel's LDS cycles -- per block.)
 #pragma unroll
     for (int qi = 0; qi < QB; ++qi) {
       const float l_tot = l_run[qi] + __shfl_xor(l_run[qi], 32, 64);
@@ -926,52 +928,15 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         }
     }
     tb += ntiles;
-  } else {
-  __builtin_amdgcn_s_waitcnt(0x0f70);  // look-ahead loads must not land on the output staging
-  __syncthreads();
-
-  unsigned char *so = smem + wave * (WQ * ROW_BYTES);
-#pragma unroll
-  for (int qi = 0; qi < QB; ++qi) {
-    const float l_tot = l_run[qi] + __shfl_xor(l_run[qi], 32, 64);
-    const float inv_l = 1.0f / l_tot;
-#pragma unroll
-    for (int d = 0; d < DB; ++d)
-#pragma unroll
-      for (int v4 = 0; v4 < 4; ++v4) {
-        float x[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) x[e] = o[qi][d][v4 * 4 + e] * inv_l;
-        u32x2 w;
-        if constexpr (DT == DT_F16) {
-          f16x4 hq = {(_Float16)x[0], (_Float16)x[1], (_Float16)x[2], (_Float16)x[3]};
-          w = __builtin_bit_cast(u32x2, hq);
-        } else {
-          bf16x4 hq = {(__bf16)x[0], (__bf16)x[1], (__bf16)x[2], (__bf16)x[3]};
-          w = __builtin_bit_cast(u32x2, hq);
-        }
-        *(u32x2 *)(so + (qi * 32 + lrow) * ROW_BYTES + (d * 32 + v4 * 8 + g * 4) * 2) = w;
-      }
-  }
-  __syncthreads();
-#pragma unroll
-  for (int i = 0; i < WQ * CH / 64; ++i) {
-    const int p = lane + i * 64;
-    const int row = p / CH, c = p % CH;
-    const int q = q_wave0 + row;
-    if (q < S)
-      *(u32x4 *)(Og + (long long)q * a.o_ss + c * 8) = *(const u32x4 *)(so + row * ROW_BYTES + c * 16);
-  }
   }
   }  // items
   // (the last item's look-ahead requests write LDS: they must have landed before the workgroup gives it up)
-  if constexpr (ITEMS > 1) __builtin_amdgcn_s_waitcnt(0x0f70);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 
 template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1, int ITEMS = 1>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
-  constexpr size_t ring = 2 * (size_t)NSTG * FA_BKV * D * 2, staging = ITEMS > 1 ? 0 : (size_t)WAVES * 32 * QB * D * 2;
-  constexpr size_t lds = ring > staging ? ring : staging;
+  constexpr size_t lds = 2 * (size_t)NSTG * FA_BKV * D * 2;  // the K and V rings; O leaves from registers
   const int nqb = (a.S + 32 * QB * WAVES - 1) / (32 * QB * WAVES);
   if (nqb % ITEMS != 0) return (int)hipErrorInvalidValue;  // (feasible_pairs keeps such a call away)
   const dim3 grid((unsigned)(nqb / ITEMS * a.B * a.H)), block(WAVES * 64);
