@@ -584,6 +584,22 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   static_assert(!B_NCONTIG || (NT % (BN / 8) == 0), "bad BN for N-contiguous B");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  // Everything the prologue reads from the kernel arguments, asked for HERE in one batch of scalar loads.
+  // Left to itself the compiler loads each field where it is first used, behind the branch that needs it:
+  // eight or more dependent round trips to the scalar cache's backing memory in front of the first tile
+  // request (4.1 k cycles from kernel entry to that request in the 4096^3 launch).
+  // (Not in the eight-wave 256x256 kernels: at 256 registers a wave they have none to hold the batch in.)
+  constexpr bool BATCH_ARGS = !(WM * WN == 8 && BM * BN >= 256 * 256);
+  if constexpr (BATCH_ARGS)
+  asm volatile("" ::"s"(args.A), "s"(args.B), "s"(args.M), "s"(args.N), "s"(args.K), "s"(args.lda), "s"(args.ldb),
+               "s"(args.a_bytes), "s"(args.b_bytes), "s"(args.grid_m), "s"(args.grid_n), "s"(args.k_split),
+               "s"(args.fuse_ws), "s"(args.group_m), "s"(args.tile_list), "s"(args.epi.n_ops));
+  if constexpr (CONV && BATCH_ARGS) {
+    asm volatile("" ::"s"(args.h_in), "s"(args.w_in), "s"(args.c_in), "s"(args.h_out), "s"(args.w_out), "s"(args.s_sz),
+                 "s"(args.stride_h), "s"(args.stride_w), "s"(args.pad_h), "s"(args.pad_w), "s"(args.dil_h), "s"(args.dil_w),
+                 "s"(args.hw_m), "s"(args.hw_s), "s"(args.w_m), "s"(args.w_s), "s"(args.sc_m), "s"(args.sc_s),
+                 "s"(args.c_m), "s"(args.c_s), "s"(args.phases));
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
