@@ -460,6 +460,9 @@ int launch_gemm_generic(const GenericGemmArgs &a, hipStream_t stream) {
 // ---------------------------------------------------------------------------
 template <int V>
 __global__ void __launch_bounds__(256) splitk_reduce_kernel(const SplitKReduceArgs a) {
+  // (every argument of the prologue in one batch of scalar loads instead of one round trip per field)
+  asm volatile("" ::"s"(a.partial), "s"(a.out), "s"(a.out_dtype), "s"(a.splits), "s"(a.M), "s"(a.N), "s"(a.ldc),
+               "s"(a.tile_counts), "s"(a.epi.n_ops));
   const int groups = (a.N + V - 1) / V;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (long long)a.M * groups) return;
