@@ -126,6 +126,36 @@ def test_members_on_16x16x32_mfmas(tracea_gpu):
     assert not capi.last_variant("gemm").endswith("_m16")
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_tiles_stored_from_registers_equal_the_staged_rows(tracea_gpu, dtype):
+    """With an empty chain the four-wave members on 16x16x32 MFMAs store a tile from registers (a lane swap
+    per packed register pair) instead of staging it in LDS.  Adding a bias of zeros forces the staged rows:
+    the two outputs must be equal element for element, on full tiles, on a tile cut by the end of M, and on
+    both layouts of B."""
+    from tracea_amd import capi
+    tdt, rnd = (torch.float16, round_f16) if dtype == "f16" else (torch.bfloat16, round_bf16)
+    names = capi.variants("gemm")
+    members = [nm for nm in names if nm.endswith("_m16") and "w2x4" not in nm]
+    assert members
+    rng = np.random.default_rng(5)
+    try:
+        for (m, n, k) in [(512, 512, 320), (300, 768, 200)]:
+            a = _dev(rnd(rng.standard_normal((m, k)) / np.sqrt(k)), tdt)
+            bt = _dev(rnd(rng.standard_normal((n, k))), tdt)
+            zeros = torch.zeros(n, device="cuda", dtype=torch.float32)
+            ref = oracle.gemm_f64(a.float().cpu().numpy(), bt.float().cpu().numpy().T)
+            for nm in members:
+                capi.force_variant("gemm", nm)
+                for b in (bt.t(), bt.t().contiguous()):
+                    plain = tracea_gpu.gemm(a, b)
+                    assert capi.last_variant("gemm") == nm
+                    staged = tracea_gpu.gemm_ex(a, b, [(capi.OP_BIAS_ADD, zeros)])
+                    assert torch.equal(plain, staged), "%s (%d, %d, %d)" % (nm, m, n, k)
+                    assert_close_scaled(plain.float().cpu().numpy(), ref, tol_half(k, dtype), nm)
+    finally:
+        capi.force_variant("gemm", -1)
+
+
 def test_epilogue_kinds_match_oracle_chain(tracea_gpu):
     # operator order of src/interface/c_bindings.rs:144-197, functors of epilogue.cuh
     m, n, k = 256, 320, 256
