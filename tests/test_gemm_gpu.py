@@ -117,13 +117,14 @@ def test_members_on_16x16x32_mfmas(tracea_gpu):
                     assert_close_scaled(c.float().cpu().numpy(), c_t.float().cpu().numpy(), 2.0 ** -10, nm + " vs twin")
     finally:
         capi.force_variant("gemm", -1)
-    # the default for a large product with a K-contiguous B is a 16x16x32 member; an N-contiguous B stays on 32x32x16
-    big = torch.randn(4096, 512, device="cuda").half()
-    wide = torch.randn(4096, 512, device="cuda").half()
+    # the default for a large product is a 16x16x32 member: four waves for a K-contiguous B, eight for an
+    # N-contiguous one (twice the B fragments per wave on four)
+    big = torch.randn(4096, 4096, device="cuda").half()
+    wide = torch.randn(4096, 4096, device="cuda").half()
     tracea_gpu.gemm(big, wide.t())
-    assert capi.last_variant("gemm").endswith("_m16")
+    assert capi.last_variant("gemm") == "t256x256x64_w2x2_p2_m16"
     tracea_gpu.gemm(big, wide.t().contiguous())
-    assert not capi.last_variant("gemm").endswith("_m16")
+    assert capi.last_variant("gemm") == "t256x256x64_w2x4_p2_m16"
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

@@ -915,12 +915,41 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       tr_off16[j] = row * NB_ROWB + (((col >> 3) ^ nb_swz(row)) << 4) + (col & 7) * 2;
     }
   }
+  // The two transposing reads are written as instructions.  Through the builtin the compiler puts a
+  // vmcnt(0) in front of every one of them that follows a direct-to-LDS tile request (it cannot tell that the
+  // request writes the other stage), and the k-step behind the barrier, where requests and reads alternate,
+  // took 5600 cycles instead of 1200.  As instructions they are outside its bookkeeping altogether: the
+  // fragments are complete only after wait_b_tr below, which the MFMAs depend on through its operands.
+  // (The hardware counts them like any LDS read, so the full LDS wait the compiler places in front of a
+  // barrier covers them too.)
   auto read_b_tr16 = [&](const unsigned char *sB, int j, int ks) -> u32x4 {
-    const unsigned char *p = sB + tr_off16[j] + ks * 32 * NB_ROWB;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)p);
-    const s16x4 hi =
-        __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(p + 4 * NB_ROWB));
-    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+    const unsigned addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)(sB + tr_off16[j] + ks * 32 * NB_ROWB);
+    u32x2 lo2, hi2;
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo2) : "v"(addr) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi2) : "v"(addr), "i"(4 * NB_ROWB) : "memory");
+    u32x4 v;
+    v[0] = lo2[0]; v[1] = lo2[1]; v[2] = hi2[0]; v[3] = hi2[1];
+    return v;
+  };
+  constexpr int TR_FRAGS = (MS == 16 ? 2 : 1) * FN;  // B fragments of a k-step
+  auto wait_b_tr = [&](u32x4 (&f)[TR_FRAGS]) __attribute__((always_inline)) {
+    static_assert(TR_FRAGS == 1 || TR_FRAGS == 2 || TR_FRAGS == 4 || TR_FRAGS == 8, "fragments of a k-step");
+    if constexpr (TR_FRAGS == 1)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]));
+    else if constexpr (TR_FRAGS == 2)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]));
+    else if constexpr (TR_FRAGS == 4)
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]));
+    else
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(f[0]), "+v"(f[1]), "+v"(f[2]), "+v"(f[3]), "+v"(f[4]), "+v"(f[5]), "+v"(f[6]), "+v"(f[7]));
+  };
+  // (the same for the 32x32x16 fragments of the direct-to-LDS loop)
+  auto read_b_tr_asm = [&](const unsigned char *sB, int j, int ks) -> u32x4 {
+    const unsigned addr = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)(sB + tr_off[j] + ks * 16 * NB_ROWB);
+    u32x2 lo2, hi2;
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo2) : "v"(addr) : "memory");
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi2) : "v"(addr), "i"(4 * NB_ROWB) : "memory");
     u32x4 v;
     v[0] = lo2[0]; v[1] = lo2[1]; v[2] = hi2[0]; v[3] = hi2[1];
     return v;
@@ -1145,7 +1174,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         for (int i = 0; i < FM; ++i) fa[set][i] = *(const u32x4 *)(pa + i * 32 * ROW_BYTES + coff);
 #pragma unroll
         for (int j = 0; j < FN; ++j) {
-          if constexpr (B_NCONTIG) fb[set][j] = read_b_tr(sB, j, ks);
+          if constexpr (B_NCONTIG) fb[set][j] = read_b_tr_asm(sB, j, ks);
           else fb[set][j] = *(const u32x4 *)(pb + j * 32 * ROW_BYTES + coff);
         }
       }
@@ -1173,6 +1202,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       }
     };
     auto mma = [&](int set) {
+      if constexpr (B_NCONTIG) wait_b_tr(fb[set]);
       if constexpr (MS == 16) {
 #pragma unroll
         for (int i = 0; i < 2 * FM; ++i)

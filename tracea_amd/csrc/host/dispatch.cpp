@@ -487,10 +487,12 @@ int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig) {
     // 36.3 against 35.0 at 4096x4096x1024 (the four-wave factor also undoes the few-waves penalty below).
     if (v.mfma == 16) prior *= v.bm * v.bn >= 256 * 256 ? (v.waves_m * v.waves_n == 4 ? (k >= 2048 ? 1.35 : 1.2) : 1.06) : 0.9;
     // An N-contiguous B is fetched with two transposing LDS reads per fragment, and four waves have twice the
-    // B fragments of eight.  4096^3 with this layout, operands N(0,1)/sqrt(K), stream launches: eight waves on
-    // 32x32x16 115-118 us, eight on 16x16x32 128-132, four on 16x16x32 209 (the library GEMM itself 113 us):
-    // the 32x32x16 eight-wave member runs this layout.
-    if (b_ncontig && !conv && v.bm * v.bn >= 256 * 256 && (v.waves_m * v.waves_n == 4 || v.mfma == 16)) prior *= 0.8;
+    // B fragments of eight.  4096^3 with this layout, operands N(0,1)/sqrt(K), replayed graphs, one box: eight
+    // waves on 16x16x32 112.6 us, eight on 32x32x16 116.2-119.8, four on 16x16x32 129.6 (the library GEMM itself
+    // 107.8): the eight-wave 16x16x32 member runs this layout.  (Before the transposing reads were written as
+    // instructions the compiler put a vmcnt(0) in front of each one that followed a tile request: 128-132 and
+    // 209 us for the two 16x16x32 members.)
+    if (b_ncontig && !conv && v.bm * v.bn >= 256 * 256 && v.waves_m * v.waves_n == 4) prior *= 0.8;
     {
       // A CU with fewer than 8 resident waves (one 4-wave workgroup, the launch too small or
       // the tile's LDS too large for a second) hides less latency.  The fourth root is fitted
