@@ -1258,7 +1258,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         else Interleave<0, R, 0x100, D, 0x100, 0>::run();
         __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): tile kt+1 has landed
+      // vmcnt(0): tile kt+1 has landed.  (With an N-contiguous B also lgkmcnt(0): the transposing reads of `cur`
+      // issued in front of this barrier are instructions the compiler does not count, and they must have
+      // executed before another wave's requests may overwrite `cur`.)
+      __builtin_amdgcn_s_waitcnt(B_NCONTIG ? 0x0070 : 0x0f70);
       __syncthreads();
       // every wave has finished reading `cur`: request the first share of tile
       // kt+2 into it (clamped to the last tile, whose second copy is never read)
