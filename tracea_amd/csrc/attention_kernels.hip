@@ -659,7 +659,10 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // branch-free up to the optional rescale, so MFMAs and vector-ALU work can be
   // interleaved instruction by instruction.  For EARLY_MAX the tag describes
   // tile t+1, the one whose maximum the iteration takes.
-  auto iteration = [&](int t, auto edge_tag) __attribute__((always_inline)) {
+  // cur / nxt: the score arrays of tile t (read) and tile t+1 (written); with copy_tag the new scores are
+  // moved into cur at the end, without it the caller swaps the roles of the two arrays for the next tile
+  // (the interior loop does, two tiles per trip: the move is 16 of a tile's 165 vector instructions).
+  auto iteration_on = [&](int t, auto edge_tag, f32x16 (&cur)[QB][2], f32x16 (&nxt)[QB][2], auto copy_tag) __attribute__((always_inline)) {
     const unsigned char *sV = sVbase + ((tb + t) % NSTG) * TILE_BYTES;
     if constexpr (!EARLY_MAX) {
       const bool moved = take_max(t, edge_tag, s_cur);
@@ -701,14 +704,14 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         for (int qi = 0; qi < QB; ++qi) {
           // (the first k-step starts from the MFMA's constant zero: no 32 registers to clear per tile)
           const f32x16 zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-          s_nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], ks == 0 ? zero16 : s_nxt[qi][0]);
-          s_nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], ks == 0 ? zero16 : s_nxt[qi][1]);
+          nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], ks == 0 ? zero16 : nxt[qi][0]);
+          nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], ks == 0 ? zero16 : nxt[qi][1]);
         }
 #pragma unroll
         for (int j = 0; j < EPC; ++j) {
           const int idx = ks * EPC + j;  // 0..32*QB-1 over (query block, blk, element): block idx/32, blk (idx%32)/16
           const int qi = idx >> 5, w = idx & 31;
-          const float x = __builtin_amdgcn_exp2f(fmaf(s_cur[qi][w >> 4][w & 15], a.scale_log2, -m_run[qi]));
+          const float x = __builtin_amdgcn_exp2f(fmaf(cur[qi][w >> 4][w & 15], a.scale_log2, -m_run[qi]));
           p[idx & 7] = x;
           lsum[qi] += x;
           if ((idx & 7) == 7) pf[qi][w >> 3] = pack8<DT>(p);
@@ -750,8 +753,8 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) {
             const int idx = kk * 8 + j, blk = idx >> 4, e = idx & 15;
-            if constexpr (EDGE) s_nxt[qi][blk][e] = blk * 32 + (e >> 2) * 8 + (e & 3) > last_key[qi] - kv0n ? -INFINITY : s_nxt[qi][blk][e];
-            mx[qi] = fmaxf(mx[qi], s_nxt[qi][blk][e]);
+            if constexpr (EDGE) nxt[qi][blk][e] = blk * 32 + (e >> 2) * 8 + (e & 3) > last_key[qi] - kv0n ? -INFINITY : nxt[qi][blk][e];
+            mx[qi] = fmaxf(mx[qi], nxt[qi][blk][e]);
           }
         if constexpr (QB > 1) MfmaValu<0, DB * QB, (8 * QB * (EDGE ? 4 : 1) + DB * QB - 1) / (DB * QB), 2 * DB>::run();
         __builtin_amdgcn_sched_barrier(0);
@@ -764,10 +767,16 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       }
       rescale(moved);
     }
+    if constexpr (decltype(copy_tag)::value) {
 #pragma unroll
-    for (int qi = 0; qi < QB; ++qi)
+      for (int qi = 0; qi < QB; ++qi)
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk) s_cur[qi][blk] = s_nxt[qi][blk];
+        for (int blk = 0; blk < 2; ++blk) cur[qi][blk] = nxt[qi][blk];
+    }
+  };
+  // (the form every caller but the interior loop uses: scores of tile t in s_cur on entry, of tile t+1 on exit)
+  auto iteration = [&](int t, auto edge_tag) __attribute__((always_inline)) {
+    iteration_on(t, edge_tag, s_cur, s_nxt, std::true_type{});
   };
 
   // The iteration of the last tile any query of the wave may keep: its exponentials and its P.V product.
@@ -851,12 +860,31 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   int t = 0;
   // The barrier at the head of iteration t publishes K(t+1) and V(t) and retires K(t) and V(t-1),
   // whose stages then receive K(t+NSTG) and V(t+NSTG-1).
-  for (; t < interior_end; ++t) {
-    __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(t+1) and V(t), requested NSTG-1 iterations ago
+  auto head_of = [&](int tt) __attribute__((always_inline)) {
+    __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(tt+1) and V(tt), requested NSTG-1 iterations ago
     __syncthreads();
-    load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
-    load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
-    iteration(t, std::false_type{});
+    load_k(ahead(tt + NSTG), sKbase + ((tb + tt) % NSTG) * TILE_BYTES);
+    load_v(ahead(tt + NSTG - 1), sVbase + ((tb + tt + NSTG - 1) % NSTG) * TILE_BYTES);
+  };
+  if constexpr (EARLY_MAX && QB == 1) {
+    // an odd tile first, then two per trip with the score arrays changing roles
+    // (one query block per wave: with two the kernel has no register to spare and spills)
+    if (t < interior_end && ((interior_end - t) & 1)) {
+      head_of(t);
+      iteration(t, std::false_type{});
+      ++t;
+    }
+    for (; t < interior_end; t += 2) {
+      head_of(t);
+      iteration_on(t, std::false_type{}, s_cur, s_nxt, std::false_type{});
+      head_of(t + 1);
+      iteration_on(t + 1, std::false_type{}, s_nxt, s_cur, std::false_type{});
+    }
+  } else {
+    for (; t < interior_end; ++t) {
+      head_of(t);
+      iteration(t, std::false_type{});
+    }
   }
   if constexpr (EARLY_MAX) {
     // A tile none of whose keys any query of this wave may keep -- the one after the last, and under a causal
