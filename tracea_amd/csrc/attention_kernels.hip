@@ -662,8 +662,12 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // cur / nxt: the score arrays of tile t (read) and tile t+1 (written); with copy_tag the new scores are
   // moved into cur at the end, without it the caller swaps the roles of the two arrays for the next tile
   // (the interior loop does, two tiles per trip: the move is 16 of a tile's 165 vector instructions).
-  auto iteration_on = [&](int t, auto edge_tag, f32x16 (&cur)[QB][2], f32x16 (&nxt)[QB][2], auto copy_tag) __attribute__((always_inline)) {
-    const unsigned char *sV = sVbase + ((tb + t) % NSTG) * TILE_BYTES;
+  // stage_tag: the ring stage of tile t where the caller knows it at compile time (the interior loop, which
+  // starts its pairs on stage 0 of a two-stage ring), else -1: with a constant stage the LDS addresses of the
+  // K and V fragments are loop invariants plus immediates instead of an addition per read group.
+  auto iteration_on = [&](int t, auto edge_tag, f32x16 (&cur)[QB][2], f32x16 (&nxt)[QB][2], auto copy_tag, auto stage_tag) __attribute__((always_inline)) {
+    constexpr int STG = decltype(stage_tag)::value;
+    const unsigned char *sV = sVbase + (STG >= 0 ? STG : (tb + t) % NSTG) * TILE_BYTES;
     if constexpr (!EARLY_MAX) {
       const bool moved = take_max(t, edge_tag, s_cur);
       rescale(moved);
@@ -680,7 +684,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       // matrix pipe works on its MFMAs, whatever order the compiler gives them
       // inside the chunk.
       constexpr bool EDGE = decltype(edge_tag)::value;
-      const unsigned char *sKn = sKbase + ((tb + t + 1) % NSTG) * TILE_BYTES;
+      const unsigned char *sKn = sKbase + (STG >= 0 ? (STG + 1) % NSTG : (tb + t + 1) % NSTG) * TILE_BYTES;
       // ---- phase A: S^T(t+1) = K(t+1) Q^T  with  P(t) = exp2(S(t)*scale - m), row sums ----
       // chunk ks: the 2*QB MFMAs of k-step ks (operands read one chunk ahead) and
       // 32*QB/KS of the 32*QB exponentials
@@ -776,7 +780,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   };
   // (the form every caller but the interior loop uses: scores of tile t in s_cur on entry, of tile t+1 on exit)
   auto iteration = [&](int t, auto edge_tag) __attribute__((always_inline)) {
-    iteration_on(t, edge_tag, s_cur, s_nxt, std::true_type{});
+    iteration_on(t, edge_tag, s_cur, s_nxt, std::true_type{}, std::integral_constant<int, -1>{});
   };
 
   // The iteration of the last tile any query of the wave may keep: its exponentials and its P.V product.
@@ -867,18 +871,28 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     load_v(ahead(tt + NSTG - 1), sVbase + ((tb + tt + NSTG - 1) % NSTG) * TILE_BYTES);
   };
   if constexpr (EARLY_MAX && QB == 1) {
-    // an odd tile first, then two per trip with the score arrays changing roles
-    // (one query block per wave: with two the kernel has no register to spare and spills)
-    if (t < interior_end && ((interior_end - t) & 1)) {
+    // Two tiles per trip with the score arrays changing roles, and (two-stage rings) the pairs starting on
+    // ring stage 0: a single tile in front if the first one lies on stage 1, a single one behind if one is left.
+    // (One query block per wave: with two the kernel has no register to spare and spills.)
+    // (one-block members only: the four-wave paired kernel at head dimension 128 spills four registers with
+    // the hoisted addresses, and the eight-wave paired kernels measured level with and without)
+    constexpr bool CONST_STAGES = NSTG == 2 && ITEMS == 1;
+    constexpr int S0 = CONST_STAGES ? 0 : -1, S1 = CONST_STAGES ? 1 : -1;
+    if (CONST_STAGES && t < interior_end && ((tb + t) & 1)) {
       head_of(t);
       iteration(t, std::false_type{});
       ++t;
     }
-    for (; t < interior_end; t += 2) {
+    for (; t + 1 < interior_end; t += 2) {
       head_of(t);
-      iteration_on(t, std::false_type{}, s_cur, s_nxt, std::false_type{});
+      iteration_on(t, std::false_type{}, s_cur, s_nxt, std::false_type{}, std::integral_constant<int, S0>{});
       head_of(t + 1);
-      iteration_on(t + 1, std::false_type{}, s_nxt, s_cur, std::false_type{});
+      iteration_on(t + 1, std::false_type{}, s_nxt, s_cur, std::false_type{}, std::integral_constant<int, S1>{});
+    }
+    if (t < interior_end) {
+      head_of(t);
+      iteration(t, std::false_type{});
+      ++t;
     }
   } else {
     for (; t < interior_end; ++t) {
