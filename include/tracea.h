@@ -353,8 +353,10 @@ TraceaStatus tracea_gemm_noalloc(TraceaTensorView a, TraceaTensorView b, const T
 
 /* Kernel-variant control for tuners and benchmarks.  `op` is "gemm", "conv2d"
  * or "attention".  A variant forced with tracea_force_variant (index >= 0) is
- * used by every later call of that operator in the process whenever it is
- * feasible for the problem; -1 restores automatic selection. */
+ * used by every later call of that operator FROM THE CALLING THREAD whenever it
+ * is feasible for the problem (other threads keep their own choice, so a tuner
+ * timing variants does not steer calls made elsewhere in the process); -1
+ * restores automatic selection. */
 int32_t tracea_variant_count(const char *op);
 const char *tracea_variant_name(const char *op, int32_t index); /* library-owned */
 int32_t tracea_force_variant(const char *op, int32_t index);    /* 0 ok, -1 bad argument */

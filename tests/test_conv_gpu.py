@@ -147,23 +147,30 @@ RESIDENT_SHAPES = [  # n, h, w, k, stride, pad, dilation: 64 input channels, 3x3
 ]
 
 
+# the members that keep the input patch in LDS with the filter slab resident beside it or in a ring of taps,
+# and the input channels each is compiled for
+LDS_MEMBERS = [("c448x64_k576_resident", 64), ("c400x64_c64_w16_resident", 64), ("c208x64_c128_s4_w16_patch", 128)]
+
+
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_filter_resident_variant(tracea_gpu, dtype):
-    """The kernel that keeps input patch and filter bank in LDS together (64 filters of 3x3x64),
+@pytest.mark.parametrize("member,cin", LDS_MEMBERS)
+def test_filter_resident_variant(tracea_gpu, dtype, member, cin):
+    """The kernels that keep the input patch in LDS together with the filter slab (or a ring of its taps),
     forced, against the oracle: tile cuts, strides, dilation, padding, partial filter slabs."""
     from tracea_amd import capi
     names = capi.variants("conv2d")
-    vi = [i for i, nm in enumerate(names) if nm.endswith("_resident")]
-    assert vi, "no filter-resident variant in the build"
+    assert member in names, "no member %s in the build" % member
+    vi = [names.index(member)]
     tdt = torch.float16 if dtype == "f16" else torch.bfloat16
     rnd = round_f16 if dtype == "f16" else round_bf16
+    kg = 9 * cin
     capi.force_variant("conv2d", vi[0])
     try:
         for shape in RESIDENT_SHAPES:
             n, h, w, k, stride, pad, dil = shape
             rng = np.random.default_rng(h * 31 + w + k)
-            x = rnd(rng.standard_normal((n, h, w, 64)))
-            wk = rnd(rng.standard_normal((k, 3, 3, 64)) * np.sqrt(2.0 / 576))
+            x = rnd(rng.standard_normal((n, h, w, cin)))
+            wk = rnd(rng.standard_normal((k, 3, 3, cin)) * np.sqrt(2.0 / kg))
             bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
             ref = torch.nn.functional.conv2d(
                 torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
@@ -175,22 +182,24 @@ def test_filter_resident_variant(tracea_gpu, dtype):
                 assert np.abs(want - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
             y = tracea_gpu.conv2d(_dev(x, tdt), _dev(wk, tdt), bias=_dev(bias), stride=stride, padding=pad,
                                   dilation=dil, epilogue="bias+relu")
-            assert capi.last_variant("conv2d") == names[vi[0]], "the resident kernel refused %s" % (shape,)
-            assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(576, dtype), "%s %s" % (dtype, shape))
+            assert capi.last_variant("conv2d") == names[vi[0]], "%s refused %s" % (member, shape)
+            assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(kg, dtype), "%s %s %s" % (member, dtype, shape))
     finally:
         capi.force_variant("conv2d", -1)
 
 
-def test_filter_resident_variant_operator_chains(tracea_gpu):
-    """Every form of its straight-line epilogue ([affine] [ReLU] [residual] [ReLU]) and chains outside it,
-    against the oracle's chain on the oracle's accumulator."""
+@pytest.mark.parametrize("member,cin", LDS_MEMBERS)
+def test_filter_resident_variant_operator_chains(tracea_gpu, member, cin):
+    """Every form of their straight-line epilogue ([affine] [ReLU] [residual] [ReLU]) and chains outside it
+    (SiLU and GELU among them), against the oracle's chain on the oracle's accumulator."""
     from tracea_amd import capi
     names = capi.variants("conv2d")
-    vi = [i for i, nm in enumerate(names) if nm.endswith("_resident")][0]
+    vi = names.index(member)
     n, h, w, k = 2, 18, 25, 64
+    kg = 9 * cin
     rng = np.random.default_rng(77)
-    x = round_f16(rng.standard_normal((n, h, w, 64)))
-    w_rsck = round_f16(rng.standard_normal((3, 3, 64, k)) * np.sqrt(2.0 / 576))
+    x = round_f16(rng.standard_normal((n, h, w, cin)))
+    w_rsck = round_f16(rng.standard_normal((3, 3, cin, k)) * np.sqrt(2.0 / kg))
     acc = oracle.conv2d_nhwc(x, w_rsck, 1, 1, 1)
     bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
     (gamma, beta, mean, var), (scale, shift) = _bn_params(rng, k)
@@ -205,6 +214,7 @@ def test_filter_resident_variant_operator_chains(tracea_gpu):
     relu = ((O.OP_RELU,), (E.EPI_RELU,))
     resid = ((O.OP_RESIDUAL_ADD, dres), (E.EPI_RESIDUAL_ADD, res))
     gelu = ((O.OP_GELU,), (E.EPI_GELU,))
+    silu = ((O.OP_SILU,), (E.EPI_SILU,))
     chains = [[]]
     for a in (None, "bias", "ss", "bn"):                      # the 16 forms (each affine kind once over them)
         for r1 in (False, True):
@@ -214,25 +224,71 @@ def test_filter_resident_variant_operator_chains(tracea_gpu):
                     if c and (a != "bn" or rs):                # keep the list short: BatchNorm with a residual only
                         chains.append(c)
     chains += [[aff["bias16"], relu], [relu, aff["bias"]], [resid, aff["ss"]], [aff["bias"], gelu], [resid, resid, relu],
-               [aff["ss"], aff["bias"], relu]]                # outside the fast form: general path
+               [aff["ss"], aff["bias"], relu], [silu], [aff["bias"], silu], [aff["bn"], silu, resid]]  # outside the fast form: general path
     capi.force_variant("conv2d", vi)
     try:
         for chain in chains:
             want = oracle.epilogue_apply(acc, [c[1] for c in chain])
             y = tracea_gpu.conv2d_ex(dx, dw, [c[0] for c in chain], stride=1, padding=1)
             assert capi.last_variant("conv2d") == names[vi]
-            assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "chain %s" % ([c[1][0] for c in chain],))
+            assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(kg), "%s chain %s" % (member, [c[1][0] for c in chain]))
         # fp32 output and a bf16 residual on f16 operands leave the fast form too
         y = tracea_gpu.conv2d_ex(dx, dw, [aff["bias"][0], relu[0]], stride=1, padding=1, out_dtype=torch.float32)
         want = oracle.epilogue_apply(acc, [aff["bias"][1], relu[1]])
         assert y.dtype == torch.float32
-        assert_close_scaled(y.cpu().numpy(), want, tol_for_k(576), "fp32 output")
+        assert_close_scaled(y.cpu().numpy(), want, tol_for_k(kg), "fp32 output")
         resb = round_bf16(res)
         y = tracea_gpu.conv2d_ex(dx, dw, [(O.OP_RESIDUAL_ADD, _dev(resb, torch.bfloat16)), relu[0]], stride=1, padding=1)
         want = oracle.epilogue_apply(acc, [(E.EPI_RESIDUAL_ADD, resb), relu[1]])
-        assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "bf16 residual on f16 operands")
+        assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(kg), "bf16 residual on f16 operands")
     finally:
         capi.force_variant("conv2d", -1)
+
+
+@pytest.mark.parametrize("kernel", ["t128x64x64_w4x1_p2", "t64x64x64_w2x2_p2", "c256x64_w8x1_s3_patch",
+                                    "c448x64_k576_resident", "c400x64_c64_w16_resident", None])
+def test_conv_silu_kinds_through_tracea_conv2d(tracea_gpu, kernel):
+    """TRACEA_EPILOGUE_SILU and TRACEA_EPILOGUE_BIAS_SILU through tracea_conv2d on the streamed, the
+    patch-resident and the filter-resident kernels (and whatever the selector picks), against
+    oracle.epilogue_apply on the oracle's accumulator (x / (1 + exp(-x)), src/kernels/gpu/epilogue.cuh)."""
+    from tracea_amd import capi
+    rng = np.random.default_rng(0x51)
+    x = round_f16(rng.standard_normal((2, 20, 20, 64)))
+    w_rsck = round_f16(rng.standard_normal((3, 3, 64, 64)) * np.sqrt(2.0 / 576))
+    bias = (rng.standard_normal(64) * 0.5).astype(np.float32)
+    acc = oracle.conv2d_nhwc(x, w_rsck, 1, 1, 1)
+    dx, dw = _dev(x, torch.float16), _dev(w_rsck, torch.float16).permute(3, 0, 1, 2).contiguous()
+    if kernel is not None:
+        capi.force_variant("conv2d", kernel)
+    try:
+        y = tracea_gpu.conv2d(dx, dw, stride=1, padding=1, epilogue="silu")
+        if kernel is not None:
+            assert capi.last_variant("conv2d") == kernel
+        want = oracle.epilogue_apply(acc, [(oracle.EPI_SILU,)])
+        assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "silu on %s" % kernel)
+        y = tracea_gpu.conv2d(dx, dw, bias=_dev(bias), stride=1, padding=1, epilogue="bias+silu")
+        want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_SILU,)])
+        assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(576), "bias+silu on %s" % kernel)
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
+def test_k576_with_other_channel_counts_runs_on_another_kernel(tracea_gpu):
+    """K = 576 with 16 or 32 input channels (6x6 and 3x6 filters): the kernels compiled for 3x3x64 must
+    refuse and the selector's choice must compute it."""
+    from tracea_amd import capi
+    for cin, (r, sz) in ((16, (6, 6)), (32, (3, 6))):
+        rng = np.random.default_rng(cin)
+        x = round_f16(rng.standard_normal((32, 56, 56, cin)))
+        w_rsck = round_f16(rng.standard_normal((r, sz, cin, 64)) * np.sqrt(2.0 / 576))
+        dx, dw = _dev(x, torch.float16), _dev(w_rsck, torch.float16).permute(3, 0, 1, 2).contiguous()
+        y = tracea_gpu.conv2d(dx, dw, stride=1, padding=(1, 2), epilogue="relu")
+        used = capi.last_variant("conv2d")
+        assert used is not None and not used.endswith("_resident"), used
+        ref = torch.relu(torch.nn.functional.conv2d(
+            torch.from_numpy(x[:2]).permute(0, 3, 1, 2).double(), torch.from_numpy(w_rsck).permute(3, 2, 0, 1).double(),
+            padding=(1, 2))).permute(0, 2, 3, 1).numpy()
+        assert_close_scaled(y[:2].float().cpu().numpy(), ref, tol_for_k(576), "C=%d" % cin)
 
 
 def test_asymmetric_stride_and_padding_bf16(tracea_gpu):

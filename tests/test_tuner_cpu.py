@@ -277,7 +277,7 @@ def test_proposed_configs_name_compiled_variants():
         assert all(c["instruction"] == "RocmMFMA" for c in cands)
         # the MFMA shape is part of the search space: 16x16x32 members under the reference's M16N16K4
         shapes = {names[T.variant_for_config(c)]: c["intrinsic_shape"] for c in cands}
-        assert all(sh == ("M16N16K4" if nm.endswith("_m16") else "M32N32K2") for nm, sh in shapes.items())
+        assert all(sh == ("M16N16K4" if nm.endswith("_m16") or "_w16_" in nm else "M32N32K2") for nm, sh in shapes.items())
         assert sum(nm.endswith("_m16") for nm in shapes) >= 3
     first = T.propose_gemm_configs(4096, 4096, 4096)[0]
     assert T.variant_for_config(first) == capi.lib().tracea_select_variant(b"gemm", 4096, 4096, 4096)

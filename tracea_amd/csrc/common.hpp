@@ -79,6 +79,8 @@ struct ContractionArgs {
   // instructions per padded patch row, pixels per load instruction
   int p_tm, p_seg, p_ppi;
   unsigned p_cpp_m, p_cpp_s, p_pw_m, p_pw_s;
+  // pipelines 7 and 8 only: reciprocals of grid_n and p_tiles (workgroup index -> filter slab, tile, image)
+  unsigned gn_m, gn_s, pt_m, pt_s;
   // pipeline 5 only: the chain in the fast form of conv_resident_kernel.hpp, or sig < 0
   struct FastEpilogue {
     int sig;                  // bit 0 affine, 1 ReLU, 2 residual, 3 ReLU (in this order); < 0: not of this form

@@ -4,6 +4,7 @@
 #include "contraction_kernel.hpp"
 #include "conv_patch_kernel.hpp"
 #include "conv_resident_kernel.hpp"
+#include "conv_wave16_kernel.hpp"
 
 #define TRACEA_CAT2(a, b) a##b
 #define TRACEA_CAT(a, b) TRACEA_CAT2(a, b)
@@ -21,6 +22,12 @@ const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
 #elif V_DIRECT == 5
       (size_t)rs_filter_bytes(V_STAGES) + RS_TABLE_BYTES,  // the patch, sized by the problem, comes on top
       &launch_conv_resident<V_STAGES, 4>, 32};  // 64 input channels: 4 k-steps per tap
+#elif V_DIRECT == 7
+      (size_t)CW_TABLE_BYTES,  // patch and filter slab, sized by the problem, come on top
+      &launch_conv_wave16<V_BK, (V_BM / 16 - 1) / 4, 0>, 16};
+#elif V_DIRECT == 8
+      (size_t)V_STAGES * cw_ring_stage_bytes(V_BK) + CW_TABLE_BYTES,  // the patch comes on top
+      &launch_conv_wave16<V_BK, (V_BM / 16 - 1) / 4, V_STAGES>, 16};
 #elif V_DIRECT == 6
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
       &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, 2, 16>, 16};  // pipeline 2 on 16x16x32 MFMAs

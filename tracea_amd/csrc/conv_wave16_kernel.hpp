@@ -1,0 +1,587 @@
+// Convolution on 16x16x32 MFMAs with the input patch resident in LDS and the filter slab either
+// resident beside it or streamed through a ring of one filter tap per stage (gfx950).
+//
+// Same arithmetic as the reference's kernel_main (src/emitter/cuda/conv.rs:153-331):
+// out[n,ho,wo,k] = epilogue(sum_{r,s,c} x[n, ho*sh-ph+r*dh, wo*sw-pw+s*dw, c] * w[k,r,s,c]),
+// fp32 accumulation in ascending (r,s,c) order, 32 channels per MFMA, zero padding.
+//
+// Work split.  A workgroup owns p_tm <= 16 * (4 * PBW + 1) consecutive output pixels of one image and
+// 64 filters; the host picks p_tm so that the launch is one balanced round over the CUs.  Pixels are cut
+// into blocks of 16, filters into 4 blocks of 16, and the unit of work is one pixel block x one filter
+// block = one v_mfma_f32_16x16x32 per 32-wide k-step.  Four multiplying waves, one per SIMD: wave w takes
+// the PBW consecutive pixel blocks w*PBW .. with all four filter blocks, and filter block w of the one
+// pixel block 4*PBW that is left over (392 pixels = 24.5 blocks: 6 whole blocks per wave and a quarter of
+// the 25th; with 32-pixel blocks the same tile was 28 units of which 24.5 held pixels).  A wave reads
+// PBW + 1 pixel fragments and 4 filter fragments of 1 KB per k-step for 4*PBW + 1 MFMAs of 16 cycles;
+// LDS delivers 128 bytes per clock to the CU, i.e. 0.5 KB per MFMA slot with all four matrix pipes busy:
+// PBW = 6 stays below that (0.44), PBW = 3 (0.62) runs at the LDS rate.  Four more waves only move data.
+//
+// A wave's pixels are consecutive, its results leave from registers (below), and nothing after the
+// operand wait is shared between the multiplying waves: each runs on its own.
+//
+// LDS layouts.  Patch: whole padded rows, pixel (hp, wp) at ((hp - hp0) * PW + wp) * cpp 16-byte chunks,
+// cpp = C/8 rounded up to odd, so that the 16 pixels of a fragment start in 16 different bank groups.
+// Filters, resident: row n at n * (K/8 | 1) chunks.  Filters, ring: stage t % RING holds tap t of the 64
+// filters, row n at n * (C/8 | 1) chunks.
+//
+// Epilogue.  The filter fragment is the first MFMA operand, so a lane ends with 4 consecutive output
+// channels (4q .. 4q+3 of a filter block, q = lane >> 4) of pixel lane & 15 of a pixel block.  For the
+// chains of the form [affine] [ReLU] [residual] [ReLU] everything happens in registers: per pair of filter
+// blocks one v_permlane16_swap per packed register gives every lane 8 consecutive channels of its pixel,
+// one 16-byte store; a residual is fetched in that layout, 16 bytes per lane, and taken back to the
+// accumulators' layout by the same swap.  Any other chain goes through LDS and the general operator loop.
+#pragma once
+#include "contraction_kernel.hpp"
+
+namespace tracea_amd {
+
+constexpr int CW_THREADS = 512;
+constexpr int CW_TABLE_BYTES = TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
+// bytes of the filter area: whole load iterations of the eight waves (resident) or RING stages of 64 rows
+constexpr int cw_ring_cpb(int cin) { return (cin / 8) | 1; }
+// (a stage is whole load instructions of the four helper waves: the lanes past its 64 rows write zeros)
+constexpr int cw_ring_iters(int cin) { return (64 * cw_ring_cpb(cin) + 255) / 256; }
+constexpr int cw_ring_stage_bytes(int cin) { return cw_ring_iters(cin) * 256 * 16; }
+// (the resident slab: whole load instructions of the eight waves)
+inline int cw_resident_filter_bytes(int k) {
+  const int chunks = 64 * ((k / 8) | 1);
+  return (chunks + CW_THREADS - 1) / CW_THREADS * CW_THREADS * 16;
+}
+
+template <int DT, int CIN, int PBW, int RING>
+__global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const ContractionArgs args) {
+  constexpr int NT = CW_THREADS, BN = 64, NW = NT / 64;
+  constexpr int KPT = CIN / 32;   // 32-wide k-steps per filter tap
+  constexpr int TAPB = CIN * 2;   // bytes of one tap in a filter row
+  constexpr int NPF = PBW + 1;    // pixel fragments per k-step
+  static_assert(KPT >= 2 && KPT % 2 == 0, "the two operand sets alternate with the k-steps of a tap");
+  static_assert(RING == 0 || RING >= 3, "the ring keeps two taps readable and at least one in flight");
+  constexpr int RCPB = cw_ring_cpb(CIN), RSTAGE = cw_ring_stage_bytes(CIN);
+  constexpr int RIT = cw_ring_iters(CIN);  // load instructions per helper wave and tap
+
+  // Everything the prologue reads from the kernel arguments, asked for here in one batch of scalar loads
+  // (left alone the compiler loads each field where it is first used, one round trip after the other).
+  asm volatile("" ::"s"(args.A), "s"(args.B), "s"(args.N), "s"(args.K), "s"(args.ldb), "s"(args.b_bytes), "s"(args.grid_n),
+               "s"(args.h_in), "s"(args.w_in), "s"(args.h_out), "s"(args.w_out), "s"(args.s_sz), "s"(args.r_sz));
+  asm volatile("" ::"s"(args.stride_h), "s"(args.stride_w), "s"(args.pad_h), "s"(args.pad_w), "s"(args.dil_h), "s"(args.dil_w),
+               "s"(args.w_m), "s"(args.w_s), "s"(args.p_tiles), "s"(args.p_pw), "s"(args.p_cpp), "s"(args.p_np_bytes),
+               "s"(args.p_tm), "s"(args.p_seg), "s"(args.p_ppi), "s"(args.p_cpp_m), "s"(args.p_cpp_s), "s"(args.p_pw_m),
+               "s"(args.p_pw_s), "s"(args.gn_m), "s"(args.gn_s), "s"(args.pt_m), "s"(args.pt_s));
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  unsigned char *patch = smem;
+  unsigned char *filt = smem + args.p_np_bytes;
+  const int K = args.K;
+  const int taps = args.r_sz * args.s_sz;
+  const int CPB = RING ? RCPB : ((K >> 3) | 1);
+  const int filt_bytes = RING ? RING * RSTAGE : (64 * CPB + NT - 1) / NT * NT * 16;
+  float *table = (float *)(filt + filt_bytes);
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int w = wave_u & 3;          // SIMD; the multiplying wave's index
+  const bool worker = wave_u < 4;
+  const int l15 = lane & 15, q = lane >> 4;
+
+  // ---- which tile ----
+  int bid = blockIdx.x;
+  const int total = gridDim.x;
+  if ((total & 7) == 0) bid = (bid & 7) * (total >> 3) + (bid >> 3);  // contiguous run per XCD
+  int tile_n, tm, img, tim;
+  fast_divmod(bid, args.gn_m, args.gn_s, args.grid_n, tm, tile_n);
+  fast_divmod(tm, args.pt_m, args.pt_s, args.p_tiles, img, tim);
+  const int TM = args.p_tm;
+  const int p0 = tim * TM;
+  const int hw = args.h_out * args.w_out;
+  const int npix = min(TM, hw - p0);
+  const int n0 = tile_n * BN;
+  const int N = args.N, C = CIN;
+  const int PW = args.p_pw, cpp = args.p_cpp;
+  const int pitch = cpp * 16;
+
+  constexpr unsigned OOB = 0x80000000u;  // beyond every buffer: the load returns zeros
+  const long long img_elems = (long long)args.h_in * args.w_in * C;
+  __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+      (void *)((const unsigned short *)args.A + (long long)img * img_elems), 0, (int)(img_elems * 2), 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_w =
+      __builtin_amdgcn_make_buffer_rsrc((void *)args.B, 0, (int)args.b_bytes, 0x00020000);
+
+  // ---- filters ----
+  // resident: chunk c of the area is filter row c / CPB, 16-byte part c % CPB (the last part is padding)
+  // ring: the helper waves bring tap t into stage t % RING: chunk c is row c / RCPB, part c % RCPB of the tap
+  unsigned ring_voff[RIT];
+  const int htid = tid - 256;
+  const bool ring_wave = RING != 0 && !worker;
+  auto ring_issue = [&](int t) __attribute__((always_inline)) {
+    unsigned char *sb = filt + (t % RING) * RSTAGE;
+#pragma unroll
+    for (int it = 0; it < RIT; ++it) {
+      unsigned char *dst = sb + (it * 256 + (wave_u - 4) * 64) * 16;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void *)dst, 16,
+                                               (int)ring_voff[it], t * TAPB, 0, 0);
+    }
+  };
+  if constexpr (RING != 0) {
+#pragma unroll
+    for (int it = 0; it < RIT; ++it) {
+      const int chunk = it * 256 + htid;
+      const int row = chunk / RCPB, part = chunk - row * RCPB;
+      const bool ok = (htid >= 0) & (part < CIN / 8) & (row < BN) & (n0 + row < N);
+      ring_voff[it] = ok ? (unsigned)(((n0 + row) * (int)args.ldb + part * 8) * 2) : OOB;
+    }
+  }
+
+  // ---- patch, by columns of load instructions ----
+  // One load instruction moves the PPI = 64 / cpp pixels wp0 .. wp0 + PPI - 1 of one padded row (lane l:
+  // pixel l / cpp, 16-byte part l % cpp; the part past the channels is padding and is written as zeros).
+  // A wave takes segment j = wave, wave + 8, ... of EVERY row: what depends on the lane is then fixed per
+  // segment.  Padding pixels and rows get an out-of-range offset and are written as zeros; lanes past the
+  // row's end are switched off (they would land on the next row's pixels).
+  int ho_f, wo_f, ho_l, wo_l;
+  fast_divmod(p0, args.w_m, args.w_s, args.w_out, ho_f, wo_f);
+  fast_divmod(p0 + npix - 1, args.w_m, args.w_s, args.w_out, ho_l, wo_l);
+  const int hp0 = ho_f * args.stride_h;
+  const int tap_h = args.dil_h * PW;  // pixel index step of one filter row
+  const int n_rows = ho_l * args.stride_h + (args.r_sz - 1) * args.dil_h - hp0 + 1;
+  const int SEG = args.p_seg, PPI = args.p_ppi;
+  constexpr int cdata = CIN >> 3;
+  int ldl, lpart;
+  fast_divmod(lane, args.p_cpp_m, args.p_cpp_s, cpp, ldl, lpart);
+  const int lane_off = (ldl - args.pad_w) * C * 2 + lpart * 16;
+  const int row_bytes = args.w_in * C * 2, row_pitch = PW * pitch;
+  for (int j = wave_u; j < SEG; j += NW) {
+    const int wp = j * PPI + ldl;
+    const bool lane_ok = ((unsigned)(wp - args.pad_w) < (unsigned)args.w_in) & (lpart < cdata);
+    const unsigned v_seg = lane_ok ? (unsigned)(lane_off + j * PPI * C * 2) : OOB;
+    if (wp < PW) {
+      int hi = hp0 - args.pad_h;
+      unsigned char *dst = patch + j * PPI * pitch;
+      for (int r = 0; r < n_rows; ++r) {
+        const bool row_ok = (unsigned)hi < (unsigned)args.h_in;
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_x, (__attribute__((address_space(3))) void *)dst, 16,
+                                                 (int)(row_ok ? v_seg : OOB), row_ok ? hi * row_bytes : 0, 0, 0);
+        hi += 1;
+        dst += row_pitch;
+      }
+    }
+  }
+  // (the patch first: its rows come from memory, the filters from the L2 every workgroup shares)
+  if constexpr (RING == 0) {
+    const int fit = (64 * CPB + NT - 1) / NT;
+    for (int it = 0; it < fit; ++it) {
+      const int chunk = it * NT + tid;
+      int row, part;
+      fast_divmod(chunk, args.p_pw_m, args.p_pw_s, CPB, row, part);  // (p_pw_m/s: the reciprocal of CPB here)
+      const bool ok = (part < (K >> 3)) & (row < BN) & (n0 + row < N);
+      const unsigned voff = ok ? (unsigned)(((n0 + row) * (int)args.ldb + part * 8) * 2) : OOB;
+      unsigned char *dst = filt + (it * NT + wave_u * 64) * 16;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void *)dst, 16, (int)voff,
+                                               0, 0, 0);
+    }
+  }
+  // ring: the first RING taps follow the patch, one per stage
+  if constexpr (RING != 0) {
+    if (ring_wave) {
+#pragma unroll
+      for (int t = 0; t < RING; ++t)
+        if (t < taps) ring_issue(t);
+    }
+  }
+
+  // ---- epilogue form and this thread's entry of the operand table (requested now, read after the wait) ----
+  // sig >= 0: the chain reads [affine] [ReLU] [residual] [ReLU] (bit 0 affine, 1 first ReLU, 2 residual,
+  // 3 second ReLU), affine = v*a + b per channel; table [0..63] = a, [64..127] = b.  sig < 0: any other
+  // chain, table in the layout of chain_table_value.
+  const int sig = args.fe.sig;
+  constexpr int TPT = CW_TABLE_BYTES / 4 / NT;
+  float tabr = 0.0f, tabg[TPT];
+  if (sig < 0) {
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) {
+      const int e = tid + i * NT;
+      tabg[i] = chain_table_value(args.epi, e / (2 * BN), (e / BN) & 1, n0 + e % BN, N);
+    }
+  } else if ((sig & 1) && tid < 2 * BN) {
+    const int which = tid / BN, n = n0 + tid % BN;
+    if (args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD) {
+      float one[1] = {1.0f};
+      if (which == 1) load_as_float<1>(args.fe.p0, args.fe.aff_dtype, n, 1, one);
+      tabr = one[0];
+    } else if (args.fe.aff_kind == TRACEA_EPI_OP_SCALE_SHIFT) {
+      tabr = ((const float *)(which == 0 ? args.fe.p0 : args.fe.p1))[n];
+    } else {  // BatchNorm folded: a = gamma / sqrt(var + eps), b = beta - mean * a
+      const float scale = ((const float *)args.fe.p0)[n] * (1.0f / sqrtf(((const float *)args.fe.p3)[n] + args.fe.epsilon));
+      tabr = which == 0 ? scale : ((const float *)args.fe.p1)[n] - ((const float *)args.fe.p2)[n] * scale;
+    }
+  }
+
+  // ---- per-lane operand addresses (worked out while the operands travel) ----
+  // pixel fragment i < PBW: block w*PBW + i; fragment PBW: the shared block 4*PBW
+  int a_base[NPF];
+#pragma unroll
+  for (int i = 0; i < NPF; ++i) {
+    const int blk = i < PBW ? w * PBW + i : 4 * PBW;
+    const int pr = blk * 16 + l15;
+    const int prc = pr < npix ? pr : npix - 1;
+    int ho, wo;
+    fast_divmod(p0 + prc, args.w_m, args.w_s, args.w_out, ho, wo);
+    a_base[i] = ((ho * args.stride_h - hp0) * PW + wo * args.stride_w) * pitch + q * 16;
+  }
+  // filter fragment i: filter block w ^ i (fragment 0 is the wave's own block, which the shared pixel block
+  // multiplies; fragments 2j and 2j+1 are neighbours in the channel order): row (w ^ i)*16 + l15, 16-byte part q
+  int f_base[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) f_base[i] = (((w ^ i) * 16 + l15) * CPB + q) * 16;
+  int step_s = args.dil_w * pitch;
+  int step_r = tap_h * pitch - (args.s_sz - 1) * step_s;
+  int off_last = ((args.r_sz - 1) * tap_h + (args.s_sz - 1) * args.dil_w) * pitch;
+  int s_size = args.s_sz;
+#pragma unroll
+  for (int i = 0; i < NPF; ++i) asm volatile("" : "+v"(a_base[i]));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(f_base[i]));
+  asm volatile("" : "+s"(step_s), "+s"(step_r), "+s"(off_last), "+s"(s_size));
+
+  // A bias that opens a chain of the fast form is where the accumulators start (one fp32 rounding apart from
+  // adding it last, and a hundred additions less in the epilogue of a wave that has nobody to share them with).
+  const bool bias_init = sig >= 0 && (sig & 1) && args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD;
+  const int form_sig = bias_init ? (sig & ~1) : sig;
+  f32x4 start[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float b4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (bias_init) load_as_float<4>(args.fe.p0, args.fe.aff_dtype, n0 + (w ^ i) * 16 + q * 4, 4, b4);
+    start[i] = f32x4{b4[0], b4[1], b4[2], b4[3]};
+  }
+  f32x4 acc[PBW][4], acc_x;
+#pragma unroll
+  for (int p = 0; p < PBW; ++p)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[p][i] = start[i];
+  acc_x = start[0];
+#pragma unroll
+  for (int p = 0; p < PBW; ++p)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(acc[p][i]));
+  asm volatile("" : "+v"(acc_x));
+
+  // ring: taps 0 and 1 must have landed; the RING - 2 later taps may stay in flight
+  if constexpr (RING != 0) {
+    constexpr int fl = RIT * (RING - 2);
+    static_assert(fl <= 63, "vmcnt is a 6-bit counter");
+    if (ring_wave && taps >= RING) __builtin_amdgcn_s_waitcnt(0x0f70 | (fl & 15) | ((fl >> 4) << 14));
+    else __builtin_amdgcn_s_waitcnt(0x0f70);
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  }
+  if (sig < 0) {
+#pragma unroll
+    for (int i = 0; i < TPT; ++i) table[tid + i * NT] = tabg[i];
+  } else if (tid < 2 * BN) {
+    table[tid] = tabr;
+  }
+  __syncthreads();
+
+  if constexpr (RING != 0) {
+    if (!worker) {
+      // helper waves: taps t .. t + RING - 1 occupy the stages; before barrier t tap t + 2 has landed (the
+      // RING - 3 after it may be in flight); behind it stage t % RING is free and receives tap t + RING.
+      // (No barrier where neither matters any more: t >= taps - 2.)
+      for (int t = 0; t + 2 < taps; ++t) {
+        if (t + RING - 1 < taps) {
+          constexpr int fl = RIT * (RING - 3);
+          __builtin_amdgcn_s_waitcnt(0x0f70 | (fl & 15) | ((fl >> 4) << 14));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+        }
+        __builtin_amdgcn_s_barrier();
+        if (ring_wave && t + RING < taps) ring_issue(t + RING);
+      }
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+    }
+  }
+
+  if (worker) {
+    u32x4 xa[2][NPF], xb[2][4];
+    int ts = 0, off = 0;
+    auto next_tap = [&]() {
+      ts += 1;
+      const bool wrap_s = ts == s_size;
+      ts = wrap_s ? 0 : ts;
+      off += wrap_s ? step_r : step_s;
+      off = off < off_last ? off : off_last;
+    };
+    // operand addresses of "the tap whose first k-step was read last": one set, moved on to the next tap in
+    // front of the read of its first k-step
+    const unsigned char *pp[NPF], *fp[4];
+#pragma unroll
+    for (int i = 0; i < NPF; ++i) pp[i] = patch + a_base[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fp[i] = filt + f_base[i];
+    auto read = [&](auto setc, auto kc) __attribute__((always_inline)) {
+      constexpr int set = decltype(setc)::value, k = decltype(kc)::value;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) xb[set][i] = *(const u32x4 *)(fp[i] + k * 64);
+#pragma unroll
+      for (int i = 0; i < NPF; ++i) xa[set][i] = *(const u32x4 *)(pp[i] + k * 64);
+    };
+    auto mma = [&](auto setc) __attribute__((always_inline)) {
+      constexpr int s = decltype(setc)::value;
+#pragma unroll
+      for (int p = 0; p < PBW; ++p)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[p][i] = Mfma16<DT>::run(xb[s][i], xa[s][p], acc[p][i]);
+      acc_x = Mfma16<DT>::run(xb[s][0], xa[s][PBW], acc_x);
+      Interleave<0, 4 * PBW + 1, 0x100, NPF + 4, 0x100, 0>::run();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::integral_constant;
+    read(integral_constant<int, 0>{}, integral_constant<int, 0>{});
+    __builtin_amdgcn_sched_barrier(0);
+    int t_now = 0;
+    auto tap = [&]() __attribute__((always_inline)) {
+      static_for<0, KPT>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        if constexpr (k + 1 < KPT) {
+          read(integral_constant<int, (k + 1) & 1>{}, integral_constant<int, k + 1>{});
+        } else {
+          // on to the next tap (worked out HERE, in front of the tap's last MFMAs: behind them it is a dozen
+          // instructions during which a lone wave's matrix pipe idles); past the last tap the addresses stay
+          // (the last tap is read again, unused)
+          next_tap();
+          const bool more = t_now + 1 < taps;
+#pragma unroll
+          for (int i = 0; i < NPF; ++i) pp[i] = patch + a_base[i] + off;
+          if constexpr (RING == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fp[i] += more ? TAPB : 0;
+          } else {
+            const int st = more ? (t_now + 1) % RING : t_now % RING;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fp[i] = filt + f_base[i] + st * RSTAGE;
+          }
+          read(integral_constant<int, 0>{}, integral_constant<int, 0>{});
+        }
+        mma(integral_constant<int, k & 1>{});
+      });
+      if constexpr (RING != 0) {
+        // barrier t: taps up to t + 2 are readable behind it (see the helper waves' loop)
+        if (t_now + 2 < taps) __builtin_amdgcn_s_barrier();
+      }
+      t_now += 1;
+    };
+    if constexpr (RING == 0) {
+      // several taps per trip: a taken branch costs a lone wave more than a hundred cycles of idle matrix pipe
+      const int trips = taps / 3;
+#pragma unroll 1
+      for (int t = 0; t < trips; ++t) {
+        tap();
+        tap();
+        tap();
+      }
+#pragma unroll 1
+      for (int t = trips * 3; t < taps; ++t) tap();
+    } else {
+#pragma unroll 1
+      for (int t = 0; t < taps; ++t) tap();
+    }
+  }
+
+  const long long m_img = (long long)img * hw + p0;
+  if (sig >= 0) {
+    if (!worker) return;
+    // ---- epilogue from registers ----
+    __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((unsigned short *)args.C + m_img * args.ldc + n0), 0, (int)((long long)npix * args.ldc * 2), 0x00020000);
+    __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const unsigned short *)args.fe.res + ((sig & 4) ? m_img * args.fe.res_ld + n0 : 0ll)), 0,
+        (sig & 4) ? (int)((long long)npix * args.fe.res_ld * 2) : 0, 0x00020000);
+    const int row_c = (int)args.ldc * 2, row_r = (int)args.fe.res_ld * 2;
+    auto pack2 = [](float x, float y) __attribute__((always_inline)) -> unsigned {
+      if constexpr (DT == DT_F16) {
+        const f16x2 h = {(_Float16)x, (_Float16)y};
+        return __builtin_bit_cast(unsigned, h);
+      } else {
+        const bf16x2 h = {(__bf16)x, (__bf16)y};
+        return __builtin_bit_cast(unsigned, h);
+      }
+    };
+    auto unpack2 = [](unsigned u, float &x, float &y) __attribute__((always_inline)) {
+      if constexpr (DT == DT_F16) {
+        const f16x2 h = __builtin_bit_cast(f16x2, u);
+        x = (float)h[0];
+        y = (float)h[1];
+      } else {
+        x = __builtin_bit_cast(float, u << 16);
+        y = __builtin_bit_cast(float, u & 0xffff0000u);
+      }
+    };
+    auto run_form = [&](auto form) __attribute__((always_inline)) {
+      constexpr int F = decltype(form)::value;
+      constexpr bool AFF = (F & 1) != 0, RELU1 = (F & 2) != 0, RES = (F & 4) != 0, RELU2 = (F & 8) != 0;
+      // the chain's last ReLU on the packed halves (one v_pk_max_f16 per two values; rounding is monotonic
+      // and keeps zero, so max before or after it is the same value)
+      constexpr bool PK = DT == DT_F16 && (RELU2 || (RELU1 && !RES));
+      constexpr bool RELU1_F32 = RELU1 && !(PK && !RES), RELU2_F32 = RELU2 && !PK;
+      f32x4 ta[4] = {}, tb[4] = {};
+      if constexpr (AFF) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ta[i] = *(const f32x4 *)(table + (w ^ i) * 16 + q * 4);
+          tb[i] = *(const f32x4 *)(table + BN + (w ^ i) * 16 + q * 4);
+        }
+      }
+      auto finish = [&](f32x4 v, f32x4 a, f32x4 b, float r0, float r1, float r2, float r3) __attribute__((always_inline)) -> f32x4 {
+        if constexpr (AFF) v = v * a + b;
+        if constexpr (RELU1_F32) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = fmaxf(0.0f, v[e]);
+        }
+        if constexpr (RES) {
+          v[0] += r0; v[1] += r1; v[2] += r2; v[3] += r3;
+        }
+        if constexpr (RELU2_F32) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = fmaxf(0.0f, v[e]);
+        }
+        return v;
+      };
+      auto pack_out = [&](float x, float y) __attribute__((always_inline)) -> unsigned {
+        unsigned u = pack2(x, y);
+        if constexpr (PK) {
+          const f16x2 z = {(_Float16)0.0f, (_Float16)0.0f};
+          u = __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(f16x2, u), z));
+        }
+        return u;
+      };
+      static_for<0, PBW>([&](auto pc) {
+        constexpr int p = decltype(pc)::value;
+        const int pr = (w * PBW + p) * 16 + l15;
+        const int prow = pr < npix ? pr : -1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          // lanes of 16-lane group q hold, after the swap, channels (q>>1)*8 .. +7 of filter block w ^ (2j + (q&1))
+          const int ch = (w ^ (2 * j + (q & 1))) * 16 + (q >> 1) * 8;
+          float ra[4] = {0, 0, 0, 0}, rb[4] = {0, 0, 0, 0};
+          if constexpr (RES) {
+            u32x4 r8 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                     rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
+            unsigned r0 = r8[0], r1 = r8[1], r2 = r8[2], r3 = r8[3];
+            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
+                         : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));
+            unpack2(r0, ra[0], ra[1]);
+            unpack2(r1, ra[2], ra[3]);
+            unpack2(r2, rb[0], rb[1]);
+            unpack2(r3, rb[2], rb[3]);
+          }
+          const f32x4 va = finish(acc[p][2 * j], ta[2 * j], tb[2 * j], ra[0], ra[1], ra[2], ra[3]);
+          const f32x4 vb = finish(acc[p][2 * j + 1], ta[2 * j + 1], tb[2 * j + 1], rb[0], rb[1], rb[2], rb[3]);
+          unsigned a_lo = pack_out(va[0], va[1]), a_hi = pack_out(va[2], va[3]);
+          unsigned b_lo = pack_out(vb[0], vb[1]), b_hi = pack_out(vb[2], vb[3]);
+          // (as instructions: the compiler's builtin for the swap returns its first result twice; the s_nop is the
+          // wait the hardware asks for between a vector-ALU write of an operand and the swap)
+          asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
+                       : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi));
+          const u32x4 row8 = {a_lo, a_hi, b_lo, b_hi};
+          __builtin_amdgcn_raw_buffer_store_b128(row8, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
+        }
+      });
+      {  // the shared block: filter block w only, 4 channels (8 bytes) per lane
+        const int pr = 4 * PBW * 16 + l15;
+        const int prow = pr < npix ? pr : -1;
+        const int ch = w * 16 + q * 4;
+        float rr[4] = {0, 0, 0, 0};
+        if constexpr (RES) {
+          const u32x2 r4 = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(
+                                                          rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
+          unpack2(r4[0], rr[0], rr[1]);
+          unpack2(r4[1], rr[2], rr[3]);
+        }
+        const f32x4 v = finish(acc_x, ta[0], tb[0], rr[0], rr[1], rr[2], rr[3]);
+        const u32x2 o = {pack_out(v[0], v[1]), pack_out(v[2], v[3])};
+        __builtin_amdgcn_raw_buffer_store_b64(o, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
+      }
+    };
+    switch (form_sig) {
+#define TRACEA_CW_FORM(F) case F: run_form(std::integral_constant<int, F>{}); break;
+      TRACEA_CW_FORM(0) TRACEA_CW_FORM(1) TRACEA_CW_FORM(2) TRACEA_CW_FORM(3) TRACEA_CW_FORM(4) TRACEA_CW_FORM(5)
+      TRACEA_CW_FORM(6) TRACEA_CW_FORM(7) TRACEA_CW_FORM(8) TRACEA_CW_FORM(9) TRACEA_CW_FORM(10) TRACEA_CW_FORM(11)
+      TRACEA_CW_FORM(12) TRACEA_CW_FORM(13) TRACEA_CW_FORM(14) TRACEA_CW_FORM(15)
+#undef TRACEA_CW_FORM
+      default: break;
+    }
+    return;
+  }
+
+  // ---- any other chain: accumulators through LDS, then the general operator loop over whole pixels ----
+  constexpr int SP = BN + 4;  // floats per staged pixel
+  float *stage = (float *)smem;
+  __syncthreads();  // every wave has left the main loop: patch and filters may be overwritten
+  if (worker) {
+    static_for<0, PBW>([&](auto pc) {
+      constexpr int p = decltype(pc)::value;
+      const int pr = (w * PBW + p) * 16 + l15;
+      if (pr < npix) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *(f32x4 *)(stage + pr * SP + (w ^ i) * 16 + q * 4) = acc[p][i];
+      }
+    });
+    const int pr = 4 * PBW * 16 + l15;
+    if (pr < npix) *(f32x4 *)(stage + pr * SP + w * 16 + q * 4) = acc_x;
+  }
+  __syncthreads();
+  const int ec = (tid & 7) * 8;
+  const ChainPlan plan = chain_plan(args.epi);
+  for (int idx = tid; idx < npix * (BN / 8); idx += NT) {
+    const int pr = idx >> 3;
+    const int n = n0 + ec;
+    if (n < N) {
+      float v[8];
+      const f32x4 lo = *(const f32x4 *)(stage + pr * SP + ec);
+      const f32x4 hi = *(const f32x4 *)(stage + pr * SP + ec + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = lo[e];
+        v[4 + e] = hi[e];
+      }
+      const int nvalid = N - n;
+      const long long m = m_img + pr;
+      apply_epilogue_tab(v, m, n, nvalid, args.epi, plan, table + ec, BN);
+      store_from_float<8>(args.C, args.out_dtype, m * args.ldc + n, nvalid, v);
+    }
+  }
+}
+
+// bm = 16 * (4 * PBW + 1) pixels at most per workgroup; CIN input channels exactly; RING = 0: the whole
+// filter slab (64 x K) resident beside the patch, else a ring of RING one-tap stages.
+template <int CIN, int PBW, int RING>
+int launch_conv_wave16(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig, hipStream_t stream) {
+  if (!conv || b_ncontig || a.c_in != CIN || a.K != a.r_sz * a.s_sz * CIN || a.p_tm <= 0 || a.p_tm > 16 * (4 * PBW + 1) ||
+      a.p_np_bytes <= 0)
+    return (int)hipErrorInvalidValue;
+  const size_t filt = RING ? (size_t)RING * cw_ring_stage_bytes(CIN) : (size_t)cw_resident_filter_bytes(a.K);
+  size_t lds = (size_t)a.p_np_bytes + filt + CW_TABLE_BYTES;
+  // the general epilogue stages p_tm x 68 floats in front of the table
+  if ((size_t)a.p_tm * 68 * 4 > lds - CW_TABLE_BYTES) lds = (size_t)a.p_tm * 68 * 4 + CW_TABLE_BYTES;
+  if (lds > 160 * 1024) return (int)hipErrorInvalidValue;
+  const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(CW_THREADS);
+#define TRACEA_LAUNCH_CW(DTV)                                                                        \
+  do {                                                                                               \
+    auto kfn = conv_wave16_kernel<DTV, CIN, PBW, RING>;                                               \
+    static bool attr_done = false;                                                                   \
+    if (!attr_done) {                                                                                \
+      hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                         160 * 1024);                                                \
+      if (e != hipSuccess) return (int)e;                                                            \
+      attr_done = true;                                                                              \
+    }                                                                                                \
+    hipLaunchKernelGGL(kfn, grid, block, lds, stream, a);                                            \
+    return (int)hipGetLastError();                                                                   \
+  } while (0)
+  if (dtype == DT_F16) TRACEA_LAUNCH_CW(DT_F16);
+  else TRACEA_LAUNCH_CW(DT_BF16);
+#undef TRACEA_LAUNCH_CW
+  return (int)hipErrorInvalidValue;
+}
+
+}  // namespace tracea_amd

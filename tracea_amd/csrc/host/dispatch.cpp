@@ -245,9 +245,9 @@ TraceaStatus check_bias_residual(const char *what, const TraceaTensorView *bias,
   return TRACEA_SUCCESS;
 }
 
-std::atomic<int> g_forced_contraction{-1};
-std::atomic<int> g_forced_conv{-1};
-std::atomic<int> g_forced_attention{-1};
+// A forced variant belongs to the thread that set it: the tuner (and a test) forces a variant around its own
+// launches, and another thread dispatching meanwhile must keep its own choice.
+thread_local int t_forced_contraction = -1, t_forced_conv = -1, t_forced_attention = -1;
 std::atomic<bool> g_split_k_enabled{true};
 std::atomic<bool> g_split_k_one_launch{true};
 std::atomic<bool> g_conv_transpose_by_phase{true};
@@ -304,9 +304,9 @@ void conv_transpose_filter_cache_clear() {
 int last_split_k() { return t_last_splits; }
 
 void set_forced_variant(const char *op, int index) {
-  if (!strcmp(op, "gemm")) g_forced_contraction.store(index);
-  else if (!strcmp(op, "conv2d")) g_forced_conv.store(index);
-  else if (!strcmp(op, "attention")) g_forced_attention.store(index);
+  if (!strcmp(op, "gemm")) t_forced_contraction = index;
+  else if (!strcmp(op, "conv2d")) t_forced_conv = index;
+  else if (!strcmp(op, "attention")) t_forced_attention = index;
 }
 int last_variant(const char *op) {
   if (!strcmp(op, "gemm")) return t_last_contraction;
@@ -315,9 +315,9 @@ int last_variant(const char *op) {
   return -1;
 }
 int forced_variant(const char *op) {
-  if (!strcmp(op, "gemm")) return g_forced_contraction.load();
-  if (!strcmp(op, "conv2d")) return g_forced_conv.load();
-  if (!strcmp(op, "attention")) return g_forced_attention.load();
+  if (!strcmp(op, "gemm")) return t_forced_contraction;
+  if (!strcmp(op, "conv2d")) return t_forced_conv;
+  if (!strcmp(op, "attention")) return t_forced_attention;
   return -1;
 }
 
@@ -520,10 +520,11 @@ int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig) {
 
 namespace {
 
-int pick_contraction(const char *op, const std::string &cache_key, int m, int n, int k, bool conv, bool b_ncontig = false) {
+int pick_contraction(const char *op, const std::string &cache_key, int m, int n, int k, bool conv, int dtype,
+                     bool b_ncontig = false) {
   const int forced = forced_variant(op);
   if (forced >= 0) return forced;
-  int cached = tuning_cache_lookup_variant(cache_key);
+  int cached = tuning_cache_lookup_variant(cache_key, dtype, b_ncontig);
   if (cached >= 0) return cached;
   return select_contraction_variant(m, n, k, conv, b_ncontig);
 }
@@ -735,7 +736,7 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
       args.epi = chain;
       char key[160];
       snprintf(key, sizeof(key), "gemm_%lld_%lld_%lld_%s", M, N, K, tuning_device_name());
-      int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false, !b_kcontig);
+      int vi = pick_contraction("gemm", key, (int)M, (int)N, (int)K, false, a.dtype, !b_kcontig);
       if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "gemm: no kernel variant available");
       // direct-to-LDS variants address operands with 32-bit byte offsets below 2 GiB
       const long long a_extent = ((M - 1) * a.stride[0] + K) * 2;
@@ -1382,7 +1383,8 @@ bool plan_conv_patch(const ConvGeometry &g, const ContractionVariant &v, bool w_
 bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
   const TraceaConvParamsBlock &b = g.block;
   const int C = b.c_in;
-  if (v.pipeline != 5 || w_ncontig || C % 16 != 0 || g.k_gemm != 16 * v.stages) return false;
+  // (the compiled member walks K as taps of 64 channels: 3x3x64; another split of K = 576 is not its problem)
+  if (v.pipeline != 5 || w_ncontig || C != 64 || g.k_gemm != 16 * v.stages) return false;
   const long long img_bytes = (long long)b.h_in * b.w_in * C * 2;
   const long long w_bytes = (long long)g.n_gemm * g.k_gemm * 2;
   if (img_bytes >= (1ll << 31) || w_bytes >= (1ll << 31)) return false;
@@ -1446,6 +1448,83 @@ bool plan_conv_filter_resident(const ConvGeometry &g, const ContractionVariant &
   return true;
 }
 
+// The same for the kernels on 16x16x32 MFMAs (pipelines 7 and 8, conv_wave16_kernel.hpp): K-contiguous
+// filters, exactly v.bk input channels, a workgroup takes p_tm <= v.bm consecutive output pixels of one
+// image and 64 filters; beside the patch LDS holds the whole 64 x K filter slab (pipeline 7) or a ring of
+// v.stages one-tap stages (pipeline 8).  p_tm as for the kernel above: fewest rounds over the CUs, then the
+// most workgroups; N32 56x56 -> 8 tiles of 392 pixels per image, N32 28x28 with 128 filters -> 4 tiles of
+// 196 pixels x 2 filter slabs, 256 workgroups each.
+bool plan_conv_wave16(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  const TraceaConvParamsBlock &b = g.block;
+  const int C = b.c_in;
+  if ((v.pipeline != 7 && v.pipeline != 8) || w_ncontig || C != v.bk || g.k_gemm != b.r_sz * b.s_sz * C) return false;
+  const long long img_bytes = (long long)b.h_in * b.w_in * C * 2;
+  const long long w_bytes = (long long)g.n_gemm * g.k_gemm * 2;
+  if (img_bytes >= (1ll << 31) || w_bytes >= (1ll << 31)) return false;
+  const long long pw = (long long)b.w_in + 2ll * g.pad_w;
+  const long long ph = (long long)b.h_in + 2ll * g.pad_h;
+  if (pw * ph >= (1ll << 30) || (long long)b.h_in * b.w_in >= (1ll << 24)) return false;
+  const int f_cpb = (g.k_gemm / 8) | 1;
+  const long long filter_bytes =
+      v.pipeline == 7 ? ((64ll * f_cpb + 511) / 512) * 512 * 16 : (long long)v.lds_bytes - TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
+  const long long table_bytes = TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
+  const int hw = b.h_out * b.w_out;
+  const int grid_n = (g.n_gemm + v.bn - 1) / v.bn;
+  const long long cus = device_limits().cus;
+  const long long t_min = (hw + v.bm - 1) / v.bm;
+  const long long rounds = ((long long)b.batch * t_min * grid_n + cus - 1) / cus;
+  long long tiles = rounds * cus / ((long long)b.batch * grid_n);
+  if (tiles < t_min) tiles = t_min;
+  if (tiles > (hw + 15) / 16) tiles = (hw + 15) / 16;
+  const int tm = (int)((hw + tiles - 1) / tiles);
+  const int cpp = (C / 8) | 1;
+  const int ppi = 64 / cpp;
+  if (ppi < 1) return false;
+  const int seg = (int)((pw + ppi - 1) / ppi);
+  // LDS bytes of the patch of the worst tile when tiles hold t pixels (tiles start at multiples of t): the
+  // most output rows a tile spans, then padded input rows
+  auto patch_for = [&](int t) -> long long {
+    long long out_rows = 1;
+    for (int p0 = 0; p0 < hw; p0 += t) {
+      const int last = (p0 + t < hw ? p0 + t : hw) - 1;
+      const long long span = last / b.w_out - p0 / b.w_out + 1;
+      if (span > out_rows) out_rows = span;
+    }
+    const long long rows = (out_rows - 1) * g.stride_h + (long long)(b.r_sz - 1) * g.dil_h + 1;
+    const long long bytes = (rows * pw * cpp + 64) * 16;
+    return (bytes + 1023) / 1024 * 1024;
+  };
+  const long long room = (long long)device_limits().lds_bytes - filter_bytes - table_bytes;
+  // the largest tile up to the balanced one that fits; failing that (few, wide rows: a smaller tile still
+  // straddles two rows) the smallest larger one
+  int tm_fit = 0;
+  for (int t = tm < v.bm ? tm : v.bm; t >= 16 && tm_fit == 0; --t)
+    if (patch_for(t) <= room) tm_fit = t;
+  for (int t = tm + 1; t <= v.bm && t <= hw && tm_fit == 0; ++t)
+    if (patch_for(t) <= room) tm_fit = t;
+  if (tm_fit == 0) return false;
+  const long long patch_bytes = patch_for(tm_fit);
+  a->r_sz = b.r_sz;
+  a->p_tm = tm_fit;
+  a->p_tiles = (hw + tm_fit - 1) / tm_fit;
+  a->p_pw = (int)pw;
+  a->p_cpp = cpp;
+  a->p_iters = 0;
+  a->p_np_bytes = (int)patch_bytes;
+  a->p_seg = seg;
+  a->p_ppi = ppi;
+  magic_for_divisor((uint32_t)cpp, 64, &a->p_cpp_m, &a->p_cpp_s);
+  magic_for_divisor((uint32_t)f_cpb, (uint64_t)(64 * f_cpb + 512), &a->p_pw_m, &a->p_pw_s);  // filter rows of the resident slab
+  a->grid_m = b.batch * a->p_tiles;
+  a->grid_n = grid_n;
+  magic_for_divisor((uint32_t)grid_n, (uint64_t)a->grid_m * grid_n, &a->gn_m, &a->gn_s);
+  magic_for_divisor((uint32_t)a->p_tiles, (uint64_t)a->grid_m, &a->pt_m, &a->pt_s);
+  a->group_m = 1;
+  a->b_bytes = (unsigned)w_bytes;
+  a->a_bytes = 0;
+  return true;
+}
+
 // The operator chain in the fast form of the filter-resident kernel: [affine] [ReLU] [residual] [ReLU],
 // each part at most once and in this order, affine = bias / scale-shift / BatchNorm; every tile has all 64
 // channels, output rows and residual rows are 8-byte aligned and addressable with 32-bit byte offsets
@@ -1484,6 +1563,7 @@ void fast_epilogue_form(const EpilogueChain &chain, int dtype, ContractionArgs *
 }
 
 bool plan_conv_resident(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  if (v.pipeline == 7 || v.pipeline == 8) return plan_conv_wave16(g, v, w_ncontig, a);
   return v.pipeline == 5 ? plan_conv_filter_resident(g, v, w_ncontig, a) : plan_conv_patch(g, v, w_ncontig, a);
 }
 
@@ -1507,14 +1587,29 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   snprintf(key, sizeof(key), "conv_%d_%d_%d_%d_%d_%d_%d_%d_%d_%s", g.block.batch, g.block.h_in,
            g.block.w_in, g.block.c_in, g.block.k_out, g.block.r_sz, g.block.s_sz, g.stride_h,
            g.pad_h, tuning_device_name());
-  int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true);
+  int vi = pick_contraction("conv2d", key, a.M, a.N, a.K, true, plan.x.dtype, plan.w_ncontig);
   if (vi < 0) return fail(TRACEA_UNKNOWN_ERROR, "conv2d: no kernel variant available");
   // Default choice of the filter-resident variant (patch and 64 filters of K = 576 in LDS together, no
   // barrier in its main loop): wherever it can run and the launch fills most of the device with tiles of
   // at least 10 pixel blocks.  Measured in a replayed HIP graph against the best other variant: N32
   // 56x56x64->64 14.1 us / 16.7; N64 25.2 / 28.6; N32 64->128 24.5 / 28.8; N8 10.3 / 9.5 (not taken).
   bool resident_chosen = false;
-  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0) {
+  // First choice: the kernels on 16x16x32 MFMAs with the patch in LDS and the filter slab resident or in a
+  // ring (pipelines 7 and 8), where their plan fits, the launch fills most of the device and a workgroup's
+  // tile is at least three quarters of the kernel's largest (smaller tiles leave its waves' blocks empty).
+  if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key, plan.x.dtype, plan.w_ncontig) < 0) {
+    for (int i = 0; i < contraction_variant_count() && !resident_chosen; ++i) {
+      const ContractionVariant &cv = contraction_variant(i);
+      if (cv.pipeline != 7 && cv.pipeline != 8) continue;
+      ContractionArgs probe = a;
+      if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n * 4 >= device_limits().cus * 3 &&
+          probe.p_tm * 4 >= cv.bm * 3) {
+        vi = i;
+        resident_chosen = true;
+      }
+    }
+  }
+  if (!resident_chosen && forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key, plan.x.dtype, plan.w_ncontig) < 0) {
     for (int i = 0; i < contraction_variant_count() && !resident_chosen; ++i) {
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline != 5) continue;
@@ -1537,7 +1632,7 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // short K (one 56x56x64->64 image: 7.4 us against 8.4).  Everywhere else the streamed
   // 8-wave 128x64 and pipelined 64x64 tiles are as fast or faster.  A tuning-cache entry or
   // a forced variant wins over this rule, and tracea_autotune_conv2d measures every variant.
-  if (!resident_chosen && forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key) < 0 && g.stride_h == 1 &&
+  if (!resident_chosen && forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key, plan.x.dtype, plan.w_ncontig) < 0 && g.stride_h == 1 &&
       g.stride_w == 1 && g.block.r_sz * g.block.s_sz > 1 && a.K % 64 == 0 && a.K / 64 <= 40) {
     const long long hw = (long long)g.block.h_out * g.block.w_out;
     int chosen = -1;
@@ -1563,10 +1658,15 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   const long long w_extent = (long long)g.n_gemm * g.k_gemm * 2;
   const bool small = x_extent < (1ll << 31) && w_extent < (1ll << 31);
   if (conv_only(contraction_variant(vi)) && plan_conv_resident(g, contraction_variant(vi), plan.w_ncontig, &a)) {
-    if (contraction_variant(vi).pipeline == 5) fast_epilogue_form(chain, plan.x.dtype, &a);
-    t_last_conv = vi;
-    return hip_status("conv2d launch",
-                      contraction_variant(vi).launch(a, true, plan.x.dtype, false, stream));
+    if (contraction_variant(vi).pipeline == 5 || contraction_variant(vi).pipeline >= 7) fast_epilogue_form(chain, plan.x.dtype, &a);
+    const int e = contraction_variant(vi).launch(a, true, plan.x.dtype, false, stream);
+    // a member that refuses the arguments its plan accepted (it launched nothing) gives way to the
+    // selector's choice below, like one whose plan failed
+    if (e != (int)hipErrorInvalidValue) {
+      t_last_conv = vi;
+      return hip_status("conv2d launch", e);
+    }
+    (void)hipGetLastError();
   }
   // a patch-resident variant that cannot run this problem (asked for by a forced
   // index or a cache entry) gives way to the selector's choice, not to whatever

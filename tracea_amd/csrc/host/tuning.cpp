@@ -50,6 +50,8 @@ void load_locked() {
     if (!cfg || !PipelineConfig::from_json_value(*cfg, &e.config, &err)) continue;
     if (const Json *s = kv.second.find("score")) e.score = (float)s->num;
     if (const Json *t = kv.second.find("timestamp")) e.timestamp = (uint64_t)t->num;
+    if (const Json *t = kv.second.find("operand_dtype")) e.operand_dtype = t->str;
+    if (const Json *t = kv.second.find("b_layout")) e.b_layout = t->str;
     g_cache[kv.first] = e;
   }
 }
@@ -64,6 +66,8 @@ void save_locked() {
     e.set("config", kv.second.config.to_json_value());
     e.set("score", Json::make_num(kv.second.score));
     e.set("timestamp", Json::make_num((double)kv.second.timestamp));
+    if (!kv.second.operand_dtype.empty()) e.set("operand_dtype", Json::make_str(kv.second.operand_dtype));
+    if (!kv.second.b_layout.empty()) e.set("b_layout", Json::make_str(kv.second.b_layout));
     root.set(kv.first, e);
   }
   std::ofstream f(path);
@@ -181,9 +185,9 @@ void tuning_history_reload() {
   g_hist_loaded = false;
 }
 
-int tuning_cache_lookup_variant(const std::string &key) {
+int tuning_cache_lookup_variant(const std::string &key, int dtype, bool b_ncontig) {
   CacheEntry e;
-  if (!tuning_cache_get(key, &e)) return -1;
+  if (!tuning_cache_get(key, &e) || !e.matches(dtype, b_ncontig)) return -1;
   return contraction_variant_for_config(e.config);
 }
 
@@ -492,6 +496,8 @@ TraceaResult tune_gemm(size_t m, size_t n, size_t k) {
   e.config = config_for_contraction_variant(best);
   e.score = best_tflops;
   e.timestamp = now_seconds();
+  e.operand_dtype = "f16";
+  e.b_layout = "k_contiguous";
   tuning_cache_put(gemm_cache_key(m, n, k, tuning_device_name()), e, true);
   record_history(gemm_cache_key(m, n, k, tuning_device_name()), e, "F16");
   return success(e.config, e.score);
@@ -519,6 +525,8 @@ TraceaResult tune_conv2d(size_t n, size_t c, size_t h, size_t w, size_t k, size_
   e.config.layout_policy = "NHWC";
   e.score = best_tflops;
   e.timestamp = now_seconds();
+  e.operand_dtype = "f16";
+  e.b_layout = "k_contiguous";
   ConvProblem p;
   p.batch = (uint32_t)n; p.h_in = (uint32_t)h; p.w_in = (uint32_t)w; p.c_in = (uint32_t)c;
   p.c_out = (uint32_t)k; p.kernel_h = (uint32_t)r; p.kernel_w = (uint32_t)s;

@@ -13,6 +13,18 @@ struct CacheEntry {
   PipelineConfig config;
   float score = 0.0f;  // TFLOP/s
   uint64_t timestamp = 0;
+  // What the record was measured on.  The reference's keys (gemm_{m}_{n}_{k}_{dev}, src/core/tuning.rs:14-34)
+  // carry neither the element type nor the layout of B, so a record of one would steer calls with the other:
+  // the two are kept inside the entry (additional fields, ignored by a reader that does not know them) and a
+  // lookup for other operands skips the record.  Empty (a record written without them, e.g. by the reference):
+  // f16 with a K-contiguous B, which is what every tuner of this path measures.
+  std::string operand_dtype;  // "f16" | "bf16"
+  std::string b_layout;       // "k_contiguous" | "n_contiguous"
+  bool matches(int dtype, bool b_ncontig) const {
+    const std::string d = operand_dtype.empty() ? "f16" : operand_dtype;
+    const std::string l = b_layout.empty() ? "k_contiguous" : b_layout;
+    return d == (dtype == DT_BF16 ? "bf16" : "f16") && l == (b_ncontig ? "n_contiguous" : "k_contiguous");
+  }
 };
 
 // Name of device 0 as the cache keys spell it ("" before tracea_init succeeds).
@@ -41,8 +53,9 @@ bool tuning_history_query(const std::string &key, HistoryEntry *out);
 void tuning_history_record(const std::string &key, const HistoryEntry &e);
 void tuning_history_reload();
 
-// Index of the contraction variant a cached config names, or -1.
-int tuning_cache_lookup_variant(const std::string &key);
+// Index of the contraction variant a cached config names, or -1; a record measured on other operands
+// (element type, layout of B) than the caller's does not count.
+int tuning_cache_lookup_variant(const std::string &key, int dtype = DT_F16, bool b_ncontig = false);
 
 // PipelineConfig <-> kernel variant
 PipelineConfig config_for_contraction_variant(int index);
