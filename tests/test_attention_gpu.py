@@ -137,10 +137,11 @@ def test_scores_that_climb_along_the_sequence(tracea_gpu, variant, dtype, step):
 def test_two_query_blocks_per_workgroup(tracea_gpu, variant, d, dtype):
     """The _x2 members give a workgroup two query blocks (a heavy and a light one under a causal mask), the
     second on K/V tiles and queries requested during the first.  Every query still sees its keys in the same
-    order with the same arithmetic: the output must equal the one-block member's bit for bit, on lengths that
-    end inside a tile, on scores that climb along the sequence and with a dominant key; the one-block member
-    is checked against the oracle on the same inputs.  A length with an odd number of blocks has no pairs: a
-    forced _x2 member is then not the one that runs."""
+    order with the same arithmetic (both fold the softmax shift into the score product; at head dimension 128
+    the paired member parks half of the second block's queries in LDS to have the registers for it): the output
+    must equal the one-block member's bit for bit, on lengths that end inside a tile, on scores that climb along
+    the sequence and with a dominant key; the one-block member is checked against the oracle on the same inputs.
+    A length with an odd number of blocks has no pairs: a forced _x2 member is then not the one that runs."""
     from tracea_amd import capi
     tdt, rnd = (torch.bfloat16, round_bf16) if dtype == "bf16" else (torch.float16, round_f16)
     bq = int(variant[0][1:])
@@ -160,8 +161,8 @@ def test_two_query_blocks_per_workgroup(tracea_gpu, variant, d, dtype):
                 capi.force_variant("attention", paired)
                 two = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal)
                 assert capi.last_variant("attention") == paired, (s, causal)
-                assert torch.equal(one, two), "%s S=%d causal=%s: differs from %s" % (paired, s, causal, single)
                 want = oracle.attention_bhsd(q, k, v, 1.0 / np.sqrt(d), causal)
+                assert torch.equal(one, two), "%s S=%d causal=%s: differs from %s" % (paired, s, causal, single)
                 assert_close_scaled(one.float().cpu().numpy(), want, _tol(d, dtype), "%s S=%d causal=%s" % (single, s, causal))
         q, k, v = [_dev(rnd(np.random.default_rng(3).standard_normal((1, 2, 3 * bq, d))), tdt) for _ in range(3)]
         capi.force_variant("attention", paired)

@@ -393,9 +393,21 @@ fa2_fwd_kernel(const AttentionArgs a) {
 // Measured at B4 H32 S4096 D128 (replayed graphs, one box): dense 1002 -> 980 us on 8 waves, causal 585 -> 553
 // on 4.  (Four blocks per workgroup: the third set of queries in flight spills at head dimension 128, and the
 // coarser units balance worse: 999 and 572 us.)
-template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB, int ITEMS = 1>
+//
+// SHIFT: the softmax shift rides the score product.  The queries are multiplied by scale * log2(e) when they
+// are loaded (rounded once more to the operand type: a relative 2^-9 on q, about as much on a probability),
+// and the first MFMA of every S^T block accumulates onto a register block holding -m, the query's reference
+// maximum, instead of zero: the product comes out as z = s * scale * log2(e) - m and a probability is one
+// v_exp_f32 of it, without the multiply-add per score that the vector ALU, the busiest unit of this kernel,
+// spent on the shift.  The maximum of a tile is taken of z: while it stays below FA_RESCALE_TAU the reference
+// stays; when it moves, the tile's z are lowered by the step and O and the row sum rescaled.  Costs 16
+// registers per query block (the -m block), which the paired members at head dimension 128 do not have.
+constexpr bool fa2_pipe_parks_queries(int d, int qb, int items, bool shift) { return items > 1 && shift && d == 128 && qb == 1; }
+template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB, int ITEMS = 1, bool SHIFT = false>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 fa2_fwd_pipe_kernel(const AttentionArgs a) {
+  static_assert(!SHIFT || EARLY_MAX, "the shifted score product exists in the two-phase form only");
+  constexpr bool PARK = fa2_pipe_parks_queries(D, QB, ITEMS, SHIFT);
   static_assert(QB == 1 || (QB == 2 && EARLY_MAX), "two query blocks per wave exist in the two-phase form only");
   static_assert(ITEMS == 1 || (ITEMS == 2 && EARLY_MAX), "pairs of query blocks exist in the two-phase form only");
   constexpr int WQ = 32 * QB;  // queries per wave
@@ -451,14 +463,32 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   int last_key[QB];
   int wave_last_key;  // (wave-uniform) the last key any query of the wave may keep
   u32x4 qf[QB][KS];
-  auto load_q = [&](int first_query, u32x4 (&dst)[QB][KS]) __attribute__((always_inline)) {
+  // (SHIFT) a fragment of queries times scale * log2(e), rounded to the operand type
+  auto prescale = [&](u32x4 raw) __attribute__((always_inline)) -> u32x4 {
+    if constexpr (!SHIFT) return raw;
+    float qs[8];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if constexpr (DT == DT_F16) {
+        qs[2 * e] = (float)__builtin_bit_cast(_Float16, (unsigned short)(raw[e] & 0xffffu)) * a.scale_log2;
+        qs[2 * e + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(raw[e] >> 16)) * a.scale_log2;
+      } else {
+        qs[2 * e] = __builtin_bit_cast(float, raw[e] << 16) * a.scale_log2;
+        qs[2 * e + 1] = __builtin_bit_cast(float, raw[e] & 0xffff0000u) * a.scale_log2;
+      }
+    }
+    return pack8<DT>(qs);
+  };
+  // the first NK k-step fragments of the queries of the block that starts at first_query
+  auto load_q = [&](int first_query, auto &dst, auto nk_tag) __attribute__((always_inline)) {
+    constexpr int NK = decltype(nk_tag)::value;
 #pragma unroll
     for (int qi = 0; qi < QB; ++qi) {
       const int mine = first_query + wave * WQ + qi * 32 + lrow;
       const int qr = mine < S ? mine : S - 1;
       const unsigned short *qp = Qg + (long long)qr * a.q_ss + g * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) dst[qi][ks] = *(const u32x4 *)(qp + ks * 16);
+      for (int ks = 0; ks < NK; ++ks) dst[qi][ks] = prescale(*(const u32x4 *)(qp + ks * 16));
     }
   };
 #pragma unroll
@@ -467,7 +497,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     last_key[qi] = (a.causal && q_mine[qi] < S - 1 ? q_mine[qi] : S - 1) - g * 4;
   }
   wave_last_key = a.causal && q0 + (wave_u + 1) * WQ - 1 < S - 1 ? q0 + (wave_u + 1) * WQ - 1 : S - 1;
-  load_q(q0, qf);
+  load_q(q0, qf, std::integral_constant<int, KS>{});
 
   auto k_piece = [&](int row, int c) __attribute__((always_inline)) -> int {
     return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
@@ -561,8 +591,27 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     load_v(1, sVbase + TILE_BYTES);
     load_k(2, sKbase + 2 * TILE_BYTES);
   }
-  u32x4 qf_next[ITEMS > 1 ? QB : 1][KS];  // the second item's queries travel with the first tiles
-  if constexpr (ITEMS > 1) load_q(item_block(1) * BQ, qf_next);
+  // The second item's queries travel with the first tiles.  PARK: the upper half of their k-steps waits in LDS
+  // behind the rings (fetched there directly, each lane's fragment in a slot of its own) instead of in
+  // registers: the 16 registers that the -m block of SHIFT needs at head dimension 128.
+  constexpr int KQN = PARK ? KS / 2 : KS;  // k-step fragments of the next item's queries kept in registers
+  unsigned char *const sPark = smem + 2 * NSTG * TILE_BYTES;
+  u32x4 qf_next[ITEMS > 1 ? QB : 1][KQN];
+  if constexpr (ITEMS > 1) {
+    load_q(item_block(1) * BQ, qf_next, std::integral_constant<int, KQN>{});
+    if constexpr (PARK) {
+      const int mine = item_block(1) * BQ + wave * WQ + lrow;
+      const int qr = mine < S ? mine : S - 1;
+      __amdgpu_buffer_rsrc_t rsrc_q = __builtin_amdgcn_make_buffer_rsrc(
+          (void *)Qg, 0, (int)(((long long)(S - 1) * a.q_ss + D) * 2), 0x00020000);
+      const unsigned q_voff = (unsigned)(qr * (int)a.q_ss * 2 + g * 16);
+#pragma unroll
+      for (int ks = KQN; ks < KS; ++ks)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrc_q, (__attribute__((address_space(3))) void *)(sPark + ((wave_u * (KS - KQN) + ks - KQN) * 64) * 16), 16,
+            (int)(q_voff + ks * 32), 0, 0, 0);
+    }
+  }
   f32x16 s_cur[QB][2], s_nxt[QB][2];
 
   // Masks tile `tile`'s scores in s (EDGE only) and folds them into the running
@@ -573,10 +622,44 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   float alpha[QB];
 #pragma unroll
   for (int qi = 0; qi < QB; ++qi) alpha[qi] = 1.0f;
+  f32x16 negm[SHIFT ? QB : 1];  // SHIFT: -m_run in every element, where the score product of a tile starts
+  // SHIFT: folds the maxima mx of a tile's z (scores relative to the reference) into the reference.  It moves by
+  // the whole excess once that exceeds TAU (`force`: by whatever it is -- the first tile's case, whose reference
+  // is the arbitrary 0); the tile's z follow, O is rescaled at once, and alpha is the factor the row sum of the
+  // earlier tiles takes with the next tile's sum (exactly 1 where nothing moved).  One branch for all of it.
+  auto fold_shift = [&](const float (&mx)[QB], f32x16 (&z)[QB][2], bool force) __attribute__((always_inline)) {
+    bool moved = false;
+    float step[QB];
+#pragma unroll
+    for (int qi = 0; qi < QB; ++qi) {
+      const float mw = max_with_lane_xor32(mx[qi]);
+      const bool mv = (force & (mw > -INFINITY)) | (mw > FA_RESCALE_TAU);
+      step[qi] = mv ? mw : 0.0f;
+      alpha[qi] = __builtin_amdgcn_exp2f(-step[qi]);
+      m_run[qi] += step[qi];
+      moved |= mv;
+    }
+    if (__any(moved)) {
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) {
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) z[qi][blk][e] -= step[qi];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) negm[SHIFT ? qi : 0][e] = -m_run[qi];
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) o[qi][d][e] *= alpha[qi];
+      }
+    }
+  };
   auto take_max = [&](int tile, auto edge_tag, f32x16 (&s)[QB][2]) -> bool {
     constexpr bool EDGE = decltype(edge_tag)::value;
     const int kv0 = tile * FA_BKV;
     bool moved = false;
+    float mxs[QB];
 #pragma unroll
     for (int qi = 0; qi < QB; ++qi) {
       float mx = -INFINITY;
@@ -587,8 +670,16 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           if constexpr (EDGE) s[qi][blk][e] = blk * 32 + (e >> 2) * 8 + (e & 3) > last_key[qi] - kv0 ? -INFINITY : s[qi][blk][e];
           mx = fmaxf(mx, s[qi][blk][e]);
         }
-      mx = max_with_lane_xor32(mx);
-      moved |= lazy_running_max(m_run[qi], mx * a.scale_log2, alpha[qi]);
+      mxs[qi] = mx;
+      if constexpr (!SHIFT) {
+        mx = max_with_lane_xor32(mx);
+        moved |= lazy_running_max(m_run[qi], mx * a.scale_log2, alpha[qi]);
+      }
+    }
+    if constexpr (SHIFT) {  // (tile 0 of a block: O and the row sum are still zero, the factor stays 1)
+      fold_shift(mxs, s, true);
+#pragma unroll
+      for (int qi = 0; qi < QB; ++qi) alpha[qi] = 1.0f;
     }
     return moved;
   };
@@ -714,14 +805,16 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         for (int qi = 0; qi < QB; ++qi) {
           // (the first k-step starts from the MFMA's constant zero: no 32 registers to clear per tile)
           const f32x16 zero16 = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-          nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], ks == 0 ? zero16 : nxt[qi][0]);
-          nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], ks == 0 ? zero16 : nxt[qi][1]);
+          // (SHIFT: from -m, and the shift of the whole block costs no instruction)
+          nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], ks == 0 ? (SHIFT ? negm[SHIFT ? qi : 0] : zero16) : nxt[qi][0]);
+          nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], ks == 0 ? (SHIFT ? negm[SHIFT ? qi : 0] : zero16) : nxt[qi][1]);
         }
 #pragma unroll
         for (int j = 0; j < EPC; ++j) {
           const int idx = ks * EPC + j;  // 0..32*QB-1 over (query block, blk, element): block idx/32, blk (idx%32)/16
           const int qi = idx >> 5, w = idx & 31;
-          const float x = __builtin_amdgcn_exp2f(fmaf(cur[qi][w >> 4][w & 15], a.scale_log2, -m_run[qi]));
+          const float x = SHIFT ? __builtin_amdgcn_exp2f(cur[qi][w >> 4][w & 15])
+                                : __builtin_amdgcn_exp2f(fmaf(cur[qi][w >> 4][w & 15], a.scale_log2, -m_run[qi]));
           p[idx & 7] = x;
           lsum[qi] += x;
           if ((idx & 7) == 7) pf[qi][w >> 3] = pack8<DT>(p);
@@ -770,13 +863,17 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         if constexpr (QB > 1) MfmaValu<0, DB * QB, (8 * QB * (EDGE ? 4 : 1) + DB * QB - 1) / (DB * QB), 2 * DB>::run();
         __builtin_amdgcn_sched_barrier(0);
       }
-      bool moved = false;
+      if constexpr (SHIFT) {
+        fold_shift(mx, nxt, false);
+      } else {
+        bool moved = false;
 #pragma unroll
-      for (int qi = 0; qi < QB; ++qi) {
-        const float mw = max_with_lane_xor32(mx[qi]);
-        moved |= lazy_running_max(m_run[qi], mw * a.scale_log2, alpha[qi]);
+        for (int qi = 0; qi < QB; ++qi) {
+          const float mw = max_with_lane_xor32(mx[qi]);
+          moved |= lazy_running_max(m_run[qi], mw * a.scale_log2, alpha[qi]);
+        }
+        rescale(moved);
       }
-      rescale(moved);
     }
     if constexpr (decltype(copy_tag)::value) {
 #pragma unroll
@@ -802,7 +899,8 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         float p[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          p[j] = __builtin_amdgcn_exp2f(fmaf(s_cur[qi][w >> 1][(w & 1) * 8 + j], a.scale_log2, -m_run[qi]));
+          p[j] = SHIFT ? __builtin_amdgcn_exp2f(s_cur[qi][w >> 1][(w & 1) * 8 + j])
+                       : __builtin_amdgcn_exp2f(fmaf(s_cur[qi][w >> 1][(w & 1) * 8 + j], a.scale_log2, -m_run[qi]));
           lsum += p[j];
         }
         pf[qi][w] = pack8<DT>(p);
@@ -831,7 +929,10 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
         q_mine[qi] = q_wave0 + qi * 32 + lrow;
         last_key[qi] = (a.causal && q_mine[qi] < S - 1 ? q_mine[qi] : S - 1) - g * 4;
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) qf[qi][ks] = qf_next[qi][ks];
+        for (int ks = 0; ks < KS; ++ks) {
+          if (ks < KQN) qf[qi][ks] = qf_next[qi][ks < KQN ? ks : 0];
+          else qf[qi][ks] = prescale(*(const u32x4 *)(sPark + ((wave * (KS - KQN) + ks - KQN) * 64 + lane) * 16));
+        }
       }
     }
   }
@@ -841,9 +942,13 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     for (int d = 0; d < DB; ++d)
 #pragma unroll
       for (int e = 0; e < 16; ++e) o[qi][d][e] = 0.0f;
-    m_run[qi] = -1.0e30f;
+    m_run[qi] = SHIFT ? 0.0f : -1.0e30f;
     l_run[qi] = 0.0f;
     alpha[qi] = 1.0f;
+    if constexpr (SHIFT) {
+#pragma unroll
+      for (int e = 0; e < 16; ++e) negm[qi][e] = 0.0f;
+    }
   }
   // (a later item finds its first tiles requested by the item before it, and published by that item's last barrier)
   __builtin_amdgcn_s_waitcnt(WAIT_TILES);
@@ -983,15 +1088,17 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 
-template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1, int ITEMS = 1>
+template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1, int ITEMS = 1, bool SHIFT = false>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
-  constexpr size_t lds = 2 * (size_t)NSTG * FA_BKV * D * 2;  // the K and V rings; O leaves from registers
+  // the K and V rings (O leaves from registers), and where they are parked half of the next block's queries
+  constexpr size_t lds = 2 * (size_t)NSTG * FA_BKV * D * 2 +
+                         (fa2_pipe_parks_queries(D, QB, ITEMS, SHIFT) ? (size_t)WAVES * (D / 32) * 1024 : 0);
   const int nqb = (a.S + 32 * QB * WAVES - 1) / (32 * QB * WAVES);
   if (nqb % ITEMS != 0) return (int)hipErrorInvalidValue;  // (feasible_pairs keeps such a call away)
   const dim3 grid((unsigned)(nqb / ITEMS * a.B * a.H)), block(WAVES * 64);
 #define TRACEA_FA_LAUNCH(DTV)                                                                  \
   do {                                                                                         \
-    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB, ITEMS>;                 \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB, ITEMS, SHIFT>;          \
     static bool attr_done = false;                                                             \
     if (!attr_done) {                                                                          \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
@@ -1063,22 +1170,22 @@ static bool feasible_d64(const AttentionArgs &a) { return a.D == 64; }
 // dimension 128 has no 3-stage member: the third set of per-lane tile addresses does not fit the 256
 // registers of two waves per SIMD and the kernel spills.)
 static const AttentionVariant kAttentionVariants[] = {
-    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2>, &feasible_pipe_d128, 32, 1},
-    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d128_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 1, 1, true>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q128_kv64_d64_pipe2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 1, 1, true>, &feasible_pipe_d64, 32, 1},
     {"fa2_q128_kv64_d128_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<128, 4>, &feasible_pipe_d128, 16, 1},
     {"fa2_q128_kv64_d64_m16", 128, FA_BKV, 4, 2, &launch_fa2_m16<64, 4>, &feasible_pipe_d64, 16, 1},
     {"fa2_q256_kv64_d128_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<128, 8>, &feasible_pipe_d128, 16, 1},
     {"fa2_q256_kv64_d64_s2_m16", 256, FA_BKV, 8, 2, &launch_fa2_m16<64, 8>, &feasible_pipe_d64, 16, 1},
-    {"fa2_q128_kv64_d128_pipe2_x2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 1, 2>, &feasible_pairs<128, 128>, 32, 2},
-    {"fa2_q128_kv64_d64_pipe2_x2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 1, 2>, &feasible_pairs<64, 128>, 32, 2},
-    {"fa2_q256_kv64_d128_s2_pipe2_x2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2, 1, 2>, &feasible_pairs<128, 256>, 32, 2},
-    {"fa2_q256_kv64_d64_s2_pipe2_x2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2, 1, 2>, &feasible_pairs<64, 256>, 32, 2},
+    {"fa2_q128_kv64_d128_pipe2_x2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 1, 2, true>, &feasible_pairs<128, 128>, 32, 2},
+    {"fa2_q128_kv64_d64_pipe2_x2", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 1, 2, true>, &feasible_pairs<64, 128>, 32, 2},
+    {"fa2_q256_kv64_d128_s2_pipe2_x2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2, 1, 2, true>, &feasible_pairs<128, 256>, 32, 2},
+    {"fa2_q256_kv64_d64_s2_pipe2_x2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2, 1, 2, true>, &feasible_pairs<64, 256>, 32, 2},
     {"fa2_q256_kv64_d128_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<128, true, 4, 2, 2>, &feasible_pipe_d128, 32, 1},
     {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64, 32, 1},
-    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2>, &feasible_pipe_d128, 32, 1},
-    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2>, &feasible_pipe_d64, 32, 1},
-    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3>, &feasible_pipe_d64, 32, 1},
-    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2, 1, 1, true>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2, 1, 1, true>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3, 1, 1, true>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3, 1, 1, true>, &feasible_pipe_d64, 32, 1},
     {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128, 32, 1},
     {"fa2_q128_kv64_d64_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<64, false, 4, 2>, &feasible_pipe_d64, 32, 1},
     {"fa2_q128_kv64_d128_tr", FA_BQ, FA_BKV, FA_WAVES, 2, &launch_fa2<128, true>, &feasible_d128, 32, 1},

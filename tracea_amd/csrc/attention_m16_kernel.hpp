@@ -13,6 +13,15 @@
 // 0-3 are keys 32 s + 4 g + e, slots 4-7 keys 32 s + 16 + 4 g + e (g = l >> 4), and the V^T operand
 // enumerates the keys in that order: two transposing reads of four consecutive key rows each.
 // O^T block (db, qb): lane l holds query l & 15, head-dim 16 db + 4 g + e.
+//
+// The softmax shift rides the score product.  The queries are multiplied by scale * log2(e) when they are
+// loaded (rounded once more to the operand type: a relative 2^-9 on q, about 2^-9 on a probability), and
+// the first MFMA of every S^T block accumulates onto a register block holding -m, the query's running
+// reference maximum, instead of zero: the product comes out as z = s * scale * log2(e) - m and a
+// probability is one v_exp_f32 of it, without the multiply-add per score that the vector ALU, the busiest
+// unit of this kernel, spent on the shift.  The maximum of a tile is taken of z: while it stays below
+// FA_RESCALE_TAU the reference stays (the lazy running maximum of fa2_fwd_pipe_kernel); when it moves, the
+// tile's z are lowered by the step and O and the row sum rescaled.
 #pragma once
 
 namespace tracea_amd {
@@ -67,7 +76,21 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
     const int qr = q_mine[qb] < S ? q_mine[qb] : S - 1;
     const unsigned short *qp = Qg + (long long)qr * a.q_ss + g4 * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[qb][ks] = *(const u32x4 *)(qp + ks * 32);
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 raw = *(const u32x4 *)(qp + ks * 32);
+      float qs[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if constexpr (DT == DT_F16) {
+          qs[2 * e] = (float)__builtin_bit_cast(_Float16, (unsigned short)(raw[e] & 0xffffu)) * a.scale_log2;
+          qs[2 * e + 1] = (float)__builtin_bit_cast(_Float16, (unsigned short)(raw[e] >> 16)) * a.scale_log2;
+        } else {
+          qs[2 * e] = __builtin_bit_cast(float, raw[e] << 16) * a.scale_log2;
+          qs[2 * e + 1] = __builtin_bit_cast(float, raw[e] & 0xffff0000u) * a.scale_log2;
+        }
+      }
+      qf[qb][ks] = pack8<DT>(qs);
+    }
   }
 
   // K tile: 16-byte column XOR row (conflict-free for 16 rows x one column group per 16 lanes).  V tile: the
@@ -147,7 +170,8 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
     for (int d = 0; d < DB; ++d)
 #pragma unroll
       for (int e = 0; e < 4; ++e) o[qb][d][e] = 0.0f;
-  float m_run[2] = {-1.0e30f, -1.0e30f}, l_run[2] = {0.0f, 0.0f}, alpha[2] = {1.0f, 1.0f};
+  float m_run[2] = {0.0f, 0.0f}, l_run[2] = {0.0f, 0.0f}, alpha[2] = {1.0f, 1.0f};
+  f32x4 negm[2];  // -m_run in every element: where the score product of a tile starts
 
   load_k(0, sKbase);
   load_v(0, sVbase);
@@ -155,20 +179,20 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   __syncthreads();
 
-  f32x4 s_cur[2][KB], s_nxt[2][KB];
+  f32x4 s_a[2][KB], s_b[2][KB];  // z of two consecutive tiles; which is which alternates
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) s_cur[qb][kb][e] = 0.0f;
+      for (int e = 0; e < 4; ++e) s_a[qb][kb][e] = 0.0f;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       const u32x4 kf = read_k(sKbase, kb, ks);
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb) s_cur[qb][kb] = Mfma16<DT>::run(kf, qf[qb][ks], s_cur[qb][kb]);
+      for (int qb = 0; qb < 2; ++qb) s_a[qb][kb] = Mfma16<DT>::run(kf, qf[qb][ks], s_a[qb][kb]);
     }
 
   // the maximum of a query's 64 scores: in-lane over 16, then across the four 16-lane groups
@@ -186,56 +210,62 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(b0), "+v"(b1));
     return fmaxf(b0, b1);
   };
-  // Masks tile `tile` (EDGE only) and folds it into the running maximum; leaves the rescale factor of the
-  // earlier tiles in alpha (exactly 1 where the maximum did not move); returns whether a maximum moved.
-  auto fold_max = [&](const float (&mx)[2]) __attribute__((always_inline)) -> bool {
-    bool moved = false;
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-      const float mw = row_max(mx[qb]);
-      moved |= lazy_running_max(m_run[qb], mw * a.scale_log2, alpha[qb]);
-    }
-    return moved;
-  };
-  auto take_max = [&](int tile, auto edge_tag, f32x4 (&s)[2][KB]) __attribute__((always_inline)) -> bool {
-    constexpr bool EDGE = decltype(edge_tag)::value;
+  auto mask_tile = [&](int tile, f32x4 (&z)[2][KB]) __attribute__((always_inline)) {
     const int kv0 = tile * FA_BKV;
-    float mx[2] = {-INFINITY, -INFINITY};
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if constexpr (EDGE) {
-            const int kv = kv0 + kb * 16 + g4 * 4 + e;
-            const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine[qb]));
-            s[qb][kb][e] = dead ? -INFINITY : s[qb][kb][e];
-          }
-          mx[qb] = fmaxf(mx[qb], s[qb][kb][e]);
+          const int kv = kv0 + kb * 16 + g4 * 4 + e;
+          const bool dead = (kv >= S) | ((a.causal != 0) & (kv > q_mine[qb]));
+          z[qb][kb][e] = dead ? -INFINITY : z[qb][kb][e];
         }
-    return fold_max(mx);
   };
-  auto rescale = [&](bool moved) __attribute__((always_inline)) {
+  // Folds the maxima mx (of z, i.e. relative to the reference) of a tile into the reference: it moves by the
+  // whole excess once that exceeds TAU (`force`: by whatever it is, the first tile's case, whose reference
+  // is the arbitrary 0), the tile's z follow, O is rescaled at once and alpha is the factor the row sum of the
+  // earlier tiles takes with the next tile's sum (exactly 1 where nothing moved).
+  auto fold_max = [&](const float (&mx)[2], f32x4 (&z)[2][KB], bool force) __attribute__((always_inline)) {
+    bool moved = false;
+    float step[2];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+      const float mw = row_max(mx[qb]);
+      const bool mv = (force & (mw > -INFINITY)) | (mw > FA_RESCALE_TAU);
+      step[qb] = mv ? mw : 0.0f;
+      alpha[qb] = __builtin_amdgcn_exp2f(-step[qb]);
+      m_run[qb] += step[qb];
+      moved |= mv;
+    }
+    // (one branch for everything a moving reference touches: the multiplies are skipped unless some lane of
+    // the wave needs them, alpha being exactly 1 and the step 0 for every other lane)
     if (__any(moved)) {
 #pragma unroll
-      for (int qb = 0; qb < 2; ++qb)
+      for (int qb = 0; qb < 2; ++qb) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) z[qb][kb][e] -= step[qb];
+        negm[qb] = f32x4{-m_run[qb], -m_run[qb], -m_run[qb], -m_run[qb]};
 #pragma unroll
         for (int d = 0; d < DB; ++d)
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[qb][d][e] *= alpha[qb];
+      }
     }
   };
 
   u32x4 pf[2][PS];
-  // One iteration, compiled twice (EDGE: the tile whose maximum the iteration takes, t+1, reaches the end of
-  // the sequence or the causal diagonal).  Both phases are short chunks of MFMAs and their share of the
-  // vector work, each closed by a scheduling fence.
-  auto iteration = [&](int t, auto edge_tag) __attribute__((always_inline)) {
+  // One iteration, compiled for both roles of the score arrays and twice more for EDGE (the tile whose
+  // maximum the iteration takes, t+1, reaches the end of the sequence or the causal diagonal).  Both phases
+  // are short chunks of MFMAs and their share of the vector work, each closed by a scheduling fence.
+  auto iteration = [&](int t, auto edge_tag, f32x4 (&s_cur)[2][KB], f32x4 (&s_nxt)[2][KB]) __attribute__((always_inline)) {
     constexpr bool EDGE = decltype(edge_tag)::value;
     const unsigned char *sV = sVbase + (t % NSTG) * TILE_BYTES;
     const unsigned char *sKn = sKbase + ((t + 1) % NSTG) * TILE_BYTES;
-    // ---- phase A: S^T(t+1) = K(t+1) Q^T  with  P(t) = exp2(S(t) * scale - m) and its row sums ----
+    // ---- phase A: z(t+1) = K(t+1) Q'^T - m  with  P(t) = exp2(z(t)) and its row sums ----
     constexpr int EPC = 32 / KS;  // exponentials per chunk (of the lane's 32 scores)
     static_assert(EPC == 8 || EPC == 16, "exponentials must come in groups of eight");
     __builtin_amdgcn_sched_barrier(0);
@@ -252,13 +282,13 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)  // (the first k-step starts from the MFMA's constant zero: no registers to clear)
-          s_nxt[qb][kb] = Mfma16<DT>::run(kf[kb], qf[qb][ks], ks == 0 ? f32x4{0.0f, 0.0f, 0.0f, 0.0f} : s_nxt[qb][kb]);
+        for (int qb = 0; qb < 2; ++qb)  // (the first k-step starts from -m: the shift costs no instruction)
+          s_nxt[qb][kb] = Mfma16<DT>::run(kf[kb], qf[qb][ks], ks == 0 ? negm[qb] : s_nxt[qb][kb]);
 #pragma unroll
       for (int j = 0; j < EPC; ++j) {
         const int idx = ks * EPC + j;  // over (query block, key block, element): 16 per query block
         const int qb = idx >> 4, kb = (idx & 15) >> 2, e = idx & 3;
-        const float x = __builtin_amdgcn_exp2f(fmaf(s_cur[qb][kb][e], a.scale_log2, -m_run[qb]));
+        const float x = __builtin_amdgcn_exp2f(s_cur[qb][kb][e]);
         p[idx & 7] = x;
         lsum[qb] += x;
         if ((idx & 7) == 7) pf[qb][kb >> 1] = pack8<DT>(p);
@@ -272,9 +302,9 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) l_run[qb] = l_run[qb] * alpha[qb] + lsum[qb];
 
-    // ---- phase B: O^T += V^T(t) P^T(t)  with  the running maximum of tile t+1 ----
+    // ---- phase B: O^T += V^T(t) P^T(t)  with  the maximum of tile t+1 ----
     // chunk c: key step c / 2, head-dim blocks (c % 2) * DB/2 .. + DB/2, and the maximum over 8 of the 32
-    // scores of S(t+1)
+    // scores of z(t+1)
     const int kv0n = (t + 1) * FA_BKV;
     float mx[2] = {-INFINITY, -INFINITY};
     constexpr int HB = DB / 2;
@@ -304,11 +334,7 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    rescale(fold_max(mx));
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) s_cur[qb][kb] = s_nxt[qb][kb];
+    fold_max(mx, s_nxt, false);
   };
 
   // interior tiles first, then the edge tiles (the tail of the sequence and, under a causal mask, the
@@ -320,23 +346,60 @@ fa2_fwd_m16_kernel(const AttentionArgs a) {
     first_edge = fe < first_edge ? fe : first_edge;
   }
   first_edge = __builtin_amdgcn_readfirstlane(first_edge);
-  if (first_edge == 0) (void)take_max(0, std::true_type{}, s_cur);
-  else (void)take_max(0, std::false_type{}, s_cur);
+  {  // tile 0: its maximum becomes the reference, whatever it is
+    if (first_edge == 0) mask_tile(0, s_a);
+    float mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mx[qb] = fmaxf(mx[qb], s_a[qb][kb][e]);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) negm[qb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    fold_max(mx, s_a, true);
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) alpha[qb] = 1.0f;
+  }
   const int interior_end = first_edge - 1;
-  int t = 0;
-  for (; t < interior_end; ++t) {
+  auto step = [&](int t, auto edge_tag, f32x4 (&s_cur)[2][KB], f32x4 (&s_nxt)[2][KB]) __attribute__((always_inline)) {
     __builtin_amdgcn_s_waitcnt(0x0f70);  // K(t+1) and V(t)
     __syncthreads();
     load_k(t + NSTG, sKbase + (t % NSTG) * TILE_BYTES);
     load_v(t + NSTG - 1, sVbase + ((t + NSTG - 1) % NSTG) * TILE_BYTES);
-    iteration(t, std::false_type{});
+    iteration(t, edge_tag, s_cur, s_nxt);
+  };
+  // D = 64: interior tiles in pairs whose second step has the arrays in the other roles (an odd tile first,
+  // with a copy); the few edge tiles copy.  D = 128 has no registers for the doubled loop body (150-200 bytes
+  // of scratch per lane) and copies every tile's z into place.
+  constexpr bool SWAP = D <= 64;
+  auto copy_back = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) s_a[qb][kb] = s_b[qb][kb];
+  };
+  int t = 0;
+  const int n_int = interior_end > 0 ? interior_end : 0;
+  if constexpr (SWAP) {
+    if (n_int & 1) {
+      step(0, std::false_type{}, s_a, s_b);
+      copy_back();
+      t = 1;
+    }
+    for (; t < n_int; t += 2) {
+      step(t, std::false_type{}, s_a, s_b);
+      step(t + 1, std::false_type{}, s_b, s_a);
+    }
+  } else {
+    for (; t < n_int; ++t) {
+      step(t, std::false_type{}, s_a, s_b);
+      copy_back();
+    }
   }
   for (; t < ntiles; ++t) {
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    load_k(t + NSTG, sKbase + (t % NSTG) * TILE_BYTES);
-    load_v(t + NSTG - 1, sVbase + ((t + NSTG - 1) % NSTG) * TILE_BYTES);
-    iteration(t, std::true_type{});
+    step(t, std::true_type{}, s_a, s_b);
+    copy_back();
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);  // look-ahead loads must not land on the output staging
   __syncthreads();

@@ -2203,8 +2203,10 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
   // B*H in {8, 32, 128, 512} and S in {512 ... 8192}, replayed graphs: with at least one pair per CU the paired
   // member wins or ties (causal B4 H32 S4096 D128 585 -> 553 us, B1 H32 S2048 63.8 -> 52.2; dense B4 H32 S4096
   // 1002 -> 980 on eight waves), with fewer it loses (causal B1 H32 S1024 26.2 -> 30.1).
+  // (Dense attention no longer takes the pairs by rule: with the softmax shift folded into the score product,
+  // which the paired members at head dimension 128 have no registers for, the one-block eight-wave member below
+  // is ahead -- B4 H32 S4096 D128 904 us against 964, B8 H32 S2048 D64 294 against 302, same box.)
   if (vi < 0 && a.causal && bh * (((S + 127) / 128) / 2) >= cus) vi = member(128, 4, 2);
-  if (vi < 0 && !a.causal && bh * (((S + 255) / 256) / 2) >= cus) vi = member(256, 8, 2);
   // Dense attention over a long sequence with enough workgroups to go round: 256 queries on eight waves share
   // every K/V tile (B4 H32 S4096 D128: 997-999 us against 1013 for 128 queries on four).  Under a causal mask
   // the smaller block wins (584 against 624 us: less masked work on the diagonal, finer load balance).
