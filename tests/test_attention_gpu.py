@@ -29,7 +29,7 @@ def _tol(d, dtype):
 # 32 queries per wave; a member that a head dimension does not have (3-stage rings at D = 128) is skipped
 FAMILY = [("q128", "pipe"), ("q128", "pipe2"), ("q128", "tr"), ("q128", "u16"), ("q256", "s2_pipe2"),
           ("q256", "s3_pipe2"), ("q128", "s3_pipe2"), ("q256", "w4_pipe2"), ("q128", "m16"), ("q256", "s2_m16"),
-          ("q128", "pipe2_x2"), ("q256", "s2_pipe2_x2")]
+          ("q128", "pipe2_x2"), ("q256", "s2_pipe2_x2"), ("q256", "s2_pp"), ("q256", "s4_pipe2"), ("q128", "s4_pipe2")]
 
 
 def _member(capi, variant, d):

@@ -403,9 +403,20 @@ fa2_fwd_kernel(const AttentionArgs a) {
 // stays; when it moves, the tile's z are lowered by the step and O and the row sum rescaled.  Costs 16
 // registers per query block (the -m block), which the paired members at head dimension 128 do not have.
 constexpr bool fa2_pipe_parks_queries(int d, int qb, int items, bool shift) { return items > 1 && shift && d == 128 && qb == 1; }
-template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB, int ITEMS = 1, bool SHIFT = false>
+//
+// PP: the two waves of a SIMD half an iteration apart.  Phase A of an iteration (exponentials of tile t under
+// the score product of tile t+1) is mostly vector ALU, phase B (P.V of tile t under the maximum of tile t+1)
+// mostly matrix pipe; with one barrier per tile every wave of the workgroup enters phase A together, the two
+// waves of a SIMD contend for the vector ALU while the matrix pipe idles, and then the other way round.  Here
+// the barrier comes twice per tile, between the phases, and waves 4-7 run one phase behind waves 0-3 (they
+// sit out the first slot, waves 0-3 the last): in every slot a SIMD holds one wave in phase A and one in
+// phase B.  K(u+2) is requested by every wave at the barrier that opens slot 2u, V(u+1) at the one that opens
+// slot 2u+1; a request has two slots to land, and a barrier waits for the one before last.  Eight waves, one
+// query block per workgroup, two-stage rings, no causal mask (waves would differ in their number of tiles).
+template <int DT, int D, bool EARLY_MAX, int WAVES, int NSTG, int QB, int ITEMS = 1, bool SHIFT = false, bool PP = false>
 __global__ void __launch_bounds__(WAVES * 64) __attribute__((amdgpu_waves_per_eu(QB == 1 ? 2 : 1, QB == 1 ? 2 : 1)))
 fa2_fwd_pipe_kernel(const AttentionArgs a) {
+  static_assert(!PP || (EARLY_MAX && WAVES == 8 && NSTG == 2 && QB == 1 && ITEMS == 1), "the half-iteration offset exists for eight waves, one block, two stages");
   static_assert(!SHIFT || EARLY_MAX, "the shifted score product exists in the two-phase form only");
   constexpr bool PARK = fa2_pipe_parks_queries(D, QB, ITEMS, SHIFT);
   static_assert(QB == 1 || (QB == 2 && EARLY_MAX), "two query blocks per wave exist in the two-phase form only");
@@ -424,13 +435,19 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   static_assert(D % 32 == 0 && FA_BKV % (RPI * WAVES) == 0, "unsupported head dim");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  static_assert(NSTG == 2 || NSTG == 3, "ring depth");
+  static_assert(NSTG == 2 || NSTG == 3 || NSTG == 4, "ring depth");
+  // Four stages: one barrier for every TWO tiles.  The barrier in front of tiles (t, t+1), t even, publishes
+  // K(t+1), K(t+2), V(t), V(t+1), requested at the barrier before, and the stages of the pair before receive
+  // K(t+3), K(t+4), V(t+2), V(t+3): half the barriers and waits per key, and a request has two tiles to land.
+  constexpr bool PAIR_SYNC = NSTG == 4;
+  static_assert(!PAIR_SYNC || (EARLY_MAX && ITEMS == 1 && !PP), "the two-tile barrier exists for one query block per workgroup");
   unsigned char *const sKbase = smem;                      // NSTG stages
   unsigned char *const sVbase = smem + NSTG * TILE_BYTES;  // NSTG stages
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int lrow = lane & 31, g = lane >> 5;
+  const int grp = wave_u >> 2;  // (PP) 0: waves 0-3, 1: waves 4-7, one phase behind
 
   const int nqb = (a.S + BQ - 1) / BQ;
   const int per_bh = nqb / ITEMS;  // workgroups per (batch, head); the host launches pairs for an even nqb only
@@ -582,11 +599,15 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // tiles at or beyond the end of the sequence lie outside the buffers and load as zeros
   // requests of a wave that may stay in flight where an iteration waits for its tiles: those of the
   // iteration before (NSTG = 3), none (NSTG = 2)
-  constexpr int FLIGHT = (NSTG - 2) * 2 * NI;
+  constexpr int FLIGHT = PAIR_SYNC ? 0 : (NSTG - 2) * 2 * NI;
   constexpr int WAIT_TILES = (FLIGHT & 15) | (7 << 4) | (15 << 8) | ((FLIGHT >> 4) << 14);
   load_k(0, sKbase);
   load_v(0, sVbase);
   load_k(1, sKbase + TILE_BYTES);
+  if constexpr (PAIR_SYNC) {
+    load_k(2, sKbase + 2 * TILE_BYTES);
+    load_v(1, sVbase + TILE_BYTES);
+  }
   if constexpr (NSTG == 3) {
     load_v(1, sVbase + TILE_BYTES);
     load_k(2, sKbase + 2 * TILE_BYTES);
@@ -745,6 +766,61 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     return vf;
   };
 
+  // The barrier at the head of iteration t publishes K(t+1) and V(t) and retires K(t) and V(t-1),
+  // whose stages then receive K(t+NSTG) and V(t+NSTG-1).  PP: the barrier that opens the slot of this wave's
+  // phase A of tile tt (head_of) or phase B (mid_of), with the slot's share of requests (see the kernel's head).
+  constexpr int WAIT_ONE_BATCH = (NI & 15) | (7 << 4) | (15 << 8) | ((NI >> 4) << 14);  // all but the latest NI requests
+  // (PP) what a wave requests at the barrier in front of its phase A (h) and of its phase B (m), by group, as
+  // data: a branch on the group inside the iteration cost the register allocation 64 bytes of scratch
+  const bool odd_grp = PP && grp != 0;
+  const __amdgpu_buffer_rsrc_t rsrc_h = odd_grp ? rsrc_v : rsrc_k, rsrc_m = odd_grp ? rsrc_k : rsrc_v;
+  unsigned char *const base_h = odd_grp ? sVbase : sKbase, *const base_m = odd_grp ? sKbase : sVbase;
+  const unsigned adv_h = (unsigned)(FA_BKV * 2) * (unsigned)(odd_grp ? a.v_ss : a.k_ss);
+  const unsigned adv_m = (unsigned)(FA_BKV * 2) * (unsigned)(odd_grp ? a.k_ss : a.v_ss);
+  unsigned voff_h[NI], voff_m[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i) {
+    voff_h[i] = odd_grp ? v_voff[i] : k_voff[i];
+    voff_m[i] = odd_grp ? k_voff[i] : v_voff[i];
+  }
+  auto slot_load = [&](__amdgpu_buffer_rsrc_t rsrc, const unsigned (&voff)[NI], unsigned adv, unsigned char *dst) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc, (__attribute__((address_space(3))) void *)(dst + (i * WAVES + wave_u) * RPI * ROW_BYTES), 16,
+          (int)(voff[i] + adv), 0, 0, 0);
+  };
+  auto head_of = [&](int tt) __attribute__((always_inline)) {
+    if constexpr (PP) {
+      __builtin_amdgcn_s_waitcnt(WAIT_ONE_BATCH);
+      __builtin_amdgcn_s_barrier();
+      // waves 0-3: K(tt+2) into stage tt % 2; waves 4-7: V(tt+1) into stage (tt+1) % 2
+      slot_load(rsrc_h, voff_h, (unsigned)(tt + 2 - grp) * adv_h, base_h + ((tt + grp) % NSTG) * TILE_BYTES);
+    } else if constexpr (PAIR_SYNC) {
+      if ((tt & 1) == 0) {
+        __builtin_amdgcn_s_waitcnt(WAIT_TILES);
+        __syncthreads();
+        load_k(tt + 3, sKbase + ((tt + 3) % NSTG) * TILE_BYTES);
+        load_v(tt + 2, sVbase + ((tt + 2) % NSTG) * TILE_BYTES);
+        load_k(tt + 4, sKbase + ((tt + 4) % NSTG) * TILE_BYTES);
+        load_v(tt + 3, sVbase + ((tt + 3) % NSTG) * TILE_BYTES);
+      }
+    } else {
+      __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(tt+1) and V(tt), requested NSTG-1 iterations ago
+      __syncthreads();
+      load_k(ahead(tt + NSTG), sKbase + ((tb + tt) % NSTG) * TILE_BYTES);
+      load_v(ahead(tt + NSTG - 1), sVbase + ((tb + tt + NSTG - 1) % NSTG) * TILE_BYTES);
+    }
+  };
+  auto mid_of = [&](int tt) __attribute__((always_inline)) {
+    if constexpr (PP) {
+      __builtin_amdgcn_s_waitcnt(WAIT_ONE_BATCH);
+      __builtin_amdgcn_s_barrier();
+      // waves 0-3: V(tt+1) into stage (tt+1) % 2; waves 4-7: K(tt+3) into stage (tt+1) % 2
+      slot_load(rsrc_m, voff_m, (unsigned)(tt + 1 + 2 * grp) * adv_m, base_m + ((tt + 1) % NSTG) * TILE_BYTES);
+    }
+  };
+
   // One iteration, compiled twice: EDGE tiles (sequence end or causal diagonal)
   // mask scores with selects, interior tiles do not test at all.  Either body is
   // branch-free up to the optional rescale, so MFMAs and vector-ALU work can be
@@ -833,6 +909,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
       for (int qi = 0; qi < QB; ++qi) l_run[qi] = l_run[qi] * alpha[qi] + lsum[qi];
       __builtin_amdgcn_s_setprio(0);
+      mid_of(t);
 
       // ---- phase B: O^T += V^T(t) P^T(t)  with  the running maximum of tile t+1 ----
       // chunk kk: the DB*QB MFMAs of key block kk (operand reads one fragment ahead) and
@@ -907,6 +984,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       }
       l_run[qi] = l_run[qi] * alpha[qi] + lsum;
     }
+    mid_of(t);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
@@ -974,14 +1052,14 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // body is the interior one while that tile is interior
   const int interior_end = EARLY_MAX ? first_edge - 1 : first_edge;
   int t = 0;
-  // The barrier at the head of iteration t publishes K(t+1) and V(t) and retires K(t) and V(t-1),
-  // whose stages then receive K(t+NSTG) and V(t+NSTG-1).
-  auto head_of = [&](int tt) __attribute__((always_inline)) {
-    __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(tt+1) and V(tt), requested NSTG-1 iterations ago
-    __syncthreads();
-    load_k(ahead(tt + NSTG), sKbase + ((tb + tt) % NSTG) * TILE_BYTES);
-    load_v(ahead(tt + NSTG - 1), sVbase + ((tb + tt + NSTG - 1) % NSTG) * TILE_BYTES);
-  };
+  // (PP) waves 4-7 sit out the first slot
+  if constexpr (PP) {
+    if (grp == 1) {
+      __builtin_amdgcn_s_waitcnt(WAIT_ONE_BATCH);
+      __builtin_amdgcn_s_barrier();
+      load_k(2, sKbase);
+    }
+  }
   if constexpr (EARLY_MAX && QB == 1) {
     // Two tiles per trip with the score arrays changing roles, and (two-stage rings) the pairs starting on
     // ring stage 0: a single tile in front if the first one lies on stage 1, a single one behind if one is left.
@@ -1020,22 +1098,21 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     // causal mask that is one and a half iterations of two of the four waves and half an iteration of the others.)
     const int last_live = wave_last_key / FA_BKV;
     for (; t < last_live; ++t) {
-      __builtin_amdgcn_s_waitcnt(WAIT_TILES);
-      __syncthreads();
-      load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
-      load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
+      head_of(t);
       iteration(t, std::true_type{});
     }
-    __builtin_amdgcn_s_waitcnt(WAIT_TILES);
-    __syncthreads();
-    load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
-    load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
+    head_of(t);
     last_live_iteration(t);
     for (++t; t < ntiles; ++t) {
-      __builtin_amdgcn_s_waitcnt(WAIT_TILES);
-      __syncthreads();
-      load_k(ahead(t + NSTG), sKbase + ((tb + t) % NSTG) * TILE_BYTES);
-      load_v(ahead(t + NSTG - 1), sVbase + ((tb + t + NSTG - 1) % NSTG) * TILE_BYTES);
+      head_of(t);
+      mid_of(t);
+    }
+    // (PP) waves 0-3 sit out the last slot
+    if constexpr (PP) {
+      if (grp == 0) {
+        __builtin_amdgcn_s_waitcnt(WAIT_ONE_BATCH);
+        __builtin_amdgcn_s_barrier();
+      }
     }
   } else {
     for (; t < ntiles; ++t) {
@@ -1088,8 +1165,9 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   __builtin_amdgcn_s_waitcnt(0x0f70);
 }
 
-template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1, int ITEMS = 1, bool SHIFT = false>
+template <int D, bool EARLY_MAX, int WAVES, int NSTG, int QB = 1, int ITEMS = 1, bool SHIFT = false, bool PP = false>
 static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream) {
+  if (PP && a.causal) return (int)hipErrorInvalidValue;  // (its feasibility test keeps such a call away)
   // the K and V rings (O leaves from registers), and where they are parked half of the next block's queries
   constexpr size_t lds = 2 * (size_t)NSTG * FA_BKV * D * 2 +
                          (fa2_pipe_parks_queries(D, QB, ITEMS, SHIFT) ? (size_t)WAVES * (D / 32) * 1024 : 0);
@@ -1098,7 +1176,7 @@ static int launch_fa2_pipe(const AttentionArgs &a, int dtype, hipStream_t stream
   const dim3 grid((unsigned)(nqb / ITEMS * a.B * a.H)), block(WAVES * 64);
 #define TRACEA_FA_LAUNCH(DTV)                                                                  \
   do {                                                                                         \
-    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB, ITEMS, SHIFT>;          \
+    auto kfn = fa2_fwd_pipe_kernel<DTV, D, EARLY_MAX, WAVES, NSTG, QB, ITEMS, SHIFT, PP>;      \
     static bool attr_done = false;                                                             \
     if (!attr_done) {                                                                          \
       hipError_t e = hipFuncSetAttribute((const void *)kfn,                                    \
@@ -1127,6 +1205,9 @@ static bool slice_fits(const AttentionArgs &a) {
 // (the running maximum is taken over raw scores, which needs a positive scale)
 static bool feasible_pipe_d128(const AttentionArgs &a) { return a.D == 128 && a.scale_log2 > 0.0f && slice_fits(a); }
 static bool feasible_pipe_d64(const AttentionArgs &a) { return a.D == 64 && a.scale_log2 > 0.0f && slice_fits(a); }
+// (the members whose wave groups run half an iteration apart: no causal mask)
+static bool feasible_dense_d128(const AttentionArgs &a) { return !a.causal && feasible_pipe_d128(a); }
+static bool feasible_dense_d64(const AttentionArgs &a) { return !a.causal && feasible_pipe_d64(a); }
 // Two query blocks per workgroup: an even number of blocks, and at least two K/V tiles in the lightest one.
 template <int D, int BQ>
 static bool feasible_pairs(const AttentionArgs &a) {
@@ -1184,6 +1265,11 @@ static const AttentionVariant kAttentionVariants[] = {
     {"fa2_q256_kv64_d64_w4_pipe2", 256, FA_BKV, 4, 2, &launch_fa2_pipe<64, true, 4, 2, 2>, &feasible_pipe_d64, 32, 1},
     {"fa2_q256_kv64_d128_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2, 1, 1, true>, &feasible_pipe_d128, 32, 1},
     {"fa2_q256_kv64_d64_s2_pipe2", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2, 1, 1, true>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q256_kv64_d128_s4_pipe2", 256, FA_BKV, 8, 4, &launch_fa2_pipe<128, true, 8, 4, 1, 1, true>, &feasible_pipe_d128, 32, 1},
+    {"fa2_q256_kv64_d64_s4_pipe2", 256, FA_BKV, 8, 4, &launch_fa2_pipe<64, true, 8, 4, 1, 1, true>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q128_kv64_d64_s4_pipe2", 128, FA_BKV, 4, 4, &launch_fa2_pipe<64, true, 4, 4, 1, 1, true>, &feasible_pipe_d64, 32, 1},
+    {"fa2_q256_kv64_d128_s2_pp", 256, FA_BKV, 8, 2, &launch_fa2_pipe<128, true, 8, 2, 1, 1, true, true>, &feasible_dense_d128, 32, 1, 1},
+    {"fa2_q256_kv64_d64_s2_pp", 256, FA_BKV, 8, 2, &launch_fa2_pipe<64, true, 8, 2, 1, 1, true, true>, &feasible_dense_d64, 32, 1, 1},
     {"fa2_q256_kv64_d64_s3_pipe2", 256, FA_BKV, 8, 3, &launch_fa2_pipe<64, true, 8, 3, 1, 1, true>, &feasible_pipe_d64, 32, 1},
     {"fa2_q128_kv64_d64_s3_pipe2", 128, FA_BKV, 4, 3, &launch_fa2_pipe<64, true, 4, 3, 1, 1, true>, &feasible_pipe_d64, 32, 1},
     {"fa2_q128_kv64_d128_pipe", 128, FA_BKV, 4, 2, &launch_fa2_pipe<128, false, 4, 2>, &feasible_pipe_d128, 32, 1},

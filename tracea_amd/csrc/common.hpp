@@ -230,6 +230,7 @@ struct AttentionVariant {
   bool (*feasible)(const AttentionArgs &);
   int mfma;   // MFMA shape: 32 (32x32x16) or 16 (16x16x32)
   int items;  // query blocks a workgroup takes one after the other (1 or 2)
+  int offset_groups;  // 1: the two waves of a SIMD run half an iteration apart, two barriers per tile (else 0)
 };
 int attention_variant_count();
 const AttentionVariant &attention_variant(int i);

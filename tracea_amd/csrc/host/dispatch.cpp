@@ -2193,7 +2193,7 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
   auto member = [&](int block_q, int waves, int items) {
     for (int i = 0; i < attention_variant_count(); ++i) {
       const AttentionVariant &v = attention_variant(i);
-      if (v.block_q == block_q && v.waves == waves && v.stages == 2 && v.mfma == 32 && v.items == items && v.feasible(a)) return i;
+      if (v.block_q == block_q && v.waves == waves && v.stages == 2 && v.mfma == 32 && v.items == items && v.offset_groups == 0 && v.feasible(a)) return i;
     }
     return -1;
   };

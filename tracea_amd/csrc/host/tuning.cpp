@@ -242,6 +242,8 @@ PipelineConfig config_for_attention_variant(int index) {
   c.double_buffer = true;
   c.bank_conflict_padding = 0;
   c.fusion_count = (uint32_t)v.items;  // tiles of the output a workgroup takes (src/optimizer/benchmark.rs:131-132)
+  // two wave groups handing the vector ALU and the matrix pipe to each other across a barrier per phase
+  c.barrier_mode = v.offset_groups ? "ProducerConsumer" : "None";
   return c;
 }
 
@@ -252,6 +254,7 @@ int attention_variant_for_config(const PipelineConfig &c, const AttentionArgs &a
     if (c.has_force_num_warps && (uint32_t)v.waves != c.force_num_warps) continue;
     if ((c.intrinsic_shape == "M16N16K4") != (v.mfma == 16)) continue;
     if ((uint32_t)v.items != (c.fusion_count > 1 ? c.fusion_count : 1u)) continue;
+    if ((v.offset_groups != 0) != (c.barrier_mode == "ProducerConsumer")) continue;
     if (v.feasible(a)) return i;
   }
   return -1;
