@@ -332,6 +332,14 @@ void tracea_set_conv_transpose_filter_cache(int32_t enabled);
 void tracea_conv_transpose_filter_cache_clear(void);
 int32_t tracea_last_split_k(void);
 
+/* Shader-clock probe for measurements (no counterpart in the reference).  Enqueues on `stream` a one-wave
+ * kernel that writes `samples` pairs of 64-bit counters to the device buffer `out` (2 * samples entries):
+ * the shader's clock ticks and the device's constant 100 MHz counter, one pair about every gap * 64 clocks
+ * (gap 0..4096).  Run on a stream of its own beside the kernels under measurement, the ratio of the two
+ * counters' increments is the clock frequency the device ran them at.  Returns TRACEA_INVALID_PARAMS for
+ * a null buffer or counts out of range, TRACEA_CUDA_ERROR when the launch fails. */
+TraceaStatus tracea_clock_probe(void *out, int32_t samples, int32_t gap, void *stream);
+
 /* tracea_gemm for callers that cannot allocate device memory: code whose stream is being
  * captured into a HIP graph, tight serving loops, harnesses that forbid hipMalloc.  No
  * counterpart in the reference (its runtime allocates freely).  Arguments, results and errors

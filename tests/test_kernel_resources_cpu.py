@@ -3,9 +3,8 @@ library by tracea_amd/build.py from -Rpass-analysis=kernel-resource-usage).
 
 No kernel of this library is meant to touch scratch memory.  Twice a kernel did after an
 innocent-looking change (a run-time index into the accumulators; the argument block read
-through nested lambdas): the results stayed right and the kernel ran at half speed.  The only
-exceptions are true register spills of the register-staged 256x256 tiles (pipeline 1), which
-run only for operands of 2 GiB and more."""
+through nested lambdas): the results stayed right and the kernel ran at half speed.  No
+exceptions: the register-staged 256x256 tiles that used to spill are no longer built."""
 import json
 import os
 import re
@@ -35,13 +34,9 @@ def test_no_kernel_uses_scratch_memory():
     bad = []
     for name, r in _resources().items():
         scratch = r.get("scratch_bytes", 0)
-        m = CONTRACTION.search(name)
-        spilling_form = m is not None and m.group(2) == "256" and m.group(3) == "256" and m.group(8) == "1"
-        limit = 256 if spilling_form else 0
-        if scratch > limit:
+        if scratch > 0:
             bad.append((scratch, name))
-        if not spilling_form:
-            assert r.get("vgpr_spills", 0) == 0, name
+        assert r.get("vgpr_spills", 0) == 0, name
     assert not bad, "kernels with a private segment: %s" % sorted(bad, reverse=True)[:8]
 
 

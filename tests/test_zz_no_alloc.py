@@ -36,7 +36,7 @@ def _pair(tracea_gpu, capi, m, n, k, dtype, seed, epilogue="bias+relu"):
 
 def test_two_calls_in_a_row_match_tracea_gemm(tracea_gpu):
     from tracea_amd import capi
-    capi.lib().tracea_set_split_k(1)
+    capi.lib().tracea_set_split_k(1)  # (on: the library's default, stated here because these shapes rely on it)
     for dtype in (torch.float16, torch.bfloat16):
         assert _pair(tracea_gpu, capi, 196, 256, 2304, dtype, 1) >= 2      # split, 196*256*4*splits bytes
         assert _pair(tracea_gpu, capi, 49, 136, 2120, dtype, 2) >= 2       # smaller, K tail, on the stale workspace

@@ -145,6 +145,7 @@ SIGNATURES = {
     "tracea_set_conv_transpose_filter_cache": (None, [C.c_int32]),
     "tracea_conv_transpose_filter_cache_clear": (None, []),
     "tracea_last_split_k": (C.c_int32, []),
+    "tracea_clock_probe": (C.c_int, [C.c_void_p, C.c_int32, C.c_int32, C.c_void_p]),
     "tracea_variant_count": (C.c_int32, [C.c_char_p]),
     "tracea_variant_name": (C.c_char_p, [C.c_char_p, C.c_int32]),
     "tracea_force_variant": (C.c_int32, [C.c_char_p, C.c_int32]),

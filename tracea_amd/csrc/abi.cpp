@@ -163,6 +163,10 @@ void tracea_set_conv_transpose_filter_cache(int32_t enabled) { set_conv_transpos
 void tracea_conv_transpose_filter_cache_clear(void) { conv_transpose_filter_cache_clear(); }
 int32_t tracea_last_split_k(void) { return last_split_k(); }
 
+TraceaStatus tracea_clock_probe(void *out, int32_t samples, int32_t gap, void *stream) {
+  TRACEA_GUARDED(dispatch_clock_probe(out, samples, gap, stream))
+}
+
 int32_t tracea_variant_count(const char *op) {
   if (op == nullptr) return -1;
   if (!strcmp(op, "gemm") || !strcmp(op, "conv2d")) return contraction_variant_count();

@@ -240,6 +240,10 @@ const AttentionVariant &attention_variant(int i);
 int launch_fill_uniform(void *ptr, size_t n, int dtype, unsigned seed, float amplitude,
                         hipStream_t stream);
 
+// One-wave kernel that samples (shader clock ticks, 100 MHz counter) `samples` times, about gap*64 clocks
+// apart, into out[2*samples]; returns hipError_t as int.
+int launch_clock_probe(unsigned long long *out, int samples, int gap, hipStream_t stream);
+
 int launch_conv_coords(const TraceaConvParamsBlock &p, int32_t *rows, int64_t *base_off,
                        int32_t *cols, hipStream_t stream);
 

@@ -2226,4 +2226,12 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
                     attention_variant(vi).launch(a, q.dtype, (hipStream_t)params.stream));
 }
 
+TraceaStatus dispatch_clock_probe(void *out, int32_t samples, int32_t gap, void *stream) {
+  if (!runtime_ready()) return fail(TRACEA_UNKNOWN_ERROR, "tracea_init has not been called");
+  if (out == nullptr || samples <= 0 || samples > (1 << 20) || gap < 0 || gap > 4096)
+    return fail(TRACEA_INVALID_PARAMS, "tracea_clock_probe: out must be a device buffer of 2*samples 64-bit words, "
+                                       "samples in 1..2^20, gap in 0..4096");
+  return hip_status("clock probe launch", launch_clock_probe((unsigned long long *)out, samples, gap, (hipStream_t)stream));
+}
+
 }  // namespace tracea_amd

@@ -106,6 +106,9 @@ TraceaStatus dispatch_attention(const TraceaTensorView &q, const TraceaTensorVie
                                 const TraceaTensorView &v, TraceaTensorView *o,
                                 const TraceaAttentionParams &params);
 
+// Shader-clock probe (tracea_clock_probe): argument checks, then the one-wave sampling kernel on `stream`.
+TraceaStatus dispatch_clock_probe(void *out, int32_t samples, int32_t gap, void *stream);
+
 // Heuristic choice among the feasible contraction variants (used when neither a
 // forced variant nor a tuning-cache entry decides).  Returns -1 if none fits.
 int select_contraction_variant(int m, int n, int k, bool conv, bool b_ncontig = false);

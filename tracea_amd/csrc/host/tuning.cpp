@@ -654,6 +654,7 @@ TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
     probe.S = (int)s;
     probe.k_ss = probe.v_ss = (long long)d;
     probe.scale_log2 = 1.0f;
+    probe.causal = causal ? 1 : 0;
     if (!attention_variant(i).feasible(probe)) continue;
     set_forced_variant("attention", i);
     const double t = time_launches(
@@ -662,6 +663,8 @@ TraceaResult tune_fa2(size_t b, size_t h, size_t s, size_t d, bool causal) {
       err = last_error_text();
       continue;
     }
+    // (a member that cannot run the problem gives way to the rule's choice: that time is not this member's)
+    if (last_variant("attention") != i) continue;
     const double tf = flops / t * 1e-12;
     if (tf > best_tflops) {
       best_tflops = tf;

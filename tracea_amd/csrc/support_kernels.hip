@@ -624,4 +624,28 @@ int launch_fill_uniform(void *ptr, size_t n, int dtype, unsigned seed, float amp
   return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Shader-clock probe: one wave that, `samples` times, writes the pair (s_memtime = shader clock ticks,
+// s_memrealtime = the constant 100 MHz counter) and sleeps for about `gap` times 64 clocks.  Launched on
+// a stream of its own beside the kernels under measurement it shares their clock domain and costs them a
+// wave slot on one CU; the slope of ticks over real time between two samples is the clock the device ran
+// at in between.  The loop is bounded by its arguments and waits for nothing.
+// ---------------------------------------------------------------------------
+__global__ void clock_probe_kernel(unsigned long long *out, int samples, int gap) {
+  if (threadIdx.x != 0) return;
+  for (int i = 0; i < samples; ++i) {
+    const unsigned long long ticks = __builtin_amdgcn_s_memtime();
+    const unsigned long long real = __builtin_amdgcn_s_memrealtime();
+    out[2 * i] = ticks;
+    out[2 * i + 1] = real;
+    for (int g = 0; g < gap; ++g) __builtin_amdgcn_s_sleep(64);
+  }
+}
+
+int launch_clock_probe(unsigned long long *out, int samples, int gap, hipStream_t stream) {
+  if (out == nullptr || samples <= 0 || samples > (1 << 20) || gap < 0 || gap > 4096) return (int)hipErrorInvalidValue;
+  hipLaunchKernelGGL(clock_probe_kernel, dim3(1), dim3(64), 0, stream, out, samples, gap);
+  return (int)hipGetLastError();
+}
+
 }  // namespace tracea_amd
