@@ -188,14 +188,66 @@ def test_filter_resident_variant(tracea_gpu, dtype, member, cin):
         capi.force_variant("conv2d", -1)
 
 
-@pytest.mark.parametrize("member,cin", LDS_MEMBERS)
+# the members for few pixels and many channels (K split over the waves of a workgroup)
+KSPLIT_MEMBERS = [("c112x64_c256_s4_w16_ksplit", 256), ("c64x64_c512_s4_w16_ksplit", 512)]
+KSPLIT_SHAPES = [  # n, h, w, k, filter size, stride, pad, dilation
+    (32, 14, 14, 256, 3, 1, 1, 1),    # a ResNet's 14x14 stage at batch 32: tiles of 98 pixels (7 rows) at 256 channels
+    (32, 7, 7, 512, 3, 1, 1, 1),      # its 7x7 stage: one tile of 49 pixels per image
+    (2, 14, 14, 64, 3, 1, 1, 1),      # small launch: tiles of one pixel block
+    (16, 14, 14, 128, 3, 1, 1, 1),    # tiles of 25 pixels that start and end inside rows
+    (1, 13, 9, 40, 3, 1, 1, 1),       # 40 filters: partial channel groups (general epilogue)
+    (2, 15, 7, 64, 3, 2, 1, 1),       # stride 2
+    (1, 12, 10, 64, 3, 1, 2, 2),      # dilation 2
+    (2, 9, 12, 64, 3, 1, 0, 1),       # no padding
+    (1, 5, 20, 64, 3, 1, (1, 3), 1),  # wide rows, asymmetric padding
+    (8, 14, 14, 128, 1, 1, 0, 1),     # 1x1 filter: two stages in all
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("member,cin", KSPLIT_MEMBERS)
+def test_ksplit_variant(tracea_gpu, dtype, member, cin):
+    """The kernels that split K over the waves of a workgroup (patch in LDS, filters through a ring of
+    128-channel stages, partial sums added in wave order), forced, against torch in double and the oracle."""
+    from tracea_amd import capi
+    names = capi.variants("conv2d")
+    assert member in names, "no member %s in the build" % member
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rnd = round_f16 if dtype == "f16" else round_bf16
+    capi.force_variant("conv2d", names.index(member))
+    try:
+        for shape in KSPLIT_SHAPES:
+            n, h, w, k, fs, stride, pad, dil = shape
+            kg = fs * fs * cin
+            rng = np.random.default_rng(h * 31 + w + k)
+            x = rnd(rng.standard_normal((n, h, w, cin)))
+            wk = rnd(rng.standard_normal((k, fs, fs, cin)) * np.sqrt(2.0 / kg))
+            bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+            ref = torch.nn.functional.conv2d(
+                torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
+                bias=torch.from_numpy(bias).double(), stride=stride, padding=pad, dilation=dil)
+            ref = torch.relu(ref).permute(0, 2, 3, 1).numpy()
+            if isinstance(pad, int) and n <= 16:  # the oracle takes symmetric geometry: torch is cross-checked with it
+                acc = oracle.conv2d_nhwc(x, np.ascontiguousarray(wk.transpose(1, 2, 3, 0)), stride, pad, dil)
+                want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+                assert np.abs(want - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+            y = tracea_gpu.conv2d(_dev(x, tdt), _dev(wk, tdt), bias=_dev(bias), stride=stride, padding=pad,
+                                  dilation=dil, epilogue="bias+relu")
+            assert capi.last_variant("conv2d") == member, "%s refused %s" % (member, shape)
+            assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(kg, dtype), "%s %s %s" % (member, dtype, shape))
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
+@pytest.mark.parametrize("member,cin", LDS_MEMBERS + KSPLIT_MEMBERS)
 def test_filter_resident_variant_operator_chains(tracea_gpu, member, cin):
     """Every form of their straight-line epilogue ([affine] [ReLU] [residual] [ReLU]) and chains outside it
     (SiLU and GELU among them), against the oracle's chain on the oracle's accumulator."""
     from tracea_amd import capi
     names = capi.variants("conv2d")
     vi = names.index(member)
-    n, h, w, k = 2, 18, 25, 64
+    # (the K-split members on a launch that gives them tiles of four pixel blocks)
+    n, h, w, k = (2, 18, 25, 64) if cin < 256 else (128, 10, 10, 64)
     kg = 9 * cin
     rng = np.random.default_rng(77)
     x = round_f16(rng.standard_normal((n, h, w, cin)))

@@ -5,6 +5,7 @@
 #include "conv_patch_kernel.hpp"
 #include "conv_resident_kernel.hpp"
 #include "conv_wave16_kernel.hpp"
+#include "conv_ksplit16_kernel.hpp"
 
 #define TRACEA_CAT2(a, b) a##b
 #define TRACEA_CAT(a, b) TRACEA_CAT2(a, b)
@@ -28,6 +29,9 @@ const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
 #elif V_DIRECT == 8
       (size_t)V_STAGES * cw_ring_stage_bytes(V_BK) + CW_TABLE_BYTES,  // the patch comes on top
       &launch_conv_wave16<V_BK, (V_BM / 16 - 1) / 4, V_STAGES>, 16};
+#elif V_DIRECT == 9
+      (size_t)V_STAGES * CK_STAGE_BYTES + CK_TABLE_BYTES,  // the patch comes on top
+      &launch_conv_ksplit16<V_BK, V_BM / 16, V_STAGES>, 16};
 #elif V_DIRECT == 6
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
       &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, 2, 16>, 16};  // pipeline 2 on 16x16x32 MFMAs

@@ -31,7 +31,7 @@
 // one 16-byte store; a residual is fetched in that layout, 16 bytes per lane, and taken back to the
 // accumulators' layout by the same swap.  Any other chain goes through LDS and the general operator loop.
 #pragma once
-#include "contraction_kernel.hpp"
+#include "conv_epilogue16.hpp"
 
 namespace tracea_amd {
 
@@ -74,7 +74,9 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   const int taps = args.r_sz * args.s_sz;
   const int CPB = RING ? RCPB : ((K >> 3) | 1);
   const int filt_bytes = RING ? RING * RSTAGE : (64 * CPB + NT - 1) / NT * NT * 16;
-  float *table = (float *)(filt + filt_bytes);
+  // (the operand table lies behind the operands or, if that is more, behind the general epilogue's staging)
+  const int operand_bytes = args.p_np_bytes + filt_bytes, staging_bytes = args.p_tm * (BN + 4) * 4;
+  float *table = (float *)(smem + (operand_bytes > staging_bytes ? operand_bytes : staging_bytes));
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -397,119 +399,32 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
         (void *)((const unsigned short *)args.fe.res + ((sig & 4) ? m_img * args.fe.res_ld + n0 : 0ll)), 0,
         (sig & 4) ? (int)((long long)npix * args.fe.res_ld * 2) : 0, 0x00020000);
     const int row_c = (int)args.ldc * 2, row_r = (int)args.fe.res_ld * 2;
-    auto pack2 = [](float x, float y) __attribute__((always_inline)) -> unsigned {
-      if constexpr (DT == DT_F16) {
-        const f16x2 h = {(_Float16)x, (_Float16)y};
-        return __builtin_bit_cast(unsigned, h);
-      } else {
-        const bf16x2 h = {(__bf16)x, (__bf16)y};
-        return __builtin_bit_cast(unsigned, h);
-      }
-    };
-    auto unpack2 = [](unsigned u, float &x, float &y) __attribute__((always_inline)) {
-      if constexpr (DT == DT_F16) {
-        const f16x2 h = __builtin_bit_cast(f16x2, u);
-        x = (float)h[0];
-        y = (float)h[1];
-      } else {
-        x = __builtin_bit_cast(float, u << 16);
-        y = __builtin_bit_cast(float, u & 0xffff0000u);
-      }
-    };
+    int fb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fb[i] = w ^ i;
     auto run_form = [&](auto form) __attribute__((always_inline)) {
-      constexpr int F = decltype(form)::value;
-      constexpr bool AFF = (F & 1) != 0, RELU1 = (F & 2) != 0, RES = (F & 4) != 0, RELU2 = (F & 8) != 0;
-      // the chain's last ReLU on the packed halves (one v_pk_max_f16 per two values; rounding is monotonic
-      // and keeps zero, so max before or after it is the same value)
-      constexpr bool PK = DT == DT_F16 && (RELU2 || (RELU1 && !RES));
-      constexpr bool RELU1_F32 = RELU1 && !(PK && !RES), RELU2_F32 = RELU2 && !PK;
+      using E = Epilogue16<DT, decltype(form)::value>;
       f32x4 ta[4] = {}, tb[4] = {};
-      if constexpr (AFF) {
+      if constexpr (E::AFF) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          ta[i] = *(const f32x4 *)(table + (w ^ i) * 16 + q * 4);
-          tb[i] = *(const f32x4 *)(table + BN + (w ^ i) * 16 + q * 4);
+          ta[i] = *(const f32x4 *)(table + fb[i] * 16 + q * 4);
+          tb[i] = *(const f32x4 *)(table + BN + fb[i] * 16 + q * 4);
         }
       }
-      auto finish = [&](f32x4 v, f32x4 a, f32x4 b, float r0, float r1, float r2, float r3) __attribute__((always_inline)) -> f32x4 {
-        if constexpr (AFF) v = v * a + b;
-        if constexpr (RELU1_F32) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = fmaxf(0.0f, v[e]);
-        }
-        if constexpr (RES) {
-          v[0] += r0; v[1] += r1; v[2] += r2; v[3] += r3;
-        }
-        if constexpr (RELU2_F32) {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = fmaxf(0.0f, v[e]);
-        }
-        return v;
-      };
-      auto pack_out = [&](float x, float y) __attribute__((always_inline)) -> unsigned {
-        unsigned u = pack2(x, y);
-        if constexpr (PK) {
-          const f16x2 z = {(_Float16)0.0f, (_Float16)0.0f};
-          u = __builtin_bit_cast(unsigned, __builtin_elementwise_max(__builtin_bit_cast(f16x2, u), z));
-        }
-        return u;
-      };
       static_for<0, PBW>([&](auto pc) {
         constexpr int p = decltype(pc)::value;
         const int pr = (w * PBW + p) * 16 + l15;
-        const int prow = pr < npix ? pr : -1;
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          // lanes of 16-lane group q hold, after the swap, channels (q>>1)*8 .. +7 of filter block w ^ (2j + (q&1))
-          const int ch = (w ^ (2 * j + (q & 1))) * 16 + (q >> 1) * 8;
-          float ra[4] = {0, 0, 0, 0}, rb[4] = {0, 0, 0, 0};
-          if constexpr (RES) {
-            u32x4 r8 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                     rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
-            unsigned r0 = r8[0], r1 = r8[1], r2 = r8[2], r3 = r8[3];
-            asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
-                         : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));
-            unpack2(r0, ra[0], ra[1]);
-            unpack2(r1, ra[2], ra[3]);
-            unpack2(r2, rb[0], rb[1]);
-            unpack2(r3, rb[2], rb[3]);
-          }
-          const f32x4 va = finish(acc[p][2 * j], ta[2 * j], tb[2 * j], ra[0], ra[1], ra[2], ra[3]);
-          const f32x4 vb = finish(acc[p][2 * j + 1], ta[2 * j + 1], tb[2 * j + 1], rb[0], rb[1], rb[2], rb[3]);
-          unsigned a_lo = pack_out(va[0], va[1]), a_hi = pack_out(va[2], va[3]);
-          unsigned b_lo = pack_out(vb[0], vb[1]), b_hi = pack_out(vb[2], vb[3]);
-          // (as instructions: the compiler's builtin for the swap returns its first result twice; the s_nop is the
-          // wait the hardware asks for between a vector-ALU write of an operand and the swap)
-          asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
-                       : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi));
-          const u32x4 row8 = {a_lo, a_hi, b_lo, b_hi};
-          __builtin_amdgcn_raw_buffer_store_b128(row8, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
-        }
+        E::pixel_block(acc[p], fb, ta, tb, pr < npix ? pr : -1, q, rsrc_c, rsrc_r, row_c, row_r);
       });
-      {  // the shared block: filter block w only, 4 channels (8 bytes) per lane
+      {  // the shared block: filter block w only
         const int pr = 4 * PBW * 16 + l15;
-        const int prow = pr < npix ? pr : -1;
-        const int ch = w * 16 + q * 4;
-        float rr[4] = {0, 0, 0, 0};
-        if constexpr (RES) {
-          const u32x2 r4 = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(
-                                                          rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
-          unpack2(r4[0], rr[0], rr[1]);
-          unpack2(r4[1], rr[2], rr[3]);
-        }
-        const f32x4 v = finish(acc_x, ta[0], tb[0], rr[0], rr[1], rr[2], rr[3]);
-        const u32x2 o = {pack_out(v[0], v[1]), pack_out(v[2], v[3])};
-        __builtin_amdgcn_raw_buffer_store_b64(o, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
+        E::single_block(acc_x, ta[0], tb[0], w * 16 + q * 4, pr < npix ? pr : -1, rsrc_c, rsrc_r, row_c, row_r);
       }
     };
-    switch (form_sig) {
-#define TRACEA_CW_FORM(F) case F: run_form(std::integral_constant<int, F>{}); break;
-      TRACEA_CW_FORM(0) TRACEA_CW_FORM(1) TRACEA_CW_FORM(2) TRACEA_CW_FORM(3) TRACEA_CW_FORM(4) TRACEA_CW_FORM(5)
-      TRACEA_CW_FORM(6) TRACEA_CW_FORM(7) TRACEA_CW_FORM(8) TRACEA_CW_FORM(9) TRACEA_CW_FORM(10) TRACEA_CW_FORM(11)
-      TRACEA_CW_FORM(12) TRACEA_CW_FORM(13) TRACEA_CW_FORM(14) TRACEA_CW_FORM(15)
+#define TRACEA_CW_FORM(F) run_form(std::integral_constant<int, F>{})
+    TRACEA_EPILOGUE16_FORMS(form_sig, TRACEA_CW_FORM)
 #undef TRACEA_CW_FORM
-      default: break;
-    }
     return;
   }
 

@@ -1525,6 +1525,71 @@ bool plan_conv_wave16(const ConvGeometry &g, const ContractionVariant &v, bool w
   return true;
 }
 
+// Plan of the K-split kernel (pipeline 9): as plan_conv_wave16, with the patch rows fetched as flat runs
+// of 16-byte chunks (a pixel may be wider than one 64-lane load) and the ring's fixed stage size.
+bool plan_conv_ksplit16(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  const TraceaConvParamsBlock &b = g.block;
+  const int C = b.c_in;
+  if (v.pipeline != 9 || w_ncontig || C != v.bk || C % 256 != 0 || g.k_gemm != b.r_sz * b.s_sz * C) return false;
+  const long long img_bytes = (long long)b.h_in * b.w_in * C * 2;
+  const long long w_bytes = (long long)g.n_gemm * g.k_gemm * 2;
+  if (img_bytes >= (1ll << 31) || w_bytes >= (1ll << 31)) return false;
+  const long long pw = (long long)b.w_in + 2ll * g.pad_w;
+  const long long ph = (long long)b.h_in + 2ll * g.pad_h;
+  if (pw * ph >= (1ll << 30) || (long long)b.h_in * b.w_in >= (1ll << 24)) return false;
+  const long long table_bytes = TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
+  const long long ring_bytes = (long long)v.lds_bytes - table_bytes;
+  const int hw = b.h_out * b.w_out;
+  const int grid_n = (g.n_gemm + v.bn - 1) / v.bn;
+  const long long cus = device_limits().cus;
+  const long long t_min = (hw + v.bm - 1) / v.bm;
+  const long long rounds = ((long long)b.batch * t_min * grid_n + cus - 1) / cus;
+  long long tiles = rounds * cus / ((long long)b.batch * grid_n);
+  if (tiles < t_min) tiles = t_min;
+  if (tiles > (hw + 15) / 16) tiles = (hw + 15) / 16;
+  const int tm = (int)((hw + tiles - 1) / tiles);
+  const int cpp = (C / 8) | 1;
+  const long long row_chunks = pw * cpp;
+  if (row_chunks >= (1ll << 20)) return false;
+  const int seg = (int)((row_chunks + 63) / 64);
+  auto patch_for = [&](int t) -> long long {
+    long long out_rows = 1;
+    for (int p0 = 0; p0 < hw; p0 += t) {
+      const int last = (p0 + t < hw ? p0 + t : hw) - 1;
+      const long long span = last / b.w_out - p0 / b.w_out + 1;
+      if (span > out_rows) out_rows = span;
+    }
+    const long long rows = (out_rows - 1) * g.stride_h + (long long)(b.r_sz - 1) * g.dil_h + 1;
+    return (rows * row_chunks * 16 + 1023) / 1024 * 1024;
+  };
+  const long long room = (long long)device_limits().lds_bytes - ring_bytes - table_bytes;
+  int tm_fit = 0;
+  for (int t = tm < v.bm ? tm : v.bm; t >= 16 && tm_fit == 0; --t)
+    if (patch_for(t) <= room) tm_fit = t;
+  for (int t = tm + 1; t <= v.bm && t <= hw && tm_fit == 0; ++t)
+    if (patch_for(t) <= room) tm_fit = t;
+  if (tm_fit == 0) return false;
+  a->r_sz = b.r_sz;
+  a->p_tm = tm_fit;
+  a->p_tiles = (hw + tm_fit - 1) / tm_fit;
+  a->p_pw = (int)pw;
+  a->p_cpp = cpp;
+  a->p_iters = 0;
+  a->p_np_bytes = (int)patch_for(tm_fit);
+  a->p_seg = seg;
+  a->p_ppi = 0;
+  magic_for_divisor((uint32_t)cpp, (uint64_t)seg * 64, &a->p_cpp_m, &a->p_cpp_s);
+  a->p_pw_m = 0; a->p_pw_s = 0;
+  a->grid_m = b.batch * a->p_tiles;
+  a->grid_n = grid_n;
+  magic_for_divisor((uint32_t)grid_n, (uint64_t)a->grid_m * grid_n, &a->gn_m, &a->gn_s);
+  magic_for_divisor((uint32_t)a->p_tiles, (uint64_t)a->grid_m, &a->pt_m, &a->pt_s);
+  a->group_m = 1;
+  a->b_bytes = (unsigned)w_bytes;
+  a->a_bytes = 0;
+  return true;
+}
+
 // The operator chain in the fast form of the filter-resident kernel: [affine] [ReLU] [residual] [ReLU],
 // each part at most once and in this order, affine = bias / scale-shift / BatchNorm; every tile has all 64
 // channels, output rows and residual rows are 8-byte aligned and addressable with 32-bit byte offsets
@@ -1564,6 +1629,7 @@ void fast_epilogue_form(const EpilogueChain &chain, int dtype, ContractionArgs *
 
 bool plan_conv_resident(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
   if (v.pipeline == 7 || v.pipeline == 8) return plan_conv_wave16(g, v, w_ncontig, a);
+  if (v.pipeline == 9) return plan_conv_ksplit16(g, v, w_ncontig, a);
   return v.pipeline == 5 ? plan_conv_filter_resident(g, v, w_ncontig, a) : plan_conv_patch(g, v, w_ncontig, a);
 }
 
@@ -1595,12 +1661,12 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // 56x56x64->64 14.1 us / 16.7; N64 25.2 / 28.6; N32 64->128 24.5 / 28.8; N8 10.3 / 9.5 (not taken).
   bool resident_chosen = false;
   // First choice: the kernels on 16x16x32 MFMAs with the patch in LDS and the filter slab resident or in a
-  // ring (pipelines 7 and 8), where their plan fits, the launch fills most of the device and a workgroup's
+  // ring (pipelines 7, 8 and 9), where their plan fits, the launch fills most of the device and a workgroup's
   // tile is at least three quarters of the kernel's largest (smaller tiles leave its waves' blocks empty).
   if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key, plan.x.dtype, plan.w_ncontig) < 0) {
     for (int i = 0; i < contraction_variant_count() && !resident_chosen; ++i) {
       const ContractionVariant &cv = contraction_variant(i);
-      if (cv.pipeline != 7 && cv.pipeline != 8) continue;
+      if (cv.pipeline < 7 || cv.pipeline > 9) continue;
       ContractionArgs probe = a;
       if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n * 4 >= device_limits().cus * 3 &&
           probe.p_tm * 4 >= cv.bm * 3) {
