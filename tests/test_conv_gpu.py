@@ -239,6 +239,85 @@ def test_ksplit_variant(tracea_gpu, dtype, member, cin):
         capi.force_variant("conv2d", -1)
 
 
+THIN_SHAPES = [  # n, h, w, k, filter (r, s), stride, pad, dilation: 8 input channels
+    (32, 224, 224, 64, (7, 7), 4, 3, 1),          # the ResNet benchmark's first layer at batch 32
+    (2, 60, 44, 64, (7, 7), 4, 3, 1),             # small launch
+    (1, 37, 53, 40, (7, 7), 2, 3, 1),             # stride 2, 40 filters (general epilogue)
+    (3, 30, 30, 128, (7, 7), 1, 3, 1),            # stride 1, two filter slabs
+    (1, 40, 33, 64, (7, 7), 4, 0, 1),             # no padding
+    (2, 31, 29, 64, (7, 5), (3, 2), (2, 4), 1),   # 7x5 filter, mixed strides, asymmetric padding
+    (2, 45, 38, 64, (7, 8), (2, 4), (6, 1), (2, 1)),  # 8 taps per row, filter rows 2 apart
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_thin8_variant(tracea_gpu, dtype):
+    """The first-layer kernel (8 input channels, filter bank in registers, patch in LDS), forced, against
+    torch in double and, on symmetric geometry, the oracle."""
+    from tracea_amd import capi
+    member = "c128x64_c8_r7_w16_thin"
+    names = capi.variants("conv2d")
+    assert member in names, "no member %s in the build" % member
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rnd = round_f16 if dtype == "f16" else round_bf16
+    capi.force_variant("conv2d", names.index(member))
+    try:
+        for shape in THIN_SHAPES:
+            n, h, w, k, (fr, fs), stride, pad, dil = shape
+            kg = fr * fs * 8
+            rng = np.random.default_rng(h * 31 + w + k)
+            x = rnd(rng.standard_normal((n, h, w, 8)))
+            x[..., 3:] = 0.0 if n == 32 else x[..., 3:]     # the benchmark's image: 3 real channels
+            wk = rnd(rng.standard_normal((k, fr, fs, 8)) * np.sqrt(2.0 / kg))
+            bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+            ref = torch.nn.functional.conv2d(
+                torch.from_numpy(x).permute(0, 3, 1, 2).double(), torch.from_numpy(wk).permute(0, 3, 1, 2).double(),
+                bias=torch.from_numpy(bias).double(), stride=stride, padding=pad, dilation=dil)
+            ref = torch.relu(ref).permute(0, 2, 3, 1).numpy()
+            if isinstance(pad, int) and isinstance(stride, int) and fr == fs and n <= 3:
+                acc = oracle.conv2d_nhwc(x, np.ascontiguousarray(wk.transpose(1, 2, 3, 0)), stride, pad, dil)
+                want = oracle.epilogue_apply(acc, [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+                assert np.abs(want - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max())
+            y = tracea_gpu.conv2d(_dev(x, tdt), _dev(wk, tdt), bias=_dev(bias), stride=stride, padding=pad,
+                                  dilation=dil, epilogue="bias+relu")
+            assert capi.last_variant("conv2d") == member, "%s refused %s" % (member, shape)
+            assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(kg, dtype), "%s %s %s" % (member, dtype, shape))
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
+def test_thin8_variant_operator_chains(tracea_gpu):
+    """The first-layer kernel's register epilogue in all its forms and two chains outside it."""
+    from tracea_amd import capi
+    member = "c128x64_c8_r7_w16_thin"
+    n, h, w, k = 6, 50, 62, 64
+    rng = np.random.default_rng(78)
+    x = round_f16(rng.standard_normal((n, h, w, 8)))
+    w_rsck = round_f16(rng.standard_normal((7, 7, 8, k)) * np.sqrt(2.0 / 392))
+    acc = oracle.conv2d_nhwc(x, w_rsck, 2, 3, 1)
+    bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+    (gamma, beta, mean, var), (scale, shift) = _bn_params(rng, k)
+    res = round_f16(rng.standard_normal(acc.shape))
+    dx, dw = _dev(x, torch.float16), _dev(w_rsck, torch.float16).permute(3, 0, 1, 2).contiguous()
+    O, E = capi, oracle
+    aff = {"bias": ((O.OP_BIAS_ADD, _dev(bias)), (E.EPI_BIAS_ADD, bias)),
+           "ss": ((O.OP_SCALE_SHIFT, _dev(scale), _dev(shift)), (E.EPI_SCALE_SHIFT, scale, shift)),
+           "bn": ((O.OP_BATCHNORM, _dev(gamma), _dev(beta), _dev(mean), _dev(var), 1e-5), (E.EPI_BATCHNORM, gamma, beta, mean, var, 1e-5))}
+    relu = ((O.OP_RELU,), (E.EPI_RELU,))
+    resid = ((O.OP_RESIDUAL_ADD, _dev(res, torch.float16)), (E.EPI_RESIDUAL_ADD, res))
+    chains = [[], [aff["bn"], relu], [aff["bias"]], [aff["ss"], relu, resid, relu], [resid], [relu, resid],
+              [aff["bias"], resid, relu], [aff["bias"], ((O.OP_SILU,), (E.EPI_SILU,))], [resid, aff["ss"]]]
+    capi.force_variant("conv2d", member)
+    try:
+        for chain in chains:
+            want = oracle.epilogue_apply(acc, [c[1] for c in chain])
+            y = tracea_gpu.conv2d_ex(dx, dw, [c[0] for c in chain], stride=2, padding=3)
+            assert capi.last_variant("conv2d") == member
+            assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(392), "%s chain %s" % (member, [c[1][0] for c in chain]))
+    finally:
+        capi.force_variant("conv2d", -1)
+
+
 @pytest.mark.parametrize("member,cin", LDS_MEMBERS + KSPLIT_MEMBERS)
 def test_filter_resident_variant_operator_chains(tracea_gpu, member, cin):
     """Every form of their straight-line epilogue ([affine] [ReLU] [residual] [ReLU]) and chains outside it

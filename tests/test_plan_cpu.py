@@ -56,7 +56,8 @@ def test_unfused_block_runs_every_node_and_reuses_freed_slots():
     assert len(add["inputs"]) == 2 and 0 in add["inputs"]
 
 
-def test_resnet18_plan_reuses_the_arena():
+def test_resnet18_plan_reuses_the_arena(monkeypatch):
+    monkeypatch.setenv("TRACEA_PLAN_SIDE_BY_SIDE", "1")
     graph, info = G.resnet18_graph(batch=1)
     assert len(graph["operators"]) == 148
     fused = G.fuse(graph)
@@ -65,7 +66,15 @@ def test_resnet18_plan_reuses_the_arena():
     assert kinds.count("Elementwise") == 0 and kinds.count("GlobalAveragePool") == 1 and kinds.count("Linear") == 1
     desc = compile_plan(fused)
     steps = desc["steps"]
-    assert len(steps) == 22 and steps[-1]["kind"] == "Linear" and steps[-1]["op_id"] == info["output"]
+    # 20 convolutions and the classifier head: the Linear step took over the pooling node in front of it
+    # (one launch) and still writes the pooling node's output
+    assert len(steps) == 21 and steps[-1]["kind"] == "Linear" and steps[-1]["op_id"] == info["output"]
+    pool_id = [list(n.values())[0]["op_id"] for n in fused["operators"] if list(n)[0] == "GlobalAveragePool"][0]
+    assert steps[-1]["pooled_from"] == pool_id and steps[-1]["inputs"] == [steps[-2]["op_id"]]
+    assert str(pool_id) in desc["output_map"] and desc["output_map"][str(pool_id)][1] == 512 * 2
+    lo, size = desc["output_map"][str(pool_id)]
+    assert lo + size <= steps[-1]["offset"] or lo >= steps[-1]["offset"] + steps[-1]["bytes"]
+    assert lo + size <= steps[-2]["offset"] or lo >= steps[-2]["offset"] + steps[-2]["bytes"]
     total = sum(s["bytes"] for s in steps)
     assert desc["arena_size"] * 3 <= total                        # 1.2 MB against 3.8 MB
     # every step's inputs precede it, and no live tensor overlaps a step's output
@@ -86,6 +95,40 @@ def test_resnet18_plan_reuses_the_arena():
     # a downsampling block: the 1x1 shortcut convolution runs before the convolution that adds it
     names = [s["name"] for s in steps]
     assert names.index("layer_128_block_0_shortcut_conv") < names.index("layer_128_block_0_conv2")
+    # ... and beside the block's first convolution, which it does not depend on: the three pairs of the
+    # network, each with both outputs and everything either step reads in disjoint memory
+    pairs = [(steps[i]["name"], steps[i + 1]["name"]) for i in range(len(steps) - 1) if steps[i]["side_by_side"] == "first"]
+    assert pairs == [("layer_%d_block_0_conv1" % c, "layer_%d_block_0_shortcut_conv" % c) for c in (128, 256, 512)]
+    assert [s["side_by_side"] for s in steps].count("second") == 3
+    for i, s in enumerate(steps):
+        if s["side_by_side"] != "first":
+            continue
+        nxt = steps[i + 1]
+        assert nxt["side_by_side"] == "second" and s["op_id"] not in nxt["inputs"]
+        spans = [(s["offset"], s["offset"] + s["bytes"]), (nxt["offset"], nxt["offset"] + nxt["bytes"])]
+        for t in set(list(s["inputs"]) + list(nxt["inputs"])):
+            if t in place:
+                spans.append((place[t][1], place[t][2]))
+                assert place[t][3] >= i + 1               # kept until the second step is done
+        spans = sorted(set(spans))
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:])), spans
+
+
+def test_split_head_switch(monkeypatch):
+    """TRACEA_PLAN_SPLIT_HEAD=1 (read when a plan is compiled) keeps pooling and the linear layer two steps."""
+    graph, _ = G.resnet18_graph(batch=1)
+    monkeypatch.setenv("TRACEA_PLAN_SPLIT_HEAD", "1")
+    steps = compile_plan(G.fuse(graph))["steps"]
+    assert len(steps) == 22 and [s["kind"] for s in steps[-2:]] == ["GlobalAveragePool", "Linear"]
+    assert all(s["pooled_from"] == 0 for s in steps)
+
+
+def test_plan_is_serial_by_default(monkeypatch):
+    """Without TRACEA_PLAN_SIDE_BY_SIDE=1 (read when a plan is compiled) every step stays on the caller's stream."""
+    graph, _ = G.resnet18_graph(batch=1)
+    monkeypatch.delenv("TRACEA_PLAN_SIDE_BY_SIDE", raising=False)
+    steps = compile_plan(G.fuse(graph))["steps"]
+    assert all(s["side_by_side"] == "no" for s in steps)
 
 
 def test_graph_outputs_stay_allocated_to_the_end():

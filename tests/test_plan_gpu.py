@@ -191,6 +191,62 @@ def test_hip_graph_replays_equal_the_eager_run(tracea_gpu):
     assert float(scratch[0]) == 4.0
 
 
+@pytest.mark.parametrize("n,c,h,classes", [(3, 44, 5, 24), (32, 512, 7, 1000), (1, 512, 7, 1000)])
+@pytest.mark.parametrize("slot", ["weight", "weight_t"])
+def test_pool_and_linear_in_one_launch(tracea_gpu, monkeypatch, n, c, h, classes, slot):
+    """A pooling node read by one Linear node runs inside the Linear's launch: means as the pooling node
+    alone computes them (same bits, still written to its place), logits against float64 and close to the
+    two-launch plan's (another order of the fp32 sums)."""
+    from tracea_amd import graph as G, plan as P
+    rng = np.random.default_rng(c + classes)
+    x = round_f16(rng.standard_normal((n, h, h, c)))
+    wt = round_f16(rng.standard_normal((c, classes)) * 0.2)
+    g = {"operators": [G.input_node(1, "x"), G.global_avg_pool_node(2, "gap", n, c, h, h), G.linear_node(3, "fc", n, 1, classes, c)],
+         "dependencies": [[1, 2], [2, 3]]}
+    dw = torch.from_numpy(wt if slot == "weight" else np.ascontiguousarray(wt.T)).cuda().half()
+
+    def run():
+        plan = P.Plan(g).bind(1, torch.from_numpy(x).cuda().half()).bind(3, dw, slot)
+        plan.run()
+        torch.cuda.synchronize()
+        return plan, plan.output(2, (n, c)).clone(), plan.output(3, (n, classes)).float().cpu().numpy()
+
+    one, gap_one, fc_one = run()
+    assert [s["kind"] for s in one.describe()["steps"]] == ["Linear"] and one.describe()["steps"][0]["pooled_from"] == 2
+    monkeypatch.setenv("TRACEA_PLAN_SPLIT_HEAD", "1")
+    two, gap_two, fc_two = run()
+    assert [s["kind"] for s in two.describe()["steps"]] == ["GlobalAveragePool", "Linear"]
+    assert torch.equal(gap_one, gap_two)
+    gap = gap_two.float().cpu().numpy()
+    np.testing.assert_allclose(gap, x.reshape(n, h * h, c).mean(axis=1), atol=1e-3)
+    want = gap.astype(np.float64) @ wt.astype(np.float64)
+    tol = 2e-3 * max(1.0, np.abs(want).max())
+    np.testing.assert_allclose(fc_one, want, atol=tol)
+    np.testing.assert_allclose(fc_one, fc_two, atol=tol)
+
+
+def test_side_by_side_steps_give_the_serial_result(tracea_gpu, monkeypatch):
+    """TRACEA_PLAN_SIDE_BY_SIDE=1: the shortcut convolutions run on the plan's side stream beside the
+    blocks' first convolutions; eager and as a replayed HIP graph the logits equal the serial plan's."""
+    plan, info, _ = _resnet18(batch=2, seed=13)
+    plan.run()
+    torch.cuda.synchronize()
+    serial = plan.output(info["output"], (2, 1000)).clone()
+    monkeypatch.setenv("TRACEA_PLAN_SIDE_BY_SIDE", "1")
+    forked, info2, _ = _resnet18(batch=2, seed=13)
+    assert [s["side_by_side"] for s in forked.describe()["steps"]].count("second") == 3
+    forked.run()
+    torch.cuda.synchronize()
+    assert torch.equal(forked.output(info2["output"], (2, 1000)), serial)
+    forked.capture()
+    for i in range(3):
+        forked.output(info2["output"]).zero_()
+        torch.cuda.synchronize()
+        forked.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(forked.output(info2["output"], (2, 1000)), serial), "replay %d" % i
+
+
 def test_unbound_inputs_are_reported_before_any_launch(tracea_gpu):
     from tracea_amd import graph as G, plan as P
     plan = P.Plan(G.fuse(basic_block(1, 16, 8)))

@@ -266,7 +266,7 @@ def test_sixth_to_tenth_observation_triggers_a_refit():
 def test_proposed_configs_name_compiled_variants():
     from tracea_amd import capi
     names = capi.variants("gemm")
-    conv_only = {i for i, nm in enumerate(names) if nm.endswith(("_patch", "_resident"))}
+    conv_only = {i for i, nm in enumerate(names) if nm.endswith(("_patch", "_resident", "_ksplit", "_thin"))}
     assert conv_only, "the build has patch-resident convolution variants"
     for propose, expect in ((T.propose_gemm_configs, set(range(len(names))) - conv_only),
                             (T.propose_conv_configs, set(range(len(names))))):

@@ -218,6 +218,17 @@ int launch_chain_apply(const ChainApplyArgs &args, hipStream_t stream);
 // out[b, c] = mean over hw of x[b, hw, c] (NHWC), fp32 sums.
 int launch_global_avg_pool(const void *x, void *out, int dtype, int out_dtype, int batch, int hw, int channels,
                            hipStream_t stream);
+// Pooling and the linear layer behind it in one launch: out[b, j] = chain(sum_k mean_hw(x[b, hw, k]) * w[k, j]),
+// the means rounded through `dtype` (and stored to `pooled` [batch, channels] when it is not null).
+struct PoolLinearArgs {
+  const void *x, *w;
+  void *out, *pooled;
+  int dtype, out_dtype;  // x, w and pooled; out
+  int batch, hw, channels, n_out;
+  long long w_ld;        // elements between rows of w (its other stride is 1)
+  EpilogueChain epi;
+};
+int launch_pool_linear(const PoolLinearArgs &args, bool k_contiguous, hipStream_t stream);
 // Row-wise softmax over the last axis, fp32 arithmetic.
 int launch_softmax_rows(const void *x, void *out, int dtype, int out_dtype, long long rows, int cols,
                         hipStream_t stream);

@@ -6,6 +6,7 @@
 #include "conv_resident_kernel.hpp"
 #include "conv_wave16_kernel.hpp"
 #include "conv_ksplit16_kernel.hpp"
+#include "conv_thin8_kernel.hpp"
 
 #define TRACEA_CAT2(a, b) a##b
 #define TRACEA_CAT(a, b) TRACEA_CAT2(a, b)
@@ -32,6 +33,9 @@ const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
 #elif V_DIRECT == 9
       (size_t)V_STAGES * CK_STAGE_BYTES + CK_TABLE_BYTES,  // the patch comes on top
       &launch_conv_ksplit16<V_BK, V_BM / 16, V_STAGES>, 16};
+#elif V_DIRECT == 10
+      (size_t)CT_TABLE_BYTES,  // the patch, sized by the problem, comes on top
+      &launch_conv_thin8<V_STAGES>, 16};
 #elif V_DIRECT == 6
       (size_t)V_STAGES * (V_BM + V_BN) * V_BK * 2,
       &launch_contraction<V_BM, V_BN, V_BK, V_WM, V_WN, V_STAGES, 2, 16>, 16};  // pipeline 2 on 16x16x32 MFMAs

@@ -62,39 +62,45 @@ struct Epilogue16 {
     }
     return v;
   }
-  // One pixel block x 64 filters.  acc[i]: the accumulators of filter block fb[i] (fb[2j] and fb[2j+1] share a
-  // store: after the swap the lanes of 16-lane group q hold channels (q>>1)*8 .. +7 of block fb[2j + (q&1)]);
+  // One pixel block x two filter blocks fa, fb (accumulators acc_a, acc_b): after the swap the lanes of
+  // 16-lane group q hold channels (q>>1)*8 .. +7 of block (q&1 ? fb : fa), one 16-byte store per lane.
   // ta/tb: the affine operands of the lane's four channels per block; prow: the pixel's row in the tile's
   // output (and residual) window, < 0 for a pixel outside the tile; row_c/row_r: row pitches in bytes.
+  static __device__ __forceinline__ void pair_block(f32x4 acc_a, f32x4 acc_b, int fa, int fb, f32x4 ta_a, f32x4 tb_a, f32x4 ta_b,
+                                                    f32x4 tb_b, int prow, int q, __amdgpu_buffer_rsrc_t rsrc_c,
+                                                    __amdgpu_buffer_rsrc_t rsrc_r, int row_c, int row_r) {
+    const int ch = ((q & 1) ? fb : fa) * 16 + (q >> 1) * 8;
+    float ra[4] = {0, 0, 0, 0}, rb[4] = {0, 0, 0, 0};
+    if constexpr (RES) {
+      const u32x4 r8 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                     rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
+      unsigned r0 = r8[0], r1 = r8[1], r2 = r8[2], r3 = r8[3];
+      asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
+                   : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));
+      unpack2(r0, ra[0], ra[1]);
+      unpack2(r1, ra[2], ra[3]);
+      unpack2(r2, rb[0], rb[1]);
+      unpack2(r3, rb[2], rb[3]);
+    }
+    const f32x4 va = finish(acc_a, ta_a, tb_a, ra);
+    const f32x4 vb = finish(acc_b, ta_b, tb_b, rb);
+    unsigned a_lo = pack2(va[0], va[1]), a_hi = pack2(va[2], va[3]);
+    unsigned b_lo = pack2(vb[0], vb[1]), b_hi = pack2(vb[2], vb[3]);
+    // (as instructions: the compiler's builtin for the swap returns its first result twice; the s_nop is the
+    // wait the hardware asks for between a vector-ALU write of an operand and the swap)
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
+                 : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi));
+    const u32x4 row8 = {a_lo, a_hi, b_lo, b_hi};
+    __builtin_amdgcn_raw_buffer_store_b128(row8, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
+  }
+  // One pixel block x 64 filters: acc[i] the accumulators of filter block fb[i]; fb[2j] and fb[2j+1] share a store.
   static __device__ __forceinline__ void pixel_block(const f32x4 (&acc)[4], const int (&fb)[4], const f32x4 (&ta)[4],
                                                      const f32x4 (&tb)[4], int prow, int q, __amdgpu_buffer_rsrc_t rsrc_c,
                                                      __amdgpu_buffer_rsrc_t rsrc_r, int row_c, int row_r) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int ch = fb[2 * j + (q & 1)] * 16 + (q >> 1) * 8;
-      float ra[4] = {0, 0, 0, 0}, rb[4] = {0, 0, 0, 0};
-      if constexpr (RES) {
-        const u32x4 r8 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                       rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
-        unsigned r0 = r8[0], r1 = r8[1], r2 = r8[2], r3 = r8[3];
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
-                     : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));
-        unpack2(r0, ra[0], ra[1]);
-        unpack2(r1, ra[2], ra[3]);
-        unpack2(r2, rb[0], rb[1]);
-        unpack2(r3, rb[2], rb[3]);
-      }
-      const f32x4 va = finish(acc[2 * j], ta[2 * j], tb[2 * j], ra);
-      const f32x4 vb = finish(acc[2 * j + 1], ta[2 * j + 1], tb[2 * j + 1], rb);
-      unsigned a_lo = pack2(va[0], va[1]), a_hi = pack2(va[2], va[3]);
-      unsigned b_lo = pack2(vb[0], vb[1]), b_hi = pack2(vb[2], vb[3]);
-      // (as instructions: the compiler's builtin for the swap returns its first result twice; the s_nop is the
-      // wait the hardware asks for between a vector-ALU write of an operand and the swap)
-      asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
-                   : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi));
-      const u32x4 row8 = {a_lo, a_hi, b_lo, b_hi};
-      __builtin_amdgcn_raw_buffer_store_b128(row8, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
-    }
+    for (int j = 0; j < 2; ++j)
+      pair_block(acc[2 * j], acc[2 * j + 1], fb[2 * j], fb[2 * j + 1], ta[2 * j], tb[2 * j], ta[2 * j + 1], tb[2 * j + 1], prow, q, rsrc_c,
+                 rsrc_r, row_c, row_r);
   }
   // One pixel block x one filter block (channels ch .. ch+3 of the lane): 8 bytes per lane.
   static __device__ __forceinline__ void single_block(f32x4 acc, f32x4 ta, f32x4 tb, int ch, int prow,

@@ -264,6 +264,11 @@ TraceaStatus hip_status(const char *what, int e) {
 
 }  // namespace
 
+TraceaStatus dispatch_lower_chain(const char *what, const TraceaEpilogueOp *ops, uint32_t n_ops, long long channels,
+                                  EpilogueChain *chain) {
+  return lower_chain(what, ops, n_ops, channels, channels, chain);
+}
+
 void set_split_k_enabled(bool on) { g_split_k_enabled.store(on); }
 void set_split_k_one_launch(bool on) { g_split_k_one_launch.store(on); }
 int last_split_k_launches() { return t_last_split_launches; }
@@ -1590,6 +1595,77 @@ bool plan_conv_ksplit16(const ConvGeometry &g, const ContractionVariant &v, bool
   return true;
 }
 
+// Plan of the 8-channel first-layer kernel (pipeline 10): tiles of whole output rows (up to 128 pixels; flat
+// runs of 128 pixels for wider rows) whose patch fits LDS twice beside the staging area; rows of RP 16-byte
+// pixels, RP a multiple of 8 that covers the padded row and the 8 taps read for the last output pixel; one
+// workgroup per CU and filter slab at most, walking the tiles.
+bool plan_conv_thin8(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
+  const TraceaConvParamsBlock &b = g.block;
+  if (v.pipeline != 10 || w_ncontig || b.c_in != 8 || b.r_sz != v.stages || b.s_sz > 8 || g.dil_w != 1 ||
+      g.k_gemm != b.r_sz * b.s_sz * 8)
+    return false;
+  const long long img_bytes = (long long)b.h_in * b.w_in * 8 * 2;
+  const long long w_bytes = (long long)g.n_gemm * g.k_gemm * 2;
+  if (img_bytes >= (1ll << 31) || w_bytes >= (1ll << 31)) return false;
+  long long pw = (long long)b.w_in + 2ll * g.pad_w;
+  const long long reach = (long long)(b.w_out - 1) * g.stride_w + 8;
+  if (reach > pw) pw = reach;
+  const long long rp = (pw + 7) / 8 * 8;
+  const long long ph = (long long)b.h_in + 2ll * g.pad_h;
+  if (rp * ph >= (1ll << 26) || (long long)b.h_in * b.w_in >= (1ll << 24)) return false;
+  const long long table_bytes = TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
+  const long long frag_bytes = (long long)b.r_sz * 8 * 1024;
+  const int hw = b.h_out * b.w_out;
+  const int grid_n = (g.n_gemm + v.bn - 1) / v.bn;
+  auto patch_for = [&](int t) -> long long {
+    long long out_rows = 1;
+    for (int p0 = 0; p0 < hw; p0 += t) {
+      const int last = (p0 + t < hw ? p0 + t : hw) - 1;
+      const long long span = last / b.w_out - p0 / b.w_out + 1;
+      if (span > out_rows) out_rows = span;
+    }
+    const long long rows = (out_rows - 1) * g.stride_h + (long long)(b.r_sz - 1) * g.dil_h + 1;
+    return (rows * rp * 16 + 1023) / 1024 * 1024;
+  };
+  auto lds_for = [&](int t) -> long long {
+    const long long pb = patch_for(t);
+    const long long staging = (long long)t * 68 * 4, spill = frag_bytes - pb;
+    return 2 * pb + (staging > spill ? staging : spill) + table_bytes;
+  };
+  // candidates: whole rows, most first; then flat tiles
+  int tm_fit = 0;
+  if (b.w_out <= v.bm) {
+    for (int rows = v.bm / b.w_out; rows >= 1 && tm_fit == 0; --rows) {
+      const int t = rows * b.w_out < hw ? rows * b.w_out : hw;
+      if (lds_for(t) <= (long long)device_limits().lds_bytes) tm_fit = t;
+    }
+  }
+  for (int t = v.bm < hw ? v.bm : hw; t >= 16 && tm_fit == 0; t -= 16)
+    if (lds_for(t) <= (long long)device_limits().lds_bytes) tm_fit = t;
+  if (tm_fit == 0) return false;
+  a->r_sz = b.r_sz;
+  a->p_tm = tm_fit;
+  a->p_tiles = (hw + tm_fit - 1) / tm_fit;
+  a->p_pw = (int)rp;
+  a->p_cpp = 1;
+  a->p_np_bytes = (int)patch_for(tm_fit);
+  a->p_seg = (int)((rp + 63) / 64);
+  a->p_ppi = 0;
+  a->p_cpp_m = 0; a->p_cpp_s = 0; a->p_pw_m = 0; a->p_pw_s = 0;
+  a->grid_m = b.batch * a->p_tiles;
+  a->grid_n = grid_n;
+  long long slots = device_limits().cus / grid_n;
+  if (slots < 1) slots = 1;
+  if (slots > a->grid_m) slots = a->grid_m;
+  a->p_iters = (int)slots;  // workgroups per filter slab
+  magic_for_divisor((uint32_t)grid_n, (uint64_t)slots * grid_n, &a->gn_m, &a->gn_s);
+  magic_for_divisor((uint32_t)a->p_tiles, (uint64_t)a->grid_m, &a->pt_m, &a->pt_s);
+  a->group_m = 1;
+  a->b_bytes = (unsigned)w_bytes;
+  a->a_bytes = 0;
+  return true;
+}
+
 // The operator chain in the fast form of the filter-resident kernel: [affine] [ReLU] [residual] [ReLU],
 // each part at most once and in this order, affine = bias / scale-shift / BatchNorm; every tile has all 64
 // channels, output rows and residual rows are 8-byte aligned and addressable with 32-bit byte offsets
@@ -1630,6 +1706,7 @@ void fast_epilogue_form(const EpilogueChain &chain, int dtype, ContractionArgs *
 bool plan_conv_resident(const ConvGeometry &g, const ContractionVariant &v, bool w_ncontig, ContractionArgs *a) {
   if (v.pipeline == 7 || v.pipeline == 8) return plan_conv_wave16(g, v, w_ncontig, a);
   if (v.pipeline == 9) return plan_conv_ksplit16(g, v, w_ncontig, a);
+  if (v.pipeline == 10) return plan_conv_thin8(g, v, w_ncontig, a);
   return v.pipeline == 5 ? plan_conv_filter_resident(g, v, w_ncontig, a) : plan_conv_patch(g, v, w_ncontig, a);
 }
 
@@ -1661,12 +1738,12 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   // 56x56x64->64 14.1 us / 16.7; N64 25.2 / 28.6; N32 64->128 24.5 / 28.8; N8 10.3 / 9.5 (not taken).
   bool resident_chosen = false;
   // First choice: the kernels on 16x16x32 MFMAs with the patch in LDS and the filter slab resident or in a
-  // ring (pipelines 7, 8 and 9), where their plan fits, the launch fills most of the device and a workgroup's
+  // ring (pipelines 7 to 10), where their plan fits, the launch fills most of the device and a workgroup's
   // tile is at least three quarters of the kernel's largest (smaller tiles leave its waves' blocks empty).
   if (forced_variant("conv2d") < 0 && tuning_cache_lookup_variant(key, plan.x.dtype, plan.w_ncontig) < 0) {
     for (int i = 0; i < contraction_variant_count() && !resident_chosen; ++i) {
       const ContractionVariant &cv = contraction_variant(i);
-      if (cv.pipeline < 7 || cv.pipeline > 9) continue;
+      if (cv.pipeline < 7 || cv.pipeline > 10) continue;
       ContractionArgs probe = a;
       if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n * 4 >= device_limits().cus * 3 &&
           probe.p_tm * 4 >= cv.bm * 3) {

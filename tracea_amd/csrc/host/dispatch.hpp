@@ -60,6 +60,10 @@ TraceaStatus dispatch_gemm_kind(const TraceaTensorView &a, const TraceaTensorVie
 TraceaStatus dispatch_gemm_ops(const TraceaTensorView &a, const TraceaTensorView &b,
                                TraceaTensorView *c, const TraceaGemmParams &params,
                                const TraceaEpilogueOp *ops, uint32_t n_ops);
+// A caller's operator list, checked and in device form, for an output of rows of `channels` elements
+// (a residual without a row stride of its own has that one).
+TraceaStatus dispatch_lower_chain(const char *what, const TraceaEpilogueOp *ops, uint32_t n_ops, long long channels,
+                                  EpilogueChain *chain);
 // GEMM over a tile list.  `tables` are the device copies of a TileLayout's tables on the
 // device of c: level-1 map in launch order, records, and (slices > 1 only) the workspace
 // row block of every workgroup.  Exactly one of (ops, n_ops) and the kind in params is used:

@@ -1,6 +1,7 @@
 #include "execution_plan.hpp"
 
 #include <algorithm>
+#include <cstdlib>
 #include <set>
 
 namespace tracea_amd {
@@ -305,9 +306,56 @@ bool ExecutionPlan::compile(const Json &graph, int dtype, std::string *err) {
       step_of[id] = (int)steps_.size();
       steps_.push_back(nodes[id]);
     }
+  // ---- a classifier head in one launch: a GlobalAveragePool node read by one Linear node only (batch 1 of the
+  // Linear's geometry, the pooled channels as its K) is taken over by that Linear step, which computes the
+  // means itself and still writes them to the pooling node's place.  TRACEA_PLAN_SPLIT_HEAD=1 at compile
+  // keeps the two launches. ----
+  {
+    const char *keep = getenv("TRACEA_PLAN_SPLIT_HEAD");
+    for (size_t i = 0; i + 1 < steps_.size() && !(keep && keep[0] == '1'); ++i) {
+      PlanStep &pool = steps_[i], &lin = steps_[i + 1];
+      if (pool.kind != "GlobalAveragePool" || lin.kind != "Linear" || lin.inputs.size() != 1 || lin.inputs[0] != pool.id) continue;
+      if (consumers[pool.id].size() != 1 || lin.g[3] * lin.g[0] != pool.g[0] || lin.g[2] != pool.g[1] || pool.g[1] > 8192) continue;
+      bool side = false;  // (the means must not be an operand of the Linear's own chain)
+      for (const PlanEpilogue &pe : lin.epilogue)
+        for (int k = 0; k < pe.n_ids; ++k) side = side || pe.ids[k] == pool.id;
+      if (side) continue;
+      lin.pool_id = pool.id;
+      lin.pool_hw = pool.g[2] * pool.g[3];
+      lin.inputs[0] = pool.inputs[0];
+      steps_.erase(steps_.begin() + (long)i);
+    }
+  }
   const int n_steps = (int)steps_.size();
+  // ---- neighbours that may run side by side: two contractions of which the second reads nothing the first
+  // writes (a block's first convolution and its shortcut convolution).  Off unless TRACEA_PLAN_SIDE_BY_SIDE=1
+  // is set when the plan is compiled: measured on ResNet-18 replayed as a HIP graph on one MI355X, the three
+  // forks and joins cost more than the overlap gains (batch 1: 235 us against 215 serial; batch 32: 300
+  // against 295) ----
+  {
+    auto heavy = [](const PlanStep &s) { return s.kind == "Conv2d" || s.kind == "Gemm" || s.kind == "Linear"; };
+    auto reads = [](const PlanStep &s, Id t) {
+      for (Id i : s.inputs)
+        if (i == t) return true;
+      for (const PlanEpilogue &pe : s.epilogue)
+        for (int k = 0; k < pe.n_ids; ++k)
+          if (pe.ids[k] == t) return true;
+      return false;
+    };
+    const char *pairs = getenv("TRACEA_PLAN_SIDE_BY_SIDE");
+    for (int i = 0; i + 1 < n_steps && pairs && pairs[0] == '1'; ++i)
+      if (steps_[i].fork == 0 && heavy(steps_[i]) && heavy(steps_[i + 1]) && !reads(steps_[i + 1], steps_[i].id)) {
+        steps_[i].fork = 1;
+        steps_[i + 1].fork = 2;
+        ++i;
+      }
+  }
   for (int i = 0; i < n_steps; ++i) {
     tensors_[steps_[i].id].born = i;
+    if (steps_[i].pool_id != 0) {
+      tensors_[steps_[i].pool_id].born = i;
+      tensors_[steps_[i].pool_id].last_use = i;
+    }
     auto touch = [&](Id t) {
       PlanTensor &pt = tensors_[t];
       if (!pt.external && pt.last_use < i) pt.last_use = i;
@@ -316,18 +364,72 @@ bool ExecutionPlan::compile(const Json &graph, int dtype, std::string *err) {
     for (const PlanEpilogue &pe : steps_[i].epilogue)
       for (int k = 0; k < pe.n_ids; ++k) touch(pe.ids[k]);
   }
+  // what the first step of a side-by-side pair reads last stays until the second is done too (the second's
+  // output must not land on memory the first still reads)
+  for (int i = 0; i + 1 < n_steps; ++i)
+    if (steps_[i].fork == 1)
+      for (auto &t : tensors_)
+        if (!t.second.external && t.second.last_use == i) t.second.last_use = i + 1;
   Arena arena;
   for (int i = 0; i < n_steps; ++i) {
     PlanTensor &out = tensors_[steps_[i].id];
     if (out.last_use < 0) out.last_use = n_steps;  // nobody reads it: a result of the graph
     out.bytes = align256((size_t)out.elems * elem_bytes(out.dtype));
     out.offset = arena.take(out.bytes);
+    if (steps_[i].pool_id != 0) {
+      PlanTensor &pt = tensors_[steps_[i].pool_id];
+      pt.bytes = align256((size_t)pt.elems * elem_bytes(pt.dtype));
+      pt.offset = arena.take(pt.bytes);
+    }
     for (auto &t : tensors_) {
       PlanTensor &pt = t.second;
       if (!pt.external && pt.born >= 0 && pt.born <= i && pt.last_use == i) arena.give(pt.offset, pt.bytes);
     }
   }
   arena_size_ = arena.top;
+  int dev = -1;
+  if (hipGetDevice(&dev) == hipSuccess) (void)ensure_side(dev, nullptr);  // best effort: run() tries again
+  else (void)hipGetLastError();
+  return true;
+}
+
+ExecutionPlan::~ExecutionPlan() {
+  if (ev_fork_) (void)hipEventDestroy((hipEvent_t)ev_fork_);
+  if (ev_join_) (void)hipEventDestroy((hipEvent_t)ev_join_);
+  if (side_stream_) (void)hipStreamDestroy((hipStream_t)side_stream_);
+}
+
+// The side stream and its two events on `device` (current when this is called).  Nothing is created while
+// `stream` is being captured: creation calls are not allowed then, and the run stays on one stream.
+bool ExecutionPlan::ensure_side(int device, void *stream) const {
+  if (side_stream_ != nullptr && side_device_ == device) return true;
+  bool any = false;
+  for (const PlanStep &st : steps_) any = any || st.fork != 0;
+  if (!any) return false;
+  if (stream != nullptr) {
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return false;
+    }
+  }
+  if (ev_fork_) (void)hipEventDestroy((hipEvent_t)ev_fork_);
+  if (ev_join_) (void)hipEventDestroy((hipEvent_t)ev_join_);
+  if (side_stream_) (void)hipStreamDestroy((hipStream_t)side_stream_);
+  ev_fork_ = ev_join_ = side_stream_ = nullptr;
+  side_device_ = -1;
+  hipStream_t s = nullptr;
+  hipEvent_t a = nullptr, b = nullptr;
+  if (hipStreamCreateWithFlags(&s, hipStreamNonBlocking) != hipSuccess || hipEventCreateWithFlags(&a, hipEventDisableTiming) != hipSuccess ||
+      hipEventCreateWithFlags(&b, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+    if (s) (void)hipStreamDestroy(s);
+    return false;
+  }
+  side_stream_ = s; ev_fork_ = a; ev_join_ = b;
+  side_device_ = device;
   return true;
 }
 
@@ -358,6 +460,8 @@ Json ExecutionPlan::describe() const {
     s.set("bytes", Json::make_num((double)t.bytes));
     s.set("elements", Json::make_num((double)t.elems));
     s.set("last_use", Json::make_num(t.last_use));
+    s.set("pooled_from", Json::make_num((double)st.pool_id));
+    s.set("side_by_side", Json::make_str(st.fork == 1 ? "first" : st.fork == 2 ? "second" : "no"));
     steps.arr.push_back(s);
   }
   root.set("steps", steps);
@@ -471,7 +575,17 @@ TraceaStatus ExecutionPlan::run(void *arena, int device, void *stream) const {
     v.ptr = ptr; v.rank = (uint32_t)rank; v.shape = shape; v.stride = stride; v.dtype = d; v.device_id = device;
     return v;
   };
+  const bool forking = ensure_side(device, stream);
+  void *const main_stream = stream;
   for (const PlanStep &st : steps_) {
+    // a pair of independent neighbours: the side stream picks up behind everything launched so far, runs the
+    // second step, and the main stream waits for it before going on
+    if (forking && st.fork == 1) {
+      hipError_t e = hipEventRecord((hipEvent_t)ev_fork_, (hipStream_t)main_stream);
+      if (e == hipSuccess) e = hipStreamWaitEvent((hipStream_t)side_stream_, (hipEvent_t)ev_fork_, 0);
+      if (e != hipSuccess) return fail(TRACEA_CUDA_ERROR, "tracea_plan_run: fork in front of '%s': %s", st.name.c_str(), hipGetErrorString(e));
+    }
+    stream = forking && st.fork == 2 ? side_stream_ : main_stream;
     void *out = address(st.id, arena);
     const PlanTensor &ot = tensors_.at(st.id);
     TraceaEpilogueOp ops[TRACEA_MAX_EPILOGUE_OPS];
@@ -508,6 +622,22 @@ TraceaStatus ExecutionPlan::run(void *arena, int device, void *stream) const {
       p.stream = stream;
       status = dispatch_conv2d_ops(view(address(st.inputs[0], arena), 4, xs, nullptr, dt),
                                    view((void *)st.weight, 4, ws, st.weight_layout ? wst : nullptr, dt), &o, p, ops, n_ops);
+    } else if (st.kind == "Linear" && st.pool_id != 0) {
+      PoolLinearArgs a{};
+      a.x = address(st.inputs[0], arena);
+      a.w = st.weight;
+      a.out = out;
+      a.pooled = address(st.pool_id, arena);
+      a.dtype = a.out_dtype = dt;
+      a.batch = (int)(st.g[3] * st.g[0]); a.hw = (int)st.pool_hw; a.channels = (int)st.g[2]; a.n_out = (int)st.g[1];
+      a.w_ld = st.weight_layout ? st.g[2] : st.g[1];  // [N,K] storage: k contiguous; else [K,N]
+      EpilogueChain chain{};
+      status = dispatch_lower_chain("tracea_plan_run", ops, n_ops, st.g[1], &chain);
+      if (status == TRACEA_SUCCESS) {
+        a.epi = chain;
+        const int e = launch_pool_linear(a, st.weight_layout != 0, (hipStream_t)stream);
+        if (e != 0) status = fail(TRACEA_CUDA_ERROR, "tracea_plan_run: '%s': %s", st.name.c_str(), hipGetErrorString((hipError_t)e));
+      }
     } else if (st.kind == "Gemm" || st.kind == "Linear") {
       const long long m = st.g[3] * st.g[0], n = st.g[1], k = st.g[2];
       const uint64_t as[2] = {(uint64_t)m, (uint64_t)k}, bs[2] = {(uint64_t)k, (uint64_t)n}, cs[2] = {(uint64_t)m, (uint64_t)n};
@@ -560,6 +690,13 @@ TraceaStatus ExecutionPlan::run(void *arena, int device, void *stream) const {
         e = launch_chain_apply(a, (hipStream_t)stream);
       }
       if (e != 0) status = fail(TRACEA_CUDA_ERROR, "tracea_plan_run: '%s': %s", st.name.c_str(), hipGetErrorString((hipError_t)e));
+    }
+    if (forking && st.fork == 2) {
+      // (joined also after a failed launch: a capture must not end with the side stream still forked)
+      hipError_t e = hipEventRecord((hipEvent_t)ev_join_, (hipStream_t)side_stream_);
+      if (e == hipSuccess) e = hipStreamWaitEvent((hipStream_t)main_stream, (hipEvent_t)ev_join_, 0);
+      if (e != hipSuccess && status == TRACEA_SUCCESS)
+        status = fail(TRACEA_CUDA_ERROR, "tracea_plan_run: join behind '%s': %s", st.name.c_str(), hipGetErrorString(e));
     }
     if (status != TRACEA_SUCCESS) return status;
   }

@@ -8,8 +8,10 @@
 // returned to a free list after its last consumer has run, so a deep network
 // needs the arena of its widest cut, not of its sum.  A plan holds no device
 // memory: the caller passes the arena to run(), and run() only launches kernels on
-// the given stream, so the whole plan can be captured into a HIP graph and
-// replayed.
+// the given stream (and, where TRACEA_PLAN_SIDE_BY_SIDE=1 was set at compile(), for the
+// second of two neighbouring steps that do not depend on each other, on a side stream of
+// the plan's own that forks from it and joins it again through events), so the whole plan
+// can be captured into a HIP graph and replayed.
 #pragma once
 #include <map>
 #include <string>
@@ -49,10 +51,22 @@ struct PlanStep {
   float epsilon = 0.0f;
   const void *weight = nullptr;     // bind(op_id, "weight", ...)
   int weight_layout = 0;            // 0: [K,R,S,C] / [K,N];  1: [R,S,C,K] / [N,K]
+  // A Linear step that took over the GlobalAveragePool node in front of it (one launch for both): the pooling
+  // node's id (its output is still written), its pixels per image; 0: none.  inputs[0] is then the pooling
+  // node's input.
+  uint64_t pool_id = 0;
+  long long pool_hw = 0;
+  // 1: the next step does not depend on this one and runs beside it on the side stream; 2: this step is
+  // that second one (the side stream forks in front of the first and joins behind the second)
+  int fork = 0;
 };
 
 class ExecutionPlan {
  public:
+  ExecutionPlan() = default;
+  ExecutionPlan(const ExecutionPlan &) = delete;
+  ExecutionPlan &operator=(const ExecutionPlan &) = delete;
+  ~ExecutionPlan();
   // Builds the plan; false and *err on a malformed or unsupported graph.
   bool compile(const Json &graph, int dtype, std::string *err);
   size_t arena_size() const { return arena_size_; }
@@ -72,6 +86,11 @@ class ExecutionPlan {
   std::vector<PlanStep> steps_;
   std::map<uint64_t, PlanTensor> tensors_;
   size_t arena_size_ = 0;
+  // side stream (default priority) and fork/join events, made at compile() for the device current then and
+  // again at a run() on another device (outside a stream capture; inside one such a run stays serial)
+  bool ensure_side(int device, void *stream) const;
+  mutable void *side_stream_ = nullptr, *ev_fork_ = nullptr, *ev_join_ = nullptr;
+  mutable int side_device_ = -1;
 };
 
 }  // namespace tracea_amd
