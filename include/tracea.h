@@ -323,7 +323,9 @@ void tracea_set_conv_transpose_by_phase(int32_t enabled);
  * cache on, the regrouped bank of a (device, filter pointer, shape, strides, stride, padding) is built once,
  * kept in device memory of its own and reused by later calls, which then launch nothing but the phase
  * convolutions and allocate nothing: for callers whose filters do not change between calls (inference).
- * Off by default: the library cannot see an in-place update of the filters.  After changing filters in place
+ * Off by default: the library cannot see an in-place update of the filters, nor that a filter tensor was freed
+ * and another of the same shape now lives at its address (the usual outcome of reloading weights under a
+ * caching allocator): both would be served the old bank.  After changing filters in place or replacing them
  * call tracea_conv_transpose_filter_cache_clear (also frees the copies; it waits for the device).  At most 64
  * banks are kept; a miss while the stream is being captured regroups per call as without the cache.  (The
  * reference's kernel indexes its [C*R*S, K] bank in place, src/emitter/conv_transpose.rs:207-236, and has

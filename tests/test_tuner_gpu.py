@@ -57,6 +57,38 @@ def test_tune_gemm_records_a_runnable_winner(tracea_gpu, cache_file):
     assert_close_scaled(c.float().cpu().numpy(), oracle.gemm_f64(a, b), tol_half(512, "f16"), "after tune")
 
 
+def test_cache_records_for_another_operand_type_or_layout_are_ignored(tracea_gpu, cache_file):
+    """A record carries the operand type and the B layout it was measured on; a launch with other operands
+    does not take its variant (a record without the tags counts as f16, k-contiguous B)."""
+    from tracea_amd import capi, tuner as T
+    a = torch.randn(1024, 512, device="cuda")
+    b = torch.randn(512, 1024, device="cuda")             # [K, N] row-major: N-contiguous B
+    tracea_gpu.gemm(a.half(), b.half())
+    default = capi.last_variant("gemm")
+    names = capi.variants("gemm")
+    planted = [c for c in T.propose_gemm_configs(1024, 1024, 512)
+               if names[T.variant_for_config(c)] not in (default, default + "_m16") and c["m_tile"] == 64][0]
+    planted_name = names[T.variant_for_config(planted)]
+    key = "gemm_1024_1024_512_%s" % _device_name()
+
+    def plant(**tags):
+        cache_file.write_text(json.dumps({key: dict(config=planted, score=1.0, timestamp=1, **tags)}))
+        T.cache_reload()
+
+    def ran(dtype, bt):
+        bb = b.to(dtype)
+        tracea_gpu.gemm(a.to(dtype), bb.t().contiguous().t() if bt else bb)
+        return capi.last_variant("gemm")
+
+    plant(operand_dtype="bf16", b_layout="n_contiguous")
+    assert ran(torch.float16, False) == default and ran(torch.bfloat16, False) == planted_name
+    assert ran(torch.bfloat16, True) != planted_name      # same type, B stored [N, K]
+    plant(operand_dtype="f16", b_layout="k_contiguous")
+    assert ran(torch.float16, True) == planted_name and ran(torch.float16, False) == default
+    plant()                                                # no tags: f16, k-contiguous
+    assert ran(torch.float16, True) == planted_name and ran(torch.bfloat16, True) != planted_name
+
+
 def test_autotune_gemm_is_cache_first_and_budgeted(tracea_gpu, cache_file):
     from tracea_amd import tuner as T
     best, score = T.autotune_gemm(512, 512, 256, iterations=4)

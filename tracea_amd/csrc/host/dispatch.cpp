@@ -393,7 +393,9 @@ TraceaStatus make_conv_geometry(int n, int h, int w, int c, int k, int r, int s,
 const DeviceLimits &device_limits() {
   static std::mutex mu;
   static DeviceLimits lim;
+  static std::atomic<bool> settled{false};  // read from the device: from then on nothing changes and nobody locks
   static bool from_device = false;
+  if (settled.load(std::memory_order_acquire)) return lim;
   std::lock_guard<std::mutex> lk(mu);
   if (!from_device && runtime_ready()) {
     hipDeviceProp_t prop;
@@ -405,14 +407,17 @@ const DeviceLimits &device_limits() {
       CacheEntry e;
       if (tuning_cache_get(gemm_cache_key(4096, 4096, 4096, prop.name), &e) && e.score > 0.0f) {
         const int vi = contraction_variant_for_config(e.config);
+        // (a record of the 32x32x16 member only: the selector gives the 16x16x32 members further factors, and a
+        // rate divided by less than the selector multiplies by would come out too high)
         if (vi >= 0 && contraction_variant(vi).bm == 256 && contraction_variant(vi).bn == 256 &&
-            contraction_variant(vi).pipeline == 2)
+            contraction_variant(vi).pipeline == 2 && contraction_variant(vi).mfma == 32)
           // score TFLOP/s = 2 MAC: MAC per microsecond and CU at the variant's efficiency prior (1.5, x1.04 on 8 waves)
           lim.slot_rate = (double)e.score * 1e6 / 2.0 / lim.cus /
                           (1.5 * (contraction_variant(vi).waves_m * contraction_variant(vi).waves_n == 8 ? 1.04 : 1.0));
       }
     }
     from_device = true;
+    settled.store(true, std::memory_order_release);
   }
   return lim;
 }
@@ -641,6 +646,18 @@ unsigned *fuse_counters(int device, hipStream_t stream) {
   return slot;
 }
 
+// A one-launch split whose launch was refused may leave tickets behind (some workgroups ran, some did
+// not): the counters of the stream go back to zero, in stream order, unless the stream is being captured
+// (then nothing was launched yet and the capture fails as a whole).
+void reset_fuse_counters(unsigned *cnt, hipStream_t stream) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (cnt == nullptr || hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return;
+  }
+  if (hipMemsetAsync(cnt, 0, kFuseTiles * sizeof(unsigned), stream) != hipSuccess) (void)hipGetLastError();
+}
+
 // Launches `args` on variant v, split along K when that pays; `chain` is the operator chain
 // of the call (args.epi is ignored).
 // The workspace of a launch split `splits` ways: the per-stream buffer (null when it cannot be had:
@@ -688,7 +705,9 @@ TraceaStatus launch_maybe_split(const char *what, const ContractionVariant &v, C
       args.fuse_ws = (float *)fws;
       args.fuse_count = cnt;
       t_last_splits = splits;
-      return hip_status(what, v.launch(args, conv, dtype, b_ncontig, stream));
+      const TraceaStatus st = hip_status(what, v.launch(args, conv, dtype, b_ncontig, stream));
+      if (st != TRACEA_SUCCESS) reset_fuse_counters(cnt, stream);
+      return st;
     }
   }
   TraceaStatus ws = TRACEA_SUCCESS;
@@ -815,7 +834,9 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
         args.fuse_ws = (float *)fws;
         args.fuse_count = cnt;
         t_last_splits = splits;
-        return hip_status("gemm_f32 launch", launch_gemm_f32(args, tile, stream));
+        const TraceaStatus fst = hip_status("gemm_f32 launch", launch_gemm_f32(args, tile, stream));
+        if (fst != TRACEA_SUCCESS) reset_fuse_counters(cnt, stream);
+        return fst;
       }
     }
     TraceaStatus ws = TRACEA_SUCCESS;
