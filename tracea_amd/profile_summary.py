@@ -26,7 +26,7 @@ import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 # dominant kernel of a workload: the first of these name fragments that occurs in the run
-KERNELS = {"gemm": ["contraction_kernel"], "conv": ["conv_resident_kernel", "conv_patch_kernel", "contraction_kernel"],
+KERNELS = {"gemm": ["contraction_kernel"], "conv": ["conv_wave16_kernel", "conv_resident_kernel", "conv_patch_kernel", "contraction_kernel"],
            "attention": ["fa2_fwd"], "attention_causal": ["fa2_fwd"], "copy": ["copyBuffer", "copy"]}
 ALGORITHMIC_BYTES = {"gemm": 2.0 * 3 * 4096 * 4096, "conv": 2.0 * (2 * 32 * 56 * 56 * 64 + 64 * 576),
                      "attention": 2.0 * 4 * 4 * 32 * 4096 * 128, "attention_causal": 2.0 * 4 * 4 * 32 * 4096 * 128}
