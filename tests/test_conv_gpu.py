@@ -189,7 +189,8 @@ def test_filter_resident_variant(tracea_gpu, dtype, member, cin):
 
 
 # the members for few pixels and many channels (K split over the waves of a workgroup)
-KSPLIT_MEMBERS = [("c112x64_c256_s4_w16_ksplit", 256), ("c64x64_c512_s4_w16_ksplit", 512)]
+KSPLIT_MEMBERS = [("c112x64_c256_s4_w16_ksplit", 256), ("c64x64_c512_s4_w16_ksplit", 512),
+                  ("c32x64_c256_s4_w16_ksplit", 256), ("c16x64_c256_s4_w16_ksplit", 256)]
 KSPLIT_SHAPES = [  # n, h, w, k, filter size, stride, pad, dilation
     (32, 14, 14, 256, 3, 1, 1, 1),    # a ResNet's 14x14 stage at batch 32: tiles of 98 pixels (7 rows) at 256 channels
     (32, 7, 7, 512, 3, 1, 1, 1),      # its 7x7 stage: one tile of 49 pixels per image

@@ -255,12 +255,15 @@ __global__ void __launch_bounds__(CK_THREADS) conv_ksplit16_kernel(const Contrac
     for (int p = 0; p < NPB; ++p) pp[p] = patch + a_base[p];
 #pragma unroll
     for (int i = 0; i < 4; ++i) fp[i] = ring + f_base[i];
+    // (in the order the MFMAs want them: the first pixel block's fragment right behind the first filter block's)
     auto read = [&](auto setc) __attribute__((always_inline)) {
       constexpr int set = decltype(setc)::value;
+      xb[set][0] = *(const u32x4 *)fp[0];
+      xa[set][0] = *(const u32x4 *)pp[0];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xb[set][i] = *(const u32x4 *)fp[i];
+      for (int i = 1; i < 4; ++i) xb[set][i] = *(const u32x4 *)fp[i];
 #pragma unroll
-      for (int p = 0; p < NPB; ++p) xa[set][p] = *(const u32x4 *)pp[p];
+      for (int p = 1; p < NPB; ++p) xa[set][p] = *(const u32x4 *)pp[p];
     };
     // on to the next stage: the next 128 channels of the tap, or the next tap; the ring slot after this one
     // (past the last stage the addresses stay: the last stage is read again, unused)
@@ -275,10 +278,12 @@ __global__ void __launch_bounds__(CK_THREADS) conv_ksplit16_kernel(const Contrac
       const int tap_step = wrap_c ? (wrap_s ? step_r : step_s) - (CPT - 1) * 256 : 256;
       const int p_step = more ? tap_step : 0;
       const int f_step = !more ? 0 : ((s_now + 1) % RING == 0 ? -(RING - 1) * CK_STAGE_BYTES : CK_STAGE_BYTES);
+      fp[0] += f_step;
+      pp[0] += p_step;
 #pragma unroll
-      for (int p = 0; p < NPB; ++p) pp[p] += p_step;
+      for (int i = 1; i < 4; ++i) fp[i] += f_step;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) fp[i] += f_step;
+      for (int p = 1; p < NPB; ++p) pp[p] += p_step;
     };
     auto mma = [&](auto setc) __attribute__((always_inline)) {
       constexpr int s = decltype(setc)::value;
@@ -286,7 +291,8 @@ __global__ void __launch_bounds__(CK_THREADS) conv_ksplit16_kernel(const Contrac
       for (int p = 0; p < NPB; ++p)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[p][i] = Mfma16<DT>::run(xb[s][i], xa[s][p], acc[p][i]);
-      Interleave<0, 4 * NPB, 0x100, NPB + 4, 0x100, 0>::run();
+      // per MFMA its share of the address updates and, behind them, of the reads they feed
+      Interleave<0, 4 * NPB, 0x002, NPB + 4, 0x100, NPB + 4>::run();
       __builtin_amdgcn_sched_barrier(0);
     };
     using std::integral_constant;

@@ -1766,7 +1766,10 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       const ContractionVariant &cv = contraction_variant(i);
       if (cv.pipeline < 7 || cv.pipeline > 10) continue;
       ContractionArgs probe = a;
-      if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n * 4 >= device_limits().cus * 3 &&
+      // (the K-split members with tiles of one or two pixel blocks are for small launches: 14x14x256 at batch 1
+      // 6.4 us on 52 workgroups against 8.4 streamed and split along K; from 48 workgroups on)
+      const long long enough = cv.pipeline == 9 && cv.bm <= 32 ? 48 * 4 : device_limits().cus * 3;
+      if (plan_conv_resident(g, cv, plan.w_ncontig, &probe) && (long long)probe.grid_m * probe.grid_n * 4 >= enough &&
           probe.p_tm * 4 >= cv.bm * 3) {
         vi = i;
         resident_chosen = true;
