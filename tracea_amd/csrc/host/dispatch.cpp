@@ -1769,11 +1769,11 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       // (the K-split members with tiles of one or two pixel blocks are for small launches: 14x14x256 at batch 1
       // 6.4 us on 52 workgroups against 8.4 streamed and split along K; from 48 workgroups on)
       const long long enough = cv.pipeline == 9 && cv.bm <= 32 ? 48 * 4 : device_limits().cus * 3;
-      // (tile at least three quarters of the member's largest; the K-split members, whose waves all work on
-      // every pixel block there is, from two fifths: 14x14x256 at batch 16, tiles of 49 of 112 pixels, 11.8 us
+      // (tile at least three quarters of the member's largest; the larger K-split members, whose waves all work
+      // on every pixel block there is, from two fifths: 14x14x256 at batch 16, tiles of 49 of 112 pixels, 11.8 us
       // against 13.1 on the 32-pixel member)
       if (!plan_conv_resident(g, cv, plan.w_ncontig, &probe)) continue;
-      const bool tile_ok = cv.pipeline == 9 ? probe.p_tm * 5 >= cv.bm * 2 : probe.p_tm * 4 >= cv.bm * 3;
+      const bool tile_ok = cv.pipeline == 9 && cv.bm > 32 ? probe.p_tm * 5 >= cv.bm * 2 : probe.p_tm * 4 >= cv.bm * 3;
       if ((long long)probe.grid_m * probe.grid_n * 4 >= enough && tile_ok) {
         vi = i;
         resident_chosen = true;
