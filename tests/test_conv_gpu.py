@@ -540,3 +540,51 @@ def test_error_paths(tracea_gpu):
     w12 = torch.zeros(8, 3, 3, 12, device="cuda", dtype=torch.float16)
     assert call(x12, w12, out) == capi.UNSUPPORTED_CONFIG             # C % 8 != 0
     assert "multiple of 8" in capi.last_error()
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_random_geometry_on_the_patch_in_lds_members(tracea_gpu, seed):
+    """Seeded random geometry (sizes, filter extents, strides, padding, dilation, batch, filter count, operand
+    type, chain) on every 16x16x32 member that keeps the input patch in LDS, forced where its plan takes the
+    shape, against torch's fp32 convolution of the same half-precision operands."""
+    from tracea_amd import capi
+    rng = np.random.default_rng(seed)
+    names = capi.variants("conv2d")
+    ran = {}
+    for _ in range(60):
+        c = int(rng.choice([8, 64, 128, 256, 512]))
+        fr = int(rng.choice([1, 3, 3, 3, 5]))
+        fs = fr if rng.random() < 0.8 else int(rng.choice([1, 3, 5]))
+        stride = (int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))) if rng.random() < 0.3 else int(rng.choice([1, 1, 1, 2]))
+        dil = int(rng.choice([1, 1, 1, 2]))
+        if c == 8:
+            fr, fs, dil = 7, int(rng.choice([7, 5, 8])), 1
+            stride = int(rng.choice([2, 4])) if isinstance(stride, int) else (stride[0] + 1, 2 * stride[1])
+        pad = (int(rng.integers(0, 4)), int(rng.integers(0, 4))) if rng.random() < 0.3 else int(rng.integers(0, 3))
+        n = int(rng.choice([1, 2, 4, 8, 16]))
+        h, w = (int(rng.integers(20, 90)), int(rng.integers(20, 90))) if c == 8 else (int(rng.integers(5, 30)), int(rng.integers(5, 30)))
+        k = int(rng.choice([64, 128, 40, 72]))
+        ph, pw = (pad, pad) if isinstance(pad, int) else pad
+        if h + 2 * ph < dil * (fr - 1) + 1 or w + 2 * pw < dil * (fs - 1) + 1:
+            continue
+        tdt = torch.float16 if rng.random() < 0.7 else torch.bfloat16
+        epi = str(rng.choice(["bias+relu", "none", "bias"]))
+        x = torch.randn(n, h, w, c, device="cuda").to(tdt)
+        wt = (torch.randn(k, fr, fs, c, device="cuda") * (2.0 / (fr * fs * c)) ** 0.5).to(tdt)
+        bias = torch.randn(k, device="cuda") * 0.1
+        ref = torch.nn.functional.conv2d(x.float().permute(0, 3, 1, 2), wt.float().permute(0, 3, 1, 2),
+                                         bias=bias if "bias" in epi else None, stride=stride, padding=pad, dilation=dil)
+        ref = (torch.relu(ref) if "relu" in epi else ref).permute(0, 2, 3, 1).cpu().numpy()
+        for member in [nm for nm in names if ("_c%d_" % c) in nm and "_w16_" in nm]:
+            capi.force_variant("conv2d", member)
+            try:
+                y = tracea_gpu.conv2d(x, wt, bias=bias if "bias" in epi else None, stride=stride, padding=pad, dilation=dil,
+                                      epilogue=epi)
+            finally:
+                capi.force_variant("conv2d", -1)
+            if capi.last_variant("conv2d") != member:
+                continue  # (its plan does not take the shape: another kernel ran, tested elsewhere)
+            ran[member] = ran.get(member, 0) + 1
+            assert_close_scaled(y.float().cpu().numpy(), ref, tol_half(fr * fs * c, "f16" if tdt == torch.float16 else "bf16"),
+                                "%s %s" % (member, (n, h, w, c, k, fr, fs, stride, pad, dil, epi)))
+    assert len(ran) >= 5 and sum(ran.values()) >= 40, ran
