@@ -114,7 +114,7 @@ def test_variant_table():
     gemm = capi.variants("gemm")
     assert gemm and gemm == capi.variants("conv2d")
     assert all(re.match(r"t\d+x\d+x\d+_w\dx\d", n) or re.match(r"c\d+x\d+_w\dx\d_s\d_patch", n) or
-               re.match(r"c\d+x\d+_k\d+_resident", n) or re.match(r"c\d+x\d+_c\d+(_s\d|_r\d)?_w16_(resident|patch|ksplit|thin)", n)
+               re.match(r"c\d+x\d+_k\d+_resident", n) or re.match(r"c\d+x\d+_c\d+(_s\d|_r\d|_w\d)?_w16_(resident|patch|ksplit|thin)", n)
                for n in gemm)
     attn = capi.variants("attention")
     assert any("d128" in n for n in attn)

@@ -149,7 +149,8 @@ RESIDENT_SHAPES = [  # n, h, w, k, stride, pad, dilation: 64 input channels, 3x3
 
 # the members that keep the input patch in LDS with the filter slab resident beside it or in a ring of taps,
 # and the input channels each is compiled for
-LDS_MEMBERS = [("c448x64_k576_resident", 64), ("c400x64_c64_w16_resident", 64), ("c208x64_c128_s4_w16_patch", 128)]
+LDS_MEMBERS = [("c448x64_k576_resident", 64), ("c400x64_c64_w16_resident", 64), ("c400x64_c64_w8_w16_resident", 64),
+               ("c208x64_c128_s4_w16_patch", 128)]
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

@@ -26,7 +26,7 @@ const ContractionVariant &TRACEA_CAT(contraction_variant_, V_NAME)() {
       &launch_conv_resident<V_STAGES, 4>, 32};  // 64 input channels: 4 k-steps per tap
 #elif V_DIRECT == 7
       (size_t)CW_TABLE_BYTES,  // patch and filter slab, sized by the problem, come on top
-      &launch_conv_wave16<V_BK, (V_BM / 16 - 1) / 4, 0>, 16};
+      &launch_conv_wave16<V_BK, (V_BM / 16 - 1) / V_WM, 0, V_WM>, 16};  // waves_m multiplying waves
 #elif V_DIRECT == 8
       (size_t)V_STAGES * cw_ring_stage_bytes(V_BK) + CW_TABLE_BYTES,  // the patch comes on top
       &launch_conv_wave16<V_BK, (V_BM / 16 - 1) / 4, V_STAGES>, 16};

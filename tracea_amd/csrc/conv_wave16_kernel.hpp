@@ -13,8 +13,10 @@
 // pixel block 4*PBW that is left over (392 pixels = 24.5 blocks: 6 whole blocks per wave and a quarter of
 // the 25th; with 32-pixel blocks the same tile was 28 units of which 24.5 held pixels).  A wave reads
 // PBW + 1 pixel fragments and 4 filter fragments of 1 KB per k-step for 4*PBW + 1 MFMAs of 16 cycles;
-// LDS delivers 128 bytes per clock to the CU, i.e. 0.5 KB per MFMA slot with all four matrix pipes busy:
-// PBW = 6 stays below that (0.44), PBW = 3 (0.62) runs at the LDS rate.  Four more waves only move data.
+// PBW = 6 is 0.44 KB of LDS reads per MFMA, PBW = 3 0.62.  Four more waves only move data; or (WK = 8) all
+// eight multiply, three blocks each: the two waves of a SIMD do not multiply faster than one (468 MFMAs in
+// 9.9 k cycles against 450 in 8.5 k), but the store phase is shared by twice the waves (11.3 us against 11.7
+// for N32 56x56 64->64).
 //
 // A wave's pixels are consecutive, its results leave from registers (below), and nothing after the
 // operand wait is shared between the multiplying waves: each runs on its own.
@@ -48,8 +50,9 @@ inline int cw_resident_filter_bytes(int k) {
   return (chunks + CW_THREADS - 1) / CW_THREADS * CW_THREADS * 16;
 }
 
-template <int DT, int CIN, int PBW, int RING>
+template <int DT, int CIN, int PBW, int RING, int WK = 4>
 __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const ContractionArgs args) {
+  static_assert(WK == 4 || (WK == 8 && RING == 0), "eight multiplying waves only with the resident filter slab");
   constexpr int NT = CW_THREADS, BN = 64, NW = NT / 64;
   constexpr int KPT = CIN / 32;   // 32-wide k-steps per filter tap
   constexpr int TAPB = CIN * 2;   // bytes of one tap in a filter row
@@ -81,8 +84,9 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int w = wave_u & 3;          // SIMD; the multiplying wave's index
-  const bool worker = wave_u < 4;
+  const int w = wave_u & 3;          // SIMD; the filter block a multiplying wave starts with
+  const int ww = wave_u & (WK - 1);  // the multiplying wave's index: its pixel blocks are ww*PBW .. + PBW-1
+  const bool worker = wave_u < WK;
   const int l15 = lane & 15, q = lane >> 4;
 
   // ---- which tile ----
@@ -222,7 +226,7 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   int a_base[NPF];
 #pragma unroll
   for (int i = 0; i < NPF; ++i) {
-    const int blk = i < PBW ? w * PBW + i : 4 * PBW;
+    const int blk = i < PBW ? ww * PBW + i : WK * PBW;
     const int pr = blk * 16 + l15;
     const int prc = pr < npix ? pr : npix - 1;
     int ho, wo;
@@ -414,12 +418,13 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
       }
       static_for<0, PBW>([&](auto pc) {
         constexpr int p = decltype(pc)::value;
-        const int pr = (w * PBW + p) * 16 + l15;
+        const int pr = (ww * PBW + p) * 16 + l15;
         E::pixel_block(acc[p], fb, ta, tb, pr < npix ? pr : -1, q, rsrc_c, rsrc_r, row_c, row_r);
       });
       {  // the shared block: filter block w only
-        const int pr = 4 * PBW * 16 + l15;
-        E::single_block(acc_x, ta[0], tb[0], w * 16 + q * 4, pr < npix ? pr : -1, rsrc_c, rsrc_r, row_c, row_r);
+        // (with eight multiplying waves the shared block is computed by waves w and w + 4 alike: one stores)
+        const int pr = WK * PBW * 16 + l15;
+        E::single_block(acc_x, ta[0], tb[0], w * 16 + q * 4, (pr < npix && wave_u < 4) ? pr : -1, rsrc_c, rsrc_r, row_c, row_r);
       }
     };
 #define TRACEA_CW_FORM(F) run_form(std::integral_constant<int, F>{})
@@ -435,14 +440,14 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   if (worker) {
     static_for<0, PBW>([&](auto pc) {
       constexpr int p = decltype(pc)::value;
-      const int pr = (w * PBW + p) * 16 + l15;
+      const int pr = (ww * PBW + p) * 16 + l15;
       if (pr < npix) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) *(f32x4 *)(stage + pr * SP + (w ^ i) * 16 + q * 4) = acc[p][i];
       }
     });
-    const int pr = 4 * PBW * 16 + l15;
-    if (pr < npix) *(f32x4 *)(stage + pr * SP + w * 16 + q * 4) = acc_x;
+    const int pr = WK * PBW * 16 + l15;
+    if (pr < npix && wave_u < 4) *(f32x4 *)(stage + pr * SP + w * 16 + q * 4) = acc_x;
   }
   __syncthreads();
   const int ec = (tid & 7) * 8;
@@ -469,9 +474,9 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
 
 // bm = 16 * (4 * PBW + 1) pixels at most per workgroup; CIN input channels exactly; RING = 0: the whole
 // filter slab (64 x K) resident beside the patch, else a ring of RING one-tap stages.
-template <int CIN, int PBW, int RING>
+template <int CIN, int PBW, int RING, int WK = 4>
 int launch_conv_wave16(const ContractionArgs &a, bool conv, int dtype, bool b_ncontig, hipStream_t stream) {
-  if (!conv || b_ncontig || a.c_in != CIN || a.K != a.r_sz * a.s_sz * CIN || a.p_tm <= 0 || a.p_tm > 16 * (4 * PBW + 1) ||
+  if (!conv || b_ncontig || a.c_in != CIN || a.K != a.r_sz * a.s_sz * CIN || a.p_tm <= 0 || a.p_tm > 16 * (WK * PBW + 1) ||
       a.p_np_bytes <= 0)
     return (int)hipErrorInvalidValue;
   const size_t filt = RING ? (size_t)RING * cw_ring_stage_bytes(CIN) : (size_t)cw_resident_filter_bytes(a.K);
@@ -482,7 +487,7 @@ int launch_conv_wave16(const ContractionArgs &a, bool conv, int dtype, bool b_nc
   const dim3 grid((unsigned)(a.grid_m * a.grid_n)), block(CW_THREADS);
 #define TRACEA_LAUNCH_CW(DTV)                                                                        \
   do {                                                                                               \
-    auto kfn = conv_wave16_kernel<DTV, CIN, PBW, RING>;                                               \
+    auto kfn = conv_wave16_kernel<DTV, CIN, PBW, RING, WK>;                                               \
     static bool attr_done = false;                                                                   \
     if (!attr_done) {                                                                                \
       hipError_t e = hipFuncSetAttribute((const void *)kfn, hipFuncAttributeMaxDynamicSharedMemorySize, \
