@@ -239,6 +239,12 @@ def roofline_block(name, flops, dev_s, dtype, cus, variant, inputs, clock_ghz=No
         block["peak_at_measured_clock"] = round(at_clock, 1)
         block["clock_ghz"] = round(clock, 3)
         block["clock_from"] = source
+        # the probe reads the clock of the one CU it sits on, averaged over windows of some 150 us: an upper
+        # bound for launches that leave that CU a free wave slot or whose phases alternate (stamps written by
+        # the kernels themselves read 1.7-1.9 GHz over a causal attention wave's life and 1.75 GHz over the
+        # convolution's main loop where the probe reads 2.4 and 2.2)
+        if name in ("conv", "attention_causal"):
+            block["clock_is_upper_bound"] = True
         block["frac_of_peak_at_measured_clock"] = round(achieved / at_clock, 4)
     if row:
         block["counters_from"] = row.get("variant")
