@@ -44,15 +44,13 @@ constexpr int cw_ring_cpb(int cin) { return (cin / 8) | 1; }
 // (a stage is whole load instructions of the four helper waves: the lanes past its 64 rows write zeros)
 constexpr int cw_ring_iters(int cin) { return (64 * cw_ring_cpb(cin) + 255) / 256; }
 constexpr int cw_ring_stage_bytes(int cin) { return cw_ring_iters(cin) * 256 * 16; }
-// (the resident slab: whole load instructions of the eight waves)
-inline int cw_resident_filter_bytes(int k) {
-  const int chunks = 64 * ((k / 8) | 1);
-  return (chunks + CW_THREADS - 1) / CW_THREADS * CW_THREADS * 16;
-}
+// (the resident slab: tap t of the 64 filters at t * 64 * 2 * CIN bytes, without padding)
+inline int cw_resident_filter_bytes(int k) { return 64 * k * 2; }
 
 template <int DT, int CIN, int PBW, int RING, int WK = 4>
 __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const ContractionArgs args) {
   static_assert(WK == 4 || (WK == 8 && RING == 0), "eight multiplying waves only with the resident filter slab");
+  static_assert(RING != 0 || CIN == 64, "the resident slab's layout: one load instruction per thread and tap");
   constexpr int NT = CW_THREADS, BN = 64, NW = NT / 64;
   constexpr int KPT = CIN / 32;   // 32-wide k-steps per filter tap
   constexpr int TAPB = CIN * 2;   // bytes of one tap in a filter row
@@ -73,10 +71,10 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   unsigned char *patch = smem;
   unsigned char *filt = smem + args.p_np_bytes;
-  const int K = args.K;
   const int taps = args.r_sz * args.s_sz;
-  const int CPB = RING ? RCPB : ((K >> 3) | 1);
-  const int filt_bytes = RING ? RING * RSTAGE : (64 * CPB + NT - 1) / NT * NT * 16;
+  constexpr int CPB = RCPB;        // (ring) 16-byte chunks per filter row of a stage
+  constexpr int TAPS = 64 * TAPB;  // (resident slab) bytes of one tap of the 64 filters
+  const int filt_bytes = RING ? RING * RSTAGE : taps * TAPS;
   // (the operand table lies behind the operands or, if that is more, behind the general epilogue's staging)
   const int operand_bytes = args.p_np_bytes + filt_bytes, staging_bytes = args.p_tm * (BN + 4) * 4;
   float *table = (float *)(smem + (operand_bytes > staging_bytes ? operand_bytes : staging_bytes));
@@ -112,8 +110,18 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   __amdgpu_buffer_rsrc_t rsrc_w =
       __builtin_amdgcn_make_buffer_rsrc((void *)args.B, 0, (int)args.b_bytes, 0x00020000);
 
+  // ---- epilogue form ----
+  // sig >= 0: the chain reads [affine] [ReLU] [residual] [ReLU] (bit 0 affine, 1 first ReLU, 2 residual,
+  // 3 second ReLU), affine = v*a + b per channel; table [0..63] = a, [64..127] = b.  sig < 0: any other
+  // chain, table in the layout of chain_table_value.
+  const int sig = args.fe.sig;
+  // the resident slab's nine taps are awaited in two groups (the general chain's table takes the old road)
+  const bool prog = RING == 0 && taps == 9 && sig >= 0;
+
   // ---- filters ----
-  // resident: chunk c of the area is filter row c / CPB, 16-byte part c % CPB (the last part is padding)
+  // resident: tap t of the 64 filters at t * TAPS, row r at r * TAPB, its 16-byte part p at position
+  // p ^ ((r >> 1) & 7) (the 16 rows of a fragment then read 16 different bank groups); one load instruction per
+  // thread and tap, taps in ascending order behind the patch: the first taps are multiplied while the others travel
   // ring: the helper waves bring tap t into stage t % RING: chunk c is row c / RCPB, part c % RCPB of the tap
   unsigned ring_voff[RIT];
   const int htid = tid - 256;
@@ -171,18 +179,15 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
       }
     }
   }
-  // (the patch first: its rows come from memory, the filters from the L2 every workgroup shares)
+  // (the patch first: every tap needs it; its rows come from memory, the filters from the L2 every workgroup shares)
   if constexpr (RING == 0) {
-    const int fit = (64 * CPB + NT - 1) / NT;
-    for (int it = 0; it < fit; ++it) {
-      const int chunk = it * NT + tid;
-      int row, part;
-      fast_divmod(chunk, args.p_pw_m, args.p_pw_s, CPB, row, part);  // (p_pw_m/s: the reciprocal of CPB here)
-      const bool ok = (part < (K >> 3)) & (row < BN) & (n0 + row < N);
-      const unsigned voff = ok ? (unsigned)(((n0 + row) * (int)args.ldb + part * 8) * 2) : OOB;
-      unsigned char *dst = filt + (it * NT + wave_u * 64) * 16;
+    const int row = tid >> 3, pos = tid & 7;
+    const unsigned voff = n0 + row < N ? (unsigned)(((n0 + row) * (int)args.ldb + ((pos ^ ((row >> 1) & 7)) << 3)) * 2) : OOB;
+    unsigned char *dst = filt + wave_u * 1024;
+    for (int t = 0; t < taps; ++t) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (__attribute__((address_space(3))) void *)dst, 16, (int)voff,
-                                               0, 0, 0);
+                                               t * TAPB, 0, 0);
+      dst += TAPS;
     }
   }
   // ring: the first RING taps follow the patch, one per stage
@@ -194,32 +199,78 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
     }
   }
 
-  // ---- epilogue form and this thread's entry of the operand table (requested now, read after the wait) ----
-  // sig >= 0: the chain reads [affine] [ReLU] [residual] [ReLU] (bit 0 affine, 1 first ReLU, 2 residual,
-  // 3 second ReLU), affine = v*a + b per channel; table [0..63] = a, [64..127] = b.  sig < 0: any other
-  // chain, table in the layout of chain_table_value.
-  const int sig = args.fe.sig;
+  // ---- this thread's entry of the operand table (requested behind the operands, worked out where the table is
+  // published: in front of the first barrier, or -- prog -- of the third, when everything has landed anyway) ----
+  // Waves 0 and 1 (threads 0..127: a of channel n0 + tid, b of channel n0 + tid - 64) request the raw vector
+  // entries, every lane and the same number per wave, so that the waits for the taps can count them: 1 (bias,
+  // scale and shift) or 4 (BatchNorm: gamma, variance, beta, mean).
   constexpr int TPT = CW_TABLE_BYTES / 4 / NT;
-  float tabr = 0.0f, tabg[TPT];
+  float tabg[TPT];
+  // (two sets of registers, one per road: a set that both roads touched would be copied where they meet, and a
+  // copy reads the registers -- it waits for the requests)
+  unsigned traw_now[4] = {0u, 0u, 0u, 0u}, traw_late[4] = {0u, 0u, 0u, 0u};
+  const int tab_loads = (sig >= 0 && (sig & 1) && wave_u < 2) ? (args.fe.aff_kind == TRACEA_EPI_OP_BATCHNORM ? 4 : 1) : 0;
   if (sig < 0) {
 #pragma unroll
     for (int i = 0; i < TPT; ++i) {
       const int e = tid + i * NT;
       tabg[i] = chain_table_value(args.epi, e / (2 * BN), (e / BN) & 1, n0 + e % BN, N);
     }
-  } else if ((sig & 1) && tid < 2 * BN) {
-    const int which = tid / BN, n = n0 + tid % BN;
-    if (args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD) {
-      float one[1] = {1.0f};
-      if (which == 1) load_as_float<1>(args.fe.p0, args.fe.aff_dtype, n, 1, one);
-      tabr = one[0];
-    } else if (args.fe.aff_kind == TRACEA_EPI_OP_SCALE_SHIFT) {
-      tabr = ((const float *)(which == 0 ? args.fe.p0 : args.fe.p1))[n];
-    } else {  // BatchNorm folded: a = gamma / sqrt(var + eps), b = beta - mean * a
-      const float scale = ((const float *)args.fe.p0)[n] * (1.0f / sqrtf(((const float *)args.fe.p3)[n] + args.fe.epsilon));
-      tabr = which == 0 ? scale : ((const float *)args.fe.p1)[n] - ((const float *)args.fe.p2)[n] * scale;
-    }
+  } else if (tab_loads != 0) {
+    auto request = [&](unsigned (&r)[4]) __attribute__((always_inline)) {
+      const int which = tid / BN;
+      const int n = min(n0 + (tid & (BN - 1)), N - 1);
+      if (args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD) {
+        r[0] = args.fe.aff_dtype == DT_F32 ? ((const unsigned *)args.fe.p0)[n] : (unsigned)((const unsigned short *)args.fe.p0)[n];
+      } else if (args.fe.aff_kind == TRACEA_EPI_OP_SCALE_SHIFT) {
+        r[0] = ((const unsigned *)(which == 0 ? args.fe.p0 : args.fe.p1))[n];
+      } else {
+        r[0] = ((const unsigned *)args.fe.p0)[n];
+        r[1] = ((const unsigned *)args.fe.p3)[n];
+        r[2] = ((const unsigned *)args.fe.p1)[n];
+        r[3] = ((const unsigned *)args.fe.p2)[n];
+      }
+    };
+    if (prog) request(traw_late);
+    else request(traw_now);
   }
+  // (called by every thread, between a wait that covers the requests above and a barrier)
+  auto publish_table = [&](unsigned (&rv)[4]) __attribute__((always_inline)) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) asm volatile("" : "+v"(rv[e]));  // (nothing of this moves in front of the wait)
+    if (sig < 0) {
+#pragma unroll
+      for (int i = 0; i < TPT; ++i) table[tid + i * NT] = tabg[i];
+    } else if (tab_loads != 0) {
+      const int which = tid / BN;
+      float t;
+      if (args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD) {
+        const float bv = args.fe.aff_dtype == DT_F32   ? __builtin_bit_cast(float, rv[0])
+                         : args.fe.aff_dtype == DT_F16 ? (float)__builtin_bit_cast(_Float16, (unsigned short)rv[0])
+                                                       : __builtin_bit_cast(float, rv[0] << 16);
+        t = which == 0 ? 1.0f : bv;
+      } else if (args.fe.aff_kind == TRACEA_EPI_OP_SCALE_SHIFT) {
+        t = __builtin_bit_cast(float, rv[0]);
+      } else {  // BatchNorm folded: a = gamma / sqrt(var + eps), b = beta - mean * a
+        const float scale = __builtin_bit_cast(float, rv[0]) * (1.0f / sqrtf(__builtin_bit_cast(float, rv[1]) + args.fe.epsilon));
+        t = which == 0 ? scale : __builtin_bit_cast(float, rv[2]) - __builtin_bit_cast(float, rv[3]) * scale;
+      }
+      table[tid] = t;
+    }
+  };
+  // vmcnt(LEFT + this wave's table requests): all but the last LEFT taps of the resident slab have landed
+  auto wait_taps = [&](auto left_tag) __attribute__((always_inline)) {
+    constexpr int L = decltype(left_tag)::value;
+    if (tab_loads == 0) __builtin_amdgcn_s_waitcnt(0x0f70 | L);
+    else if (tab_loads == 1) __builtin_amdgcn_s_waitcnt(0x0f70 | (L + 1));
+    else __builtin_amdgcn_s_waitcnt(0x0f70 | (L + 4));
+  };
+
+  // A bias that opens a chain of the fast form is where the accumulators start (one fp32 rounding apart from
+  // adding it last, and a hundred additions less in the epilogue of a wave that has nobody to share them with).
+  // (Not with the taps awaited in groups: the accumulators would wait for the last request of the wave.)
+  const bool bias_init = !prog && sig >= 0 && (sig & 1) && args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD;
+  const int form_sig = bias_init ? (sig & ~1) : sig;
 
   // ---- per-lane operand addresses (worked out while the operands travel) ----
   // pixel fragment i < PBW: block w*PBW + i; fragment PBW: the shared block 4*PBW
@@ -235,9 +286,13 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   }
   // filter fragment i: filter block w ^ i (fragment 0 is the wave's own block, which the shared pixel block
   // multiplies; fragments 2j and 2j+1 are neighbours in the channel order): row (w ^ i)*16 + l15, 16-byte part q
+  // (resident slab: the address of the tap's first k-step; the second one is 64 bytes up or down, by the row)
   int f_base[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) f_base[i] = (((w ^ i) * 16 + l15) * CPB + q) * 16;
+  for (int i = 0; i < 4; ++i) {
+    const int row = (w ^ i) * 16 + l15;
+    f_base[i] = RING ? (row * CPB + q) * 16 : row * TAPB + ((q ^ ((row >> 1) & 7)) << 4);
+  }
   int step_s = args.dil_w * pitch;
   int step_r = tap_h * pitch - (args.s_sz - 1) * step_s;
   int off_last = ((args.r_sz - 1) * tap_h + (args.s_sz - 1) * args.dil_w) * pitch;
@@ -248,28 +303,38 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(f_base[i]));
   asm volatile("" : "+s"(step_s), "+s"(step_r), "+s"(off_last), "+s"(s_size));
 
-  // A bias that opens a chain of the fast form is where the accumulators start (one fp32 rounding apart from
-  // adding it last, and a hundred additions less in the epilogue of a wave that has nobody to share them with).
-  const bool bias_init = sig >= 0 && (sig & 1) && args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD;
-  const int form_sig = bias_init ? (sig & ~1) : sig;
-  f32x4 start[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float b4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (bias_init) load_as_float<4>(args.fe.p0, args.fe.aff_dtype, n0 + (w ^ i) * 16 + q * 4, 4, b4);
-    start[i] = f32x4{b4[0], b4[1], b4[2], b4[3]};
-  }
   f32x4 acc[PBW][4], acc_x;
+  if (bias_init) {  // (a branch of its own: the wait for these loads must not stand on the other road)
+    f32x4 start[4];
 #pragma unroll
-  for (int p = 0; p < PBW; ++p)
+    for (int i = 0; i < 4; ++i) {
+      float b4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+      load_as_float<4>(args.fe.p0, args.fe.aff_dtype, n0 + (w ^ i) * 16 + q * 4, 4, b4);
+      start[i] = f32x4{b4[0], b4[1], b4[2], b4[3]};
+    }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) acc[p][i] = start[i];
-  acc_x = start[0];
+    for (int p = 0; p < PBW; ++p)
 #pragma unroll
-  for (int p = 0; p < PBW; ++p)
+      for (int i = 0; i < 4; ++i) acc[p][i] = start[i];
+    acc_x = start[0];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(acc[p][i]));
-  asm volatile("" : "+v"(acc_x));
+    for (int p = 0; p < PBW; ++p)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(acc[p][i]));
+    asm volatile("" : "+v"(acc_x));
+  } else {
+    const f32x4 zero4 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int p = 0; p < PBW; ++p)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[p][i] = zero4;
+    acc_x = zero4;
+#pragma unroll
+    for (int p = 0; p < PBW; ++p)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(acc[p][i]));
+    asm volatile("" : "+v"(acc_x));
+  }
 
   // ring: taps 0 and 1 must have landed; the RING - 2 later taps may stay in flight
   if constexpr (RING != 0) {
@@ -278,16 +343,27 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
     if (ring_wave && taps >= RING) __builtin_amdgcn_s_waitcnt(0x0f70 | (fl & 15) | ((fl >> 4) << 14));
     else __builtin_amdgcn_s_waitcnt(0x0f70);
   } else {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+    // resident slab of nine taps: the patch and taps 0 to 2 must have landed (a wave's requests complete in
+    // order, the taps are the last nine operand requests); the other six are awaited at the end of tap 1, where
+    // the second barrier stands.  Any other number of taps: everything here.
+    if (prog) wait_taps(std::integral_constant<int, 6>{});
+    else __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
   }
-  if (sig < 0) {
-#pragma unroll
-    for (int i = 0; i < TPT; ++i) table[tid + i * NT] = tabg[i];
-  } else if (tid < 2 * BN) {
-    table[tid] = tabr;
+  if (!prog) {
+    publish_table(traw_now);
+    __syncthreads();
+  } else {
+    // (the bare barrier: the fence of __syncthreads would wait for the table requests, the last of the wave)
+    __builtin_amdgcn_s_barrier();
   }
-  __syncthreads();
 
+  if constexpr (RING == 0) {
+    if (!worker && prog) {  // (four multiplying waves) the other waves' share of the second barrier
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      publish_table(traw_late);
+      __syncthreads();
+    }
+  }
   if constexpr (RING != 0) {
     if (!worker) {
       // helper waves: taps t .. t + RING - 1 occupy the stages; before barrier t tap t + 2 has landed (the
@@ -319,15 +395,21 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
     };
     // operand addresses of "the tap whose first k-step was read last": one set, moved on to the next tap in
     // front of the read of its first k-step
-    const unsigned char *pp[NPF], *fp[4];
+    const unsigned char *pp[NPF], *fp[4], *fq[RING ? 1 : 4];  // (fq: resident slab, the tap's second k-step)
 #pragma unroll
     for (int i = 0; i < NPF; ++i) pp[i] = patch + a_base[i];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fp[i] = filt + f_base[i];
+    for (int i = 0; i < 4; ++i) {
+      fp[i] = filt + f_base[i];
+      if constexpr (RING == 0) fq[i] = filt + (f_base[i] ^ 64);
+    }
     auto read = [&](auto setc, auto kc) __attribute__((always_inline)) {
       constexpr int set = decltype(setc)::value, k = decltype(kc)::value;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) xb[set][i] = *(const u32x4 *)(fp[i] + k * 64);
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (RING == 0) xb[set][i] = *(const u32x4 *)(k == 0 ? fp[i] : fq[i]);
+        else xb[set][i] = *(const u32x4 *)(fp[i] + k * 64);
+      }
 #pragma unroll
       for (int i = 0; i < NPF; ++i) xa[set][i] = *(const u32x4 *)(pp[i] + k * 64);
     };
@@ -360,7 +442,10 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
           for (int i = 0; i < NPF; ++i) pp[i] = patch + a_base[i] + off;
           if constexpr (RING == 0) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) fp[i] += more ? TAPB : 0;
+            for (int i = 0; i < 4; ++i) {
+              fp[i] += more ? TAPS : 0;
+              fq[i] += more ? TAPS : 0;
+            }
           } else {
             const int st = more ? (t_now + 1) % RING : t_now % RING;
 #pragma unroll
@@ -373,6 +458,14 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
       if constexpr (RING != 0) {
         // barrier t: taps up to t + 2 are readable behind it (see the helper waves' loop)
         if (t_now + 2 < taps) __builtin_amdgcn_s_barrier();
+      } else if (prog) {
+        // (tap 1's last k-step was issued behind the read of tap 2's first: taps 0 to 2 stand behind the first
+        // barrier, the others behind this one)
+        if (t_now == 1) {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+          publish_table(traw_late);
+          __syncthreads();
+        }
       }
       t_now += 1;
     };

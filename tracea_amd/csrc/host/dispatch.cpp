@@ -1490,9 +1490,9 @@ bool plan_conv_wave16(const ConvGeometry &g, const ContractionVariant &v, bool w
   const long long pw = (long long)b.w_in + 2ll * g.pad_w;
   const long long ph = (long long)b.h_in + 2ll * g.pad_h;
   if (pw * ph >= (1ll << 30) || (long long)b.h_in * b.w_in >= (1ll << 24)) return false;
-  const int f_cpb = (g.k_gemm / 8) | 1;
+  // (pipeline 7: the slab of all taps of 64 filters, 128 bytes per filter and tap, no padding)
   const long long filter_bytes =
-      v.pipeline == 7 ? ((64ll * f_cpb + 511) / 512) * 512 * 16 : (long long)v.lds_bytes - TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
+      v.pipeline == 7 ? 64ll * g.k_gemm * 2 : (long long)v.lds_bytes - TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
   const long long table_bytes = TRACEA_MAX_EPILOGUE_OPS * 2 * 64 * 4;
   const int hw = b.h_out * b.w_out;
   const int grid_n = (g.n_gemm + v.bn - 1) / v.bn;
@@ -1540,7 +1540,7 @@ bool plan_conv_wave16(const ConvGeometry &g, const ContractionVariant &v, bool w
   a->p_seg = seg;
   a->p_ppi = ppi;
   magic_for_divisor((uint32_t)cpp, 64, &a->p_cpp_m, &a->p_cpp_s);
-  magic_for_divisor((uint32_t)f_cpb, (uint64_t)(64 * f_cpb + 512), &a->p_pw_m, &a->p_pw_s);  // filter rows of the resident slab
+  a->p_pw_m = 0; a->p_pw_s = 0;
   a->grid_m = b.batch * a->p_tiles;
   a->grid_n = grid_n;
   magic_for_divisor((uint32_t)grid_n, (uint64_t)a->grid_m * grid_n, &a->gn_m, &a->gn_s);
