@@ -395,19 +395,24 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
     };
     // operand addresses of "the tap whose first k-step was read last": one set, moved on to the next tap in
     // front of the read of its first k-step
-    const unsigned char *pp[NPF], *fp[4], *fq[RING ? 1 : 4];  // (fq: resident slab, the tap's second k-step)
+    // (fq: resident slab, the tap's second k-step, 64 bytes up or down from the first by the row's swizzle; kept
+    // beside fp where registers allow, else worked out per read -- the kernel with six pixel blocks per wave
+    // has none to spare)
+    constexpr bool FQ = RING == 0 && PBW <= 3;
+    const unsigned char *pp[NPF], *fp[4], *fq[FQ ? 4 : 1];
 #pragma unroll
     for (int i = 0; i < NPF; ++i) pp[i] = patch + a_base[i];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       fp[i] = filt + f_base[i];
-      if constexpr (RING == 0) fq[i] = filt + (f_base[i] ^ 64);
+      if constexpr (FQ) fq[i] = filt + (f_base[i] ^ 64);
     }
     auto read = [&](auto setc, auto kc) __attribute__((always_inline)) {
       constexpr int set = decltype(setc)::value, k = decltype(kc)::value;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        if constexpr (RING == 0) xb[set][i] = *(const u32x4 *)(k == 0 ? fp[i] : fq[i]);
+        if constexpr (FQ) xb[set][i] = *(const u32x4 *)(k == 0 ? fp[i] : fq[i]);
+        else if constexpr (RING == 0) xb[set][i] = *(const u32x4 *)(smem + ((unsigned)(fp[i] - smem) ^ (k * 64u)));
         else xb[set][i] = *(const u32x4 *)(fp[i] + k * 64);
       }
 #pragma unroll
@@ -444,7 +449,7 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
               fp[i] += more ? TAPS : 0;
-              fq[i] += more ? TAPS : 0;
+              if constexpr (FQ) fq[i] += more ? TAPS : 0;
             }
           } else {
             const int st = more ? (t_now + 1) % RING : t_now % RING;
