@@ -179,6 +179,41 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
       }
     }
   }
+  // ---- per-lane operand addresses (worked out between the requests for the patch and those for the filters:
+  // the requests queue in front of the memory pipe, and what a wave computes behind its last request is time it
+  // stands between the operands' arrival and the first MFMA) ----
+  __builtin_amdgcn_sched_barrier(0);
+  // pixel fragment i < PBW: block w*PBW + i; fragment PBW: the shared block 4*PBW
+  int a_base[NPF];
+#pragma unroll
+  for (int i = 0; i < NPF; ++i) {
+    const int blk = i < PBW ? ww * PBW + i : WK * PBW;
+    const int pr = blk * 16 + l15;
+    const int prc = pr < npix ? pr : npix - 1;
+    int ho, wo;
+    fast_divmod(p0 + prc, args.w_m, args.w_s, args.w_out, ho, wo);
+    a_base[i] = ((ho * args.stride_h - hp0) * PW + wo * args.stride_w) * pitch + q * 16;
+  }
+  // filter fragment i: filter block w ^ i (fragment 0 is the wave's own block, which the shared pixel block
+  // multiplies; fragments 2j and 2j+1 are neighbours in the channel order): row (w ^ i)*16 + l15, 16-byte part q
+  // (resident slab: the address of the tap's first k-step; the second one is 64 bytes up or down, by the row)
+  int f_base[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int row = (w ^ i) * 16 + l15;
+    f_base[i] = RING ? (row * CPB + q) * 16 : row * TAPB + ((q ^ ((row >> 1) & 7)) << 4);
+  }
+  int step_s = args.dil_w * pitch;
+  int step_r = tap_h * pitch - (args.s_sz - 1) * step_s;
+  int off_last = ((args.r_sz - 1) * tap_h + (args.s_sz - 1) * args.dil_w) * pitch;
+  int s_size = args.s_sz;
+#pragma unroll
+  for (int i = 0; i < NPF; ++i) asm volatile("" : "+v"(a_base[i]));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(f_base[i]));
+  asm volatile("" : "+s"(step_s), "+s"(step_r), "+s"(off_last), "+s"(s_size));
+  __builtin_amdgcn_sched_barrier(0);
+
   // (the patch first: every tap needs it; its rows come from memory, the filters from the L2 every workgroup shares)
   if constexpr (RING == 0) {
     const int row = tid >> 3, pos = tid & 7;
@@ -200,7 +235,7 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   }
 
   // ---- this thread's entry of the operand table (requested behind the operands, worked out where the table is
-  // published: in front of the first barrier, or -- prog -- of the third, when everything has landed anyway) ----
+  // published: in front of the first barrier, or -- prog -- of the second, when everything has landed anyway) ----
   // Waves 0 and 1 (threads 0..127: a of channel n0 + tid, b of channel n0 + tid - 64) request the raw vector
   // entries, every lane and the same number per wave, so that the waits for the taps can count them: 1 (bias,
   // scale and shift) or 4 (BatchNorm: gamma, variance, beta, mean).
@@ -271,37 +306,6 @@ __global__ void __launch_bounds__(CW_THREADS) conv_wave16_kernel(const Contracti
   // (Not with the taps awaited in groups: the accumulators would wait for the last request of the wave.)
   const bool bias_init = !prog && sig >= 0 && (sig & 1) && args.fe.aff_kind == TRACEA_EPI_OP_BIAS_ADD;
   const int form_sig = bias_init ? (sig & ~1) : sig;
-
-  // ---- per-lane operand addresses (worked out while the operands travel) ----
-  // pixel fragment i < PBW: block w*PBW + i; fragment PBW: the shared block 4*PBW
-  int a_base[NPF];
-#pragma unroll
-  for (int i = 0; i < NPF; ++i) {
-    const int blk = i < PBW ? ww * PBW + i : WK * PBW;
-    const int pr = blk * 16 + l15;
-    const int prc = pr < npix ? pr : npix - 1;
-    int ho, wo;
-    fast_divmod(p0 + prc, args.w_m, args.w_s, args.w_out, ho, wo);
-    a_base[i] = ((ho * args.stride_h - hp0) * PW + wo * args.stride_w) * pitch + q * 16;
-  }
-  // filter fragment i: filter block w ^ i (fragment 0 is the wave's own block, which the shared pixel block
-  // multiplies; fragments 2j and 2j+1 are neighbours in the channel order): row (w ^ i)*16 + l15, 16-byte part q
-  // (resident slab: the address of the tap's first k-step; the second one is 64 bytes up or down, by the row)
-  int f_base[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int row = (w ^ i) * 16 + l15;
-    f_base[i] = RING ? (row * CPB + q) * 16 : row * TAPB + ((q ^ ((row >> 1) & 7)) << 4);
-  }
-  int step_s = args.dil_w * pitch;
-  int step_r = tap_h * pitch - (args.s_sz - 1) * step_s;
-  int off_last = ((args.r_sz - 1) * tap_h + (args.s_sz - 1) * args.dil_w) * pitch;
-  int s_size = args.s_sz;
-#pragma unroll
-  for (int i = 0; i < NPF; ++i) asm volatile("" : "+v"(a_base[i]));
-#pragma unroll
-  for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(f_base[i]));
-  asm volatile("" : "+s"(step_s), "+s"(step_r), "+s"(off_last), "+s"(s_size));
 
   f32x4 acc[PBW][4], acc_x;
   if (bias_init) {  // (a branch of its own: the wait for these loads must not stand on the other road)
