@@ -1767,8 +1767,9 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
       if (cv.pipeline < 7 || cv.pipeline > 10) continue;
       ContractionArgs probe = a;
       // (the K-split members with tiles of one or two pixel blocks are for small launches: 14x14x256 at batch 1
-      // 6.4 us on 52 workgroups against 8.4 streamed and split along K; from 48 workgroups on)
-      const long long enough = cv.pipeline == 9 && cv.bm <= 32 ? 48 * 4 : device_limits().cus * 3;
+      // 6.4 us on 52 workgroups against 8.4 streamed and split along K; the stride-2 3x3 and 1x1 layers from
+      // 14x14x256 to 7x7x512 at batch 1, 32 workgroups, 6.5 and 3.8 us against 7.8 and 5.1; from 32 workgroups on)
+      const long long enough = cv.pipeline == 9 && cv.bm <= 32 ? 32 * 4 : device_limits().cus * 3;
       // (tile at least three quarters of the member's largest; the larger K-split members, whose waves all work
       // on every pixel block there is, from two fifths: 14x14x256 at batch 16, tiles of 49 of 112 pixels, 11.8 us
       // against 13.1 on the 32-pixel member)
