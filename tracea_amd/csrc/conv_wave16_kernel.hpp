@@ -15,16 +15,19 @@
 // PBW + 1 pixel fragments and 4 filter fragments of 1 KB per k-step for 4*PBW + 1 MFMAs of 16 cycles;
 // PBW = 6 is 0.44 KB of LDS reads per MFMA, PBW = 3 0.62.  Four more waves only move data; or (WK = 8) all
 // eight multiply, three blocks each: the two waves of a SIMD do not multiply faster than one (468 MFMAs in
-// 9.9 k cycles against 450 in 8.5 k), but the store phase is shared by twice the waves (11.3 us against 11.7
-// for N32 56x56 64->64).
+// 9.1 k cycles against 450 in 8.5 k: eight waves read 64 KB of fragments per k-step, more than LDS delivers in
+// the 416 cycles of their MFMAs), but the store phase is shared by twice the waves (10.7-11.3 us against
+// 11.3-11.9 for N32 56x56 64->64).
 //
 // A wave's pixels are consecutive, its results leave from registers (below), and nothing after the
 // operand wait is shared between the multiplying waves: each runs on its own.
 //
 // LDS layouts.  Patch: whole padded rows, pixel (hp, wp) at ((hp - hp0) * PW + wp) * cpp 16-byte chunks,
 // cpp = C/8 rounded up to odd, so that the 16 pixels of a fragment start in 16 different bank groups.
-// Filters, resident: row n at n * (K/8 | 1) chunks.  Filters, ring: stage t % RING holds tap t of the 64
-// filters, row n at n * (C/8 | 1) chunks.
+// Filters, resident (C = 64): tap t of the 64 filters at t * 8 KB, row n at n * 128 bytes, its 16-byte part p at
+// position p ^ ((n >> 1) & 7); requested tap by tap behind the patch, and a 3x3 layer starts multiplying when
+// the patch and taps 0 to 2 have landed (a second barrier, behind the other six, stands at the end of tap 1).
+// Filters, ring: stage t % RING holds tap t of the 64 filters, row n at n * (C/8 | 1) chunks.
 //
 // Epilogue.  The filter fragment is the first MFMA operand, so a lane ends with 4 consecutive output
 // channels (4q .. 4q+3 of a filter block, q = lane >> 4) of pixel lane & 15 of a pixel block.  For the
