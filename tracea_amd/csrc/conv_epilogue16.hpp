@@ -66,14 +66,23 @@ struct Epilogue16 {
   // 16-lane group q hold channels (q>>1)*8 .. +7 of block (q&1 ? fb : fa), one 16-byte store per lane.
   // ta/tb: the affine operands of the lane's four channels per block; prow: the pixel's row in the tile's
   // output (and residual) window, < 0 for a pixel outside the tile; row_c/row_r: row pitches in bytes.
-  static __device__ __forceinline__ void pair_block(f32x4 acc_a, f32x4 acc_b, int fa, int fb, f32x4 ta_a, f32x4 tb_a, f32x4 ta_b,
-                                                    f32x4 tb_b, int prow, int q, __amdgpu_buffer_rsrc_t rsrc_c,
-                                                    __amdgpu_buffer_rsrc_t rsrc_r, int row_c, int row_r) {
+  // pair_offset: the lane's byte offset into that window (output or residual alike, by the pitch).
+  static __device__ __forceinline__ int pair_offset(int fa, int fb, int prow, int q, int pitch) {
     const int ch = ((q & 1) ? fb : fa) * 16 + (q >> 1) * 8;
+    return prow >= 0 ? prow * pitch + ch * 2 : (int)OOB;
+  }
+  // (the residual's 16 bytes of the lane, as pair_block's store would write them; zeros without a residual
+  // buffer.  A kernel with registers to spare asks for them in front of its main loop and hands them to
+  // pair_block_with: fetched in the epilogue they are a round trip to memory with nothing left to hide it.)
+  static __device__ __forceinline__ u32x4 fetch_pair_residual(int fa, int fb, int prow, int q, __amdgpu_buffer_rsrc_t rsrc_r,
+                                                              int row_r) {
+    return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_r, pair_offset(fa, fb, prow, q, row_r), 0, 0));
+  }
+  static __device__ __forceinline__ void pair_block_with(f32x4 acc_a, f32x4 acc_b, int fa, int fb, f32x4 ta_a, f32x4 tb_a,
+                                                         f32x4 ta_b, f32x4 tb_b, int prow, int q, __amdgpu_buffer_rsrc_t rsrc_c,
+                                                         int row_c, u32x4 r8) {
     float ra[4] = {0, 0, 0, 0}, rb[4] = {0, 0, 0, 0};
     if constexpr (RES) {
-      const u32x4 r8 = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(
-                                                     rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
       unsigned r0 = r8[0], r1 = r8[1], r2 = r8[2], r3 = r8[3];
       asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
                    : "+v"(r0), "+v"(r1), "+v"(r2), "+v"(r3));
@@ -91,7 +100,14 @@ struct Epilogue16 {
     asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %2\n\tv_permlane16_swap_b32 %1, %3"
                  : "+v"(a_lo), "+v"(a_hi), "+v"(b_lo), "+v"(b_hi));
     const u32x4 row8 = {a_lo, a_hi, b_lo, b_hi};
-    __builtin_amdgcn_raw_buffer_store_b128(row8, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(row8, rsrc_c, pair_offset(fa, fb, prow, q, row_c), 0, 0);
+  }
+  static __device__ __forceinline__ void pair_block(f32x4 acc_a, f32x4 acc_b, int fa, int fb, f32x4 ta_a, f32x4 tb_a, f32x4 ta_b,
+                                                    f32x4 tb_b, int prow, int q, __amdgpu_buffer_rsrc_t rsrc_c,
+                                                    __amdgpu_buffer_rsrc_t rsrc_r, int row_c, int row_r) {
+    u32x4 r8 = {0u, 0u, 0u, 0u};
+    if constexpr (RES) r8 = fetch_pair_residual(fa, fb, prow, q, rsrc_r, row_r);
+    pair_block_with(acc_a, acc_b, fa, fb, ta_a, tb_a, ta_b, tb_b, prow, q, rsrc_c, row_c, r8);
   }
   // One pixel block x 64 filters: acc[i] the accumulators of filter block fb[i]; fb[2j] and fb[2j+1] share a store.
   static __device__ __forceinline__ void pixel_block(const f32x4 (&acc)[4], const int (&fb)[4], const f32x4 (&ta)[4],
@@ -102,20 +118,37 @@ struct Epilogue16 {
       pair_block(acc[2 * j], acc[2 * j + 1], fb[2 * j], fb[2 * j + 1], ta[2 * j], tb[2 * j], ta[2 * j + 1], tb[2 * j + 1], prow, q, rsrc_c,
                  rsrc_r, row_c, row_r);
   }
+  // (the same with the residual's two 16-byte pieces already in registers: res[j] = fetch_pair_residual of pair j)
+  static __device__ __forceinline__ void pixel_block_with(const f32x4 (&acc)[4], const int (&fb)[4], const f32x4 (&ta)[4],
+                                                          const f32x4 (&tb)[4], int prow, int q, __amdgpu_buffer_rsrc_t rsrc_c,
+                                                          int row_c, const u32x4 (&res)[2]) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      pair_block_with(acc[2 * j], acc[2 * j + 1], fb[2 * j], fb[2 * j + 1], ta[2 * j], tb[2 * j], ta[2 * j + 1], tb[2 * j + 1], prow, q,
+                      rsrc_c, row_c, res[j]);
+  }
   // One pixel block x one filter block (channels ch .. ch+3 of the lane): 8 bytes per lane.
-  static __device__ __forceinline__ void single_block(f32x4 acc, f32x4 ta, f32x4 tb, int ch, int prow,
-                                                      __amdgpu_buffer_rsrc_t rsrc_c, __amdgpu_buffer_rsrc_t rsrc_r, int row_c,
-                                                      int row_r) {
+  static __device__ __forceinline__ u32x2 fetch_single_residual(int ch, int prow, __amdgpu_buffer_rsrc_t rsrc_r, int row_r) {
+    return __builtin_bit_cast(u32x2,
+                              __builtin_amdgcn_raw_buffer_load_b64(rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
+  }
+  static __device__ __forceinline__ void single_block_with(f32x4 acc, f32x4 ta, f32x4 tb, int ch, int prow,
+                                                           __amdgpu_buffer_rsrc_t rsrc_c, int row_c, u32x2 r4) {
     float rr[4] = {0, 0, 0, 0};
     if constexpr (RES) {
-      const u32x2 r4 = __builtin_bit_cast(
-          u32x2, __builtin_amdgcn_raw_buffer_load_b64(rsrc_r, prow >= 0 ? prow * row_r + ch * 2 : (int)OOB, 0, 0));
       unpack2(r4[0], rr[0], rr[1]);
       unpack2(r4[1], rr[2], rr[3]);
     }
     const f32x4 v = finish(acc, ta, tb, rr);
     const u32x2 o = {pack2(v[0], v[1]), pack2(v[2], v[3])};
     __builtin_amdgcn_raw_buffer_store_b64(o, rsrc_c, prow >= 0 ? prow * row_c + ch * 2 : (int)OOB, 0, 0);
+  }
+  static __device__ __forceinline__ void single_block(f32x4 acc, f32x4 ta, f32x4 tb, int ch, int prow,
+                                                      __amdgpu_buffer_rsrc_t rsrc_c, __amdgpu_buffer_rsrc_t rsrc_r, int row_c,
+                                                      int row_r) {
+    u32x2 r4 = {0u, 0u};
+    if constexpr (RES) r4 = fetch_single_residual(ch, prow, rsrc_r, row_r);
+    single_block_with(acc, ta, tb, ch, prow, rsrc_c, row_c, r4);
   }
 };
 
