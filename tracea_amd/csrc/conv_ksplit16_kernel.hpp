@@ -247,6 +247,25 @@ __global__ void __launch_bounds__(CK_THREADS) conv_ksplit16_kernel(const Contrac
 #pragma unroll
       for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(acc[p][i]));
 
+    // ---- the residual of the pixel blocks this wave finishes (w, w + 4), asked for now: fetched in the epilogue
+    // it is a round trip to memory with nothing left to hide it ----
+    __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)((const unsigned short *)args.fe.res + ((sig >= 0 && (sig & 4)) ? m_img * args.fe.res_ld + n0 : 0ll)), 0,
+        (sig >= 0 && (sig & 4)) ? (int)((long long)npix * args.fe.res_ld * 2) : 0, 0x00020000);
+    const int row_r = (int)args.fe.res_ld * 2;
+    u32x4 resv[OWN][2] = {};
+    if (sig >= 0 && (sig & 4)) {
+      using E0 = Epilogue16<DT, 4>;
+#pragma unroll
+      for (int o = 0; o < OWN; ++o) {
+        const int p = w + 4 * o;
+        const int pr = p * 16 + l15;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          resv[o][j] = E0::fetch_pair_residual(2 * j, 2 * j + 1, (p < NPB && pr < npix) ? pr : -1, q, rsrc_r, row_r);
+      }
+    }
+
     // ---- main loop: one stage (this wave's 32 channels of it) per step, operands read one step ahead ----
     u32x4 xa[2][NPB], xb[2][4];
     int ts = 0, chunk = 0, s_now = 0;
@@ -357,10 +376,7 @@ __global__ void __launch_bounds__(CK_THREADS) conv_ksplit16_kernel(const Contrac
       // ---- epilogue from registers ----
       __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc(
           (void *)((unsigned short *)args.C + m_img * args.ldc + n0), 0, (int)((long long)npix * args.ldc * 2), 0x00020000);
-      __amdgpu_buffer_rsrc_t rsrc_r = __builtin_amdgcn_make_buffer_rsrc(
-          (void *)((const unsigned short *)args.fe.res + ((sig & 4) ? m_img * args.fe.res_ld + n0 : 0ll)), 0,
-          (sig & 4) ? (int)((long long)npix * args.fe.res_ld * 2) : 0, 0x00020000);
-      const int row_c = (int)args.ldc * 2, row_r = (int)args.fe.res_ld * 2;
+      const int row_c = (int)args.ldc * 2;
       const int fb[4] = {0, 1, 2, 3};
       auto run_form = [&](auto form) __attribute__((always_inline)) {
         using E = Epilogue16<DT, decltype(form)::value>;
@@ -376,7 +392,7 @@ __global__ void __launch_bounds__(CK_THREADS) conv_ksplit16_kernel(const Contrac
           constexpr int o = decltype(oc)::value;
           const int p = w + 4 * o;
           const int pr = p * 16 + l15;
-          E::pixel_block(fin[o], fb, ta, tb, (p < NPB && pr < npix) ? pr : -1, q, rsrc_c, rsrc_r, row_c, row_r);
+          E::pixel_block_with(fin[o], fb, ta, tb, (p < NPB && pr < npix) ? pr : -1, q, rsrc_c, row_c, resv[o]);
         });
       };
 #define TRACEA_CK_FORM(F) run_form(std::integral_constant<int, F>{})
