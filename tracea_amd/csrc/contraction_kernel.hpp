@@ -723,15 +723,20 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int TPT = (TAB_ENTRIES + NT - 1) / NT;
   // (An empty chain branches round all of it: the entries are some 1600 instructions with scalar loads
   // between them, 4000 cycles in front of the first tile request of a launch that needs none of them.)
+  // (With direct-to-LDS tile loads the entries are worked out behind the first tile requests instead of in front
+  // of them: the requests need nothing of this, and their round trip to memory covers it.)
   float tabr[TPT];
 #pragma unroll
   for (int i = 0; i < TPT; ++i) tabr[i] = 0.0f;
-  if (plan.n_ops > 0) {
-#pragma unroll
-    for (int i = 0; i < TPT; ++i) {
-      const int idx = tid + i * NT;
-      tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;
-    }
+#define TRACEA_REQUEST_TABLE()                                                                                                  \
+  if (plan.n_ops > 0) {                                                                                                         \
+    _Pragma("unroll") for (int i = 0; i < TPT; ++i) {                                                                           \
+      const int idx = tid + i * NT;                                                                                             \
+      tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;       \
+    }                                                                                                                           \
+  }
+  if constexpr (PIPE != 2) {
+    TRACEA_REQUEST_TABLE()
   }
 
   // Every load is issued unconditionally from an address that is always
@@ -1229,6 +1234,8 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     constexpr int CUT1 = MS == 16 ? (L * 3) / 4 : L / SPREAD, CUT2 = SPREAD == 3 ? 2 * L / SPREAD : L;
     dma(smem, smem + A_STAGE, 0, 0, L);
     dma(smem + STAGE, smem + STAGE + A_STAGE, nk > 1 ? BK : 0, 0, CUT1);  // first share of tile 1
+    TRACEA_REQUEST_TABLE()
+#undef TRACEA_REQUEST_TABLE
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile 0 is in LDS
     __syncthreads();
     read_operands(0, smem, smem + A_STAGE, 0);
