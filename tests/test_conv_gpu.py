@@ -56,7 +56,7 @@ SMALL = [  # n, h, w, c, k, r, s, stride, pad, dilation
 ]
 
 
-@pytest.mark.parametrize("variant", range(32))
+@pytest.mark.parametrize("variant", range(40))
 def test_small_shapes_every_variant_both_filter_layouts(tracea_gpu, variant):
     from tracea_amd import capi
     names = capi.variants("conv2d")

@@ -66,7 +66,7 @@ def test_reference_known_answer_16cubed_f16(tracea_gpu):
 HALF_SHAPES = [(256, 256, 128), (300, 200, 136), (512, 384, 1024), (64, 72, 8), (1000, 24, 72)]
 
 
-@pytest.mark.parametrize("variant", range(32))
+@pytest.mark.parametrize("variant", range(40))
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_half_every_variant_both_b_layouts(tracea_gpu, variant, dtype):
     from tracea_amd import capi
