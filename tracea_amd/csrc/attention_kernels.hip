@@ -514,7 +514,8 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     last_key[qi] = (a.causal && q_mine[qi] < S - 1 ? q_mine[qi] : S - 1) - g * 4;
   }
   wave_last_key = a.causal && q0 + (wave_u + 1) * WQ - 1 < S - 1 ? q0 + (wave_u + 1) * WQ - 1 : S - 1;
-  load_q(q0, qf, std::integral_constant<int, KS>{});
+  // (the queries are fetched behind the first tile requests, below: the scaling of a fragment waits for its load,
+  // and in front of the requests that wait was a round trip to memory of its own at the start of every workgroup)
 
   auto k_piece = [&](int row, int c) __attribute__((always_inline)) -> int {
     return row * ROW_BYTES + ((c ^ ((row / RP) & (CH - 1))) << 4);
@@ -612,6 +613,8 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     load_v(1, sVbase + TILE_BYTES);
     load_k(2, sKbase + 2 * TILE_BYTES);
   }
+  __builtin_amdgcn_sched_barrier(0);
+  load_q(q0, qf, std::integral_constant<int, KS>{});
   // The second item's queries travel with the first tiles.  PARK: the upper half of their k-steps waits in LDS
   // behind the rings (fetched there directly, each lane's fragment in a slot of its own) instead of in
   // registers: the 16 registers that the -m block of SHIFT needs at head dimension 128.
