@@ -723,8 +723,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
   constexpr int TPT = (TAB_ENTRIES + NT - 1) / NT;
   // (An empty chain branches round all of it: the entries are some 1600 instructions with scalar loads
   // between them, 4000 cycles in front of the first tile request of a launch that needs none of them.)
-  // (With direct-to-LDS tile loads the entries are worked out behind the first tile requests instead of in front
-  // of them: the requests need nothing of this, and their round trip to memory covers it.)
+  // (The convolutions with direct-to-LDS tile loads work the entries out behind the first tile requests instead of
+  // in front of them: the requests need nothing of this, and their round trip to memory covers it.  Not the GEMMs:
+  // with the code in that place the 256x256 kernel of the 4096^3 product took 125 us instead of 101, empty chain
+  // and all.)
   float tabr[TPT];
 #pragma unroll
   for (int i = 0; i < TPT; ++i) tabr[i] = 0.0f;
@@ -735,7 +737,7 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
       tabr[i] = idx < TAB_ENTRIES ? chain_table_value(args.epi, idx / (2 * BN), (idx / BN) & 1, n0 + idx % BN, N) : 0.0f;       \
     }                                                                                                                           \
   }
-  if constexpr (PIPE != 2) {
+  if constexpr (PIPE != 2 || !CONV) {
     TRACEA_REQUEST_TABLE()
   }
 
@@ -1234,7 +1236,9 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
     constexpr int CUT1 = MS == 16 ? (L * 3) / 4 : L / SPREAD, CUT2 = SPREAD == 3 ? 2 * L / SPREAD : L;
     dma(smem, smem + A_STAGE, 0, 0, L);
     dma(smem + STAGE, smem + STAGE + A_STAGE, nk > 1 ? BK : 0, 0, CUT1);  // first share of tile 1
-    TRACEA_REQUEST_TABLE()
+    if constexpr (CONV) {
+      TRACEA_REQUEST_TABLE()
+    }
 #undef TRACEA_REQUEST_TABLE
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's share of tile 0 is in LDS
     __syncthreads();
