@@ -308,3 +308,33 @@ def test_operand_beyond_2gib_takes_the_register_staged_kernels(tracea_gpu, dtype
     # the same product from a compact copy of A runs the direct-to-LDS kernels and agrees
     compact = tracea_gpu.gemm(a_view.contiguous(), _dev(b, tdt), bias=_dev(bias), epilogue="bias+relu").float().cpu().numpy()
     np.testing.assert_allclose(got, compact, rtol=0, atol=2e-3 if dtype == "f16" else 1e-5)
+
+
+@pytest.mark.parametrize("shape", [(1000, 900, 1030), (129, 257, 203), (5, 3, 7), (300, 1001, 130), (1, 1, 1), (513, 130, 31)])
+def test_ragged_sizes_and_strided_operands_run_from_padded_copies(tracea_gpu, shape):
+    """A K or N that is not a whole number of 16-byte pieces, and operands strided along K: copied into padded rows
+    and multiplied by the tile kernels (the any-layout kernel on the vector ALU remains for what cannot be copied).
+    fp32 and both half types, B row-major and column-major, a column-major A, with a chain and with fp32 output."""
+    from tracea_amd import capi
+    m, n, k = shape
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a = (rng.standard_normal((m, k)) / np.sqrt(k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    ref = np.maximum(oracle.gemm_f64(a, b) + bias[None, :], 0.0)
+    da, db, dbias = _dev(a), _dev(b), _dev(bias)
+    for tag, xa, xb in (("row-major B", da, db), ("column-major B", da, db.t().contiguous().t()),
+                        ("column-major A", da.t().contiguous().t(), db)):
+        got = tracea_gpu.gemm(xa, xb, bias=dbias, epilogue="bias+relu").cpu().numpy()
+        assert np.abs(got - ref).max() <= 1e-4 * max(1.0, np.abs(ref).max()), "f32 " + tag
+    for dtype, tdt, rnd in (("f16", torch.float16, round_f16), ("bf16", torch.bfloat16, round_bf16)):
+        ha, hb = rnd(a), rnd(b)
+        ref16 = oracle.gemm_f64(ha, hb)
+        want = np.maximum(ref16 + bias[None, :], 0.0)
+        xa, xb = _dev(ha, tdt), _dev(hb, tdt)
+        for tag, yb in (("row-major B", xb), ("column-major B", xb.t().contiguous().t())):
+            got = tracea_gpu.gemm(xa, yb, bias=dbias, epilogue="bias+relu").float().cpu().numpy()
+            assert capi.last_variant("gemm") is not None, "the tile kernels did not run"
+            assert_close_scaled(got, want, tol_half(k, dtype), "%s %s" % (dtype, tag))
+        got = tracea_gpu.gemm(xa, xb, out_dtype=torch.float32).cpu().numpy()
+        assert np.abs(got - ref16).max() <= 1e-4 * max(1.0, np.abs(ref16).max()), dtype + " with fp32 output"

@@ -623,6 +623,31 @@ void *splitk_scratch(int device, hipStream_t stream, size_t bytes) {
   return p;
 }
 
+// Buffer of the padded operand copies (run_gemm), per (device, stream) like the split-K workspace and by the same
+// rules: grows on demand up to a cap, never while its stream is being captured, never freed.
+constexpr size_t kPadScratchCap = 1u << 30;
+std::map<std::pair<int, void *>, std::pair<void *, size_t>> g_pad_scratch;
+void *pad_scratch(int device, hipStream_t stream, size_t bytes) {
+  if (bytes > kPadScratchCap) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  auto &slot = g_pad_scratch[{device, (void *)stream}];
+  if (slot.second >= bytes) return slot.first;
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  size_t want = 1u << 20;
+  while (want < bytes) want <<= 1;
+  void *p = nullptr;
+  if (hipMalloc(&p, want) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  slot = {p, want};
+  return p;
+}
+
 // Ticket counters of the one-launch split, one per tile, kept per (device, stream) like the scratch
 // buffer: zero when allocated, and every launch leaves them at zero again.  Null while the stream is
 // being captured and the counters do not exist yet.
@@ -776,8 +801,12 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     }
   }
   if (a.dtype == TRACEA_DTYPE_FLOAT32 && b.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32 && K > 0 &&
-      a.stride[1] == 1 && b.stride[1] == 1 && c.stride[1] == 1 && K % 4 == 0 && N % 4 == 0 &&
+      a.stride[1] == 1 && b.stride[1] == 1 && c.stride[1] == 1 && K % 4 == 0 &&
+      (N % 4 == 0 || ((K - 1) * b.stride[0] + N) * 4 < (1ll << 31)) &&
       a.stride[0] % 4 == 0 && b.stride[0] % 4 == 0 && aligned(a.ptr, 16) && aligned(b.ptr, 16)) {
+    // (N itself may be ragged where B is read through a buffer descriptor, i.e. below 2 GiB: a piece that starts
+    // inside N is read whole -- what lies behind N in the row only reaches output columns that are never stored,
+    // and behind the last row the descriptor returns zeros -- and the epilogue stores by valid channels)
     ContractionArgs args{};
     args.A = a.ptr; args.B = b.ptr; args.C = c.ptr;
     args.M = (int)M; args.N = (int)N; args.K = (int)K;
@@ -859,6 +888,41 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     if (st != TRACEA_SUCCESS) return st;
     t_last_split_launches = 2;
     return hip_status("split-K reduction launch", launch_splitk_reduce(r, stream));
+  }
+  // Operands the tile kernels cannot read as they lie -- a K (or the N of a row-major B) that is not a whole
+  // number of 16-byte pieces, rows that do not start on 16 bytes, strides along K -- are copied once into
+  // padded, zero-filled rows and multiplied from there: two copy launches in front of a tile kernel instead of
+  // the any-layout kernel on the vector ALU (fp32 1000 x 900 x 1030: 794 us there).  Half precision: both as
+  // K-contiguous rows (a row-major B is transposed on the way); fp32: A by rows, B row-major.  Not for the entry
+  // point that must not allocate, nor while the buffer cannot grow (a stream under capture).
+  static thread_local bool in_padded = false;
+  const bool same_half = is_half(a.dtype) && b.dtype == a.dtype;
+  const bool all_f32 = a.dtype == TRACEA_DTYPE_FLOAT32 && b.dtype == TRACEA_DTYPE_FLOAT32 && c.dtype == TRACEA_DTYPE_FLOAT32;
+  if (!in_padded && !static_only && K > 0 && (same_half || all_f32) && c.stride[1] == 1 && M < (1ll << 31) && N < (1ll << 31) &&
+      K < (1ll << 31)) {
+    const int esz = same_half ? 2 : 4;
+    const long long Kp = (K + 31) / 32 * 32, Np = (N + 31) / 32 * 32;
+    const size_t a_bytes = (size_t)M * (size_t)Kp * esz;
+    const size_t b_bytes = same_half ? (size_t)N * (size_t)Kp * esz : (size_t)Kp * (size_t)Np * esz;
+    const size_t a_room = (a_bytes + 255) / 256 * 256;
+    unsigned char *buf = (unsigned char *)pad_scratch(c.device, stream, a_room + b_bytes);
+    if (buf != nullptr) {
+      int e = launch_pad_copy(a.ptr, buf, esz, M, K, a.stride[0], a.stride[1], M, Kp, stream);
+      if (e == 0) {
+        if (same_half) e = launch_pad_copy(b.ptr, buf + a_room, esz, N, K, b.stride[1], b.stride[0], N, Kp, stream);
+        else e = launch_pad_copy(b.ptr, buf + a_room, esz, K, N, b.stride[0], b.stride[1], Kp, Np, stream);
+      }
+      if (e != 0) return hip_status("operand copy launch", e);
+      View ap = a, bp = b;
+      ap.ptr = buf; ap.shape[1] = Kp; ap.stride[0] = Kp; ap.stride[1] = 1;
+      bp.ptr = buf + a_room; bp.shape[0] = Kp;
+      if (same_half) { bp.stride[0] = 1; bp.stride[1] = Kp; }
+      else { bp.stride[0] = Np; bp.stride[1] = 1; }
+      in_padded = true;
+      const TraceaStatus st = run_gemm(ap, bp, c, chain, stream, static_only);
+      in_padded = false;
+      return st;
+    }
   }
   GenericGemmArgs g{};
   g.A = a.ptr; g.B = b.ptr; g.C = c.ptr;

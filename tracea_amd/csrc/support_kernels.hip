@@ -448,6 +448,30 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(const GenericGemmArgs
   store_from_float<1>(a.C, a.c_dtype, (long long)m * a.scm + (long long)n * a.scn, 1, v);
 }
 
+template <typename T>
+__global__ void __launch_bounds__(256) pad_copy_kernel(const T *src, T *dst, long long rows_src, long long cols_src, long long rs,
+                                                       long long cs, long long pitch, long long total) {
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total) return;
+  const long long r = idx / pitch, c = idx - r * pitch;
+  dst[idx] = (r < rows_src && c < cols_src) ? src[r * rs + c * cs] : T(0);
+}
+
+int launch_pad_copy(const void *src, void *dst, int elt_bytes, long long rows_src, long long cols_src, long long rs,
+                    long long cs, long long rows_dst, long long pitch, hipStream_t stream) {
+  const long long total = rows_dst * pitch;
+  if (total <= 0) return 0;
+  const long long blocks = (total + 255) / 256;
+  if (blocks >= (1ll << 31) || (elt_bytes != 2 && elt_bytes != 4)) return (int)hipErrorInvalidValue;
+  if (elt_bytes == 2)
+    hipLaunchKernelGGL(pad_copy_kernel<unsigned short>, dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned short *)src,
+                       (unsigned short *)dst, rows_src, cols_src, rs, cs, pitch, total);
+  else
+    hipLaunchKernelGGL(pad_copy_kernel<unsigned>, dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned *)src, (unsigned *)dst,
+                       rows_src, cols_src, rs, cs, pitch, total);
+  return (int)hipGetLastError();
+}
+
 int launch_gemm_generic(const GenericGemmArgs &a, hipStream_t stream) {
   const dim3 grid((unsigned)((a.N + 15) / 16), (unsigned)((a.M + 15) / 16));
   hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, stream, a);
