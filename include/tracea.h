@@ -309,6 +309,13 @@ TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaT
  * tracea_last_split_k_launches says which
  * form the calling thread's latest gemm / conv2d launch took (1 or 2).  (The reference has no split along K:
  * its GEMM grid is one block per output tile, src/emitter/cuda/gemm.rs:92-207.) */
+/* Operands of tracea_gemm / tracea_gemm_ex that the tile kernels cannot read in place -- a K, or the N of a
+ * row-major B, that is not a whole number of 16-byte pieces; rows that do not start on 16 bytes; an A strided
+ * along K -- are copied into padded, zero-filled rows of a second per-(device, stream) buffer (at most 1 GiB,
+ * same rules as the one above) and multiplied from there.  Where that buffer cannot be had
+ * (tracea_gemm_noalloc, a stream under capture that made no such call before, A and B of different types) a
+ * kernel on the vector ALU that reads any layout runs instead: same results, far slower.  (The reference's
+ * kernels take M, N, K as they come: src/emitter/cuda/gemm.rs:92-207 guards every element.) */
 void tracea_set_split_k(int32_t enabled);
 void tracea_set_split_k_one_launch(int32_t enabled);
 int32_t tracea_last_split_k_launches(void);
