@@ -539,8 +539,44 @@ def test_error_paths(tracea_gpu):
     assert call(x.permute(0, 3, 1, 2).contiguous().permute(0, 2, 3, 1), w, out) == capi.UNSUPPORTED_CONFIG  # NCHW storage
     x12 = torch.zeros(1, 8, 8, 12, device="cuda", dtype=torch.float16)
     w12 = torch.zeros(8, 3, 3, 12, device="cuda", dtype=torch.float16)
-    assert call(x12, w12, out) == capi.UNSUPPORTED_CONFIG             # C % 8 != 0
-    assert "multiple of 8" in capi.last_error()
+    assert call(x12, w12, out) == capi.SUCCESS                        # C % 8 != 0: from padded copies (next test)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_channels_that_are_no_multiple_of_8_run_from_padded_copies(tracea_gpu, dtype):
+    """An RGB first layer (3 channels, 7x7 stride 2), 12 channels, [R,S,C,K] filters with a ragged K, operands that do
+    not start on 16 bytes: copied with the channels padded to 8 and run by the tile kernels; the reference's kernel
+    reads such channels element by element (src/emitter/cuda/conv.rs:228-240)."""
+    from tracea_amd import capi
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    rnd = round_f16 if dtype == "f16" else round_bf16
+    cases = [(2, 40, 36, 3, 64, 7, 7, 2, 3, "krsc"), (3, 9, 11, 12, 20, 3, 3, 1, 1, "krsc"), (1, 10, 10, 5, 13, 3, 1, 1, 0, "rsck"),
+             (2, 8, 8, 16, 12, 3, 3, 1, 1, "rsck"), (1, 6, 7, 1, 8, 1, 1, 1, 0, "krsc")]
+    for (n, h, w, c, k, r, s, stride, pad, layout) in cases:
+        rng = np.random.default_rng(n + 10 * c + k)
+        x = rnd(rng.standard_normal((n, h, w, c)))
+        w_rsck = rnd(rng.standard_normal((r, s, c, k)) * np.sqrt(2.0 / (r * s * c)))
+        bias = (rng.standard_normal(k) * 0.1).astype(np.float32)
+        want = oracle.epilogue_apply(oracle.conv2d_nhwc(x, w_rsck, stride, pad, 1), [(oracle.EPI_BIAS_ADD, bias), (oracle.EPI_RELU,)])
+        dx = _dev(x, tdt)
+        dw = _dev(w_rsck, tdt)
+        if layout == "krsc":
+            dw = dw.permute(3, 0, 1, 2).contiguous()
+        y = tracea_gpu.conv2d(dx, dw, bias=_dev(bias), stride=stride, padding=pad, epilogue="bias+relu",
+                              weight_layout=layout)
+        assert_close_scaled(y.float().cpu().numpy(), want, tol_for_k(r * s * c) if dtype == "f16" else tol_half(r * s * c, "bf16"),
+                            "%s %s" % (dtype, (n, h, w, c, k, r, s, stride, pad, layout)))
+    # an activation tensor that does not start on 16 bytes
+    n, h, w, c, k = 1, 9, 9, 16, 8
+    rng = np.random.default_rng(5)
+    x = rnd(rng.standard_normal((n, h, w, c)))
+    w_rsck = rnd(rng.standard_normal((3, 3, c, k)) * np.sqrt(2.0 / (9 * c)))
+    buf = torch.zeros(n * h * w * c + 1, device="cuda", dtype=tdt)
+    xv = buf[1:].view(n, h, w, c)
+    xv.copy_(_dev(x, tdt))
+    y = tracea_gpu.conv2d(xv, _dev(w_rsck, tdt).permute(3, 0, 1, 2).contiguous(), stride=1, padding=1)
+    assert_close_scaled(y.float().cpu().numpy(), oracle.conv2d_nhwc(x, w_rsck, 1, 1, 1),
+                        tol_for_k(9 * c) if dtype == "f16" else tol_half(9 * c, "bf16"), "unaligned x")
 
 
 @pytest.mark.parametrize("seed", [11, 12])

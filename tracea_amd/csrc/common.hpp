@@ -138,11 +138,12 @@ struct GenericGemmArgs {
   EpilogueChain epi;
 };
 int launch_gemm_generic(const GenericGemmArgs &args, hipStream_t stream);
-// dst[r][c] (rows_dst rows of `pitch` elements of elt_bytes = 2 or 4) = src[r * rs + c * cs] for r < rows_src and
-// c < cols_src, zero elsewhere: an operand as the tile kernels can read it (rows on 16 bytes, a whole number of
-// 16-byte pieces, zeros behind the data), from any two strides.
+// dst[r][c] (rows_dst rows of `pitch` elements of elt_bytes = 2 or 4) = src[(r / n1) * rs + (r % n1) * s1 + c * cs]
+// for r < rows_src and c < cols_src, zero elsewhere: an operand as the tile kernels can read it (rows on 16
+// bytes, a whole number of 16-byte pieces, zeros behind the data), from any two strides (n1 = 1) or, with the
+// rows in two levels, three.
 int launch_pad_copy(const void *src, void *dst, int elt_bytes, long long rows_src, long long cols_src, long long rs,
-                    long long cs, long long rows_dst, long long pitch, hipStream_t stream);
+                    long long cs, long long rows_dst, long long pitch, hipStream_t stream, long long n1 = 1, long long s1 = 0);
 
 // Second stage of a split-K contraction: out[m, n] = chain(sum over z of partial[z][m][n]).
 struct SplitKReduceArgs {

@@ -1340,6 +1340,7 @@ struct ConvPlan {
   ConvGeometry geo;
   bool w_ncontig;  // filters stored [R,S,C,K]
   long long ldb, ldc;
+  bool pad_c = false;  // channels not a multiple of 8, or operands not on 16 bytes: run from padded copies
 };
 
 TraceaStatus conv_common(const TraceaTensorView &tx, const TraceaTensorView &tw,
@@ -1398,14 +1399,10 @@ TraceaStatus conv_common(const TraceaTensorView &tx, const TraceaTensorView &tw,
         out.stride[0] == (long long)g.block.h_out * g.block.w_out * ldc))
     return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: output must be channel-contiguous NHWK");
   plan->ldc = ldc;
-  if (C % 8 != 0)
-    return fail(TRACEA_UNSUPPORTED_CONFIG,
-                "tracea_conv2d: input channels (%lld) must be a multiple of 8 for 16-byte loads", C);
-  if (plan->w_ncontig && K % 8 != 0)
-    return fail(TRACEA_UNSUPPORTED_CONFIG,
-                "tracea_conv2d: [R,S,C,K] filters need output channels (%lld) to be a multiple of 8", K);
-  if (!aligned(x.ptr, 16) || !aligned(w.ptr, 16))
-    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_conv2d: x and w must be 16-byte aligned");
+  // (what the kernels cannot read in place runs from padded copies where a buffer for them can be had: see
+  // run_conv_padded; these messages are what the caller reads where it cannot)
+  plan->pad_c = false;
+  if (C % 8 != 0 || (plan->w_ncontig && K % 8 != 0) || !aligned(x.ptr, 16) || !aligned(w.ptr, 16)) plan->pad_c = true;
   return TRACEA_SUCCESS;
 }
 
@@ -1920,6 +1917,45 @@ TraceaStatus run_conv(const ConvPlan &plan, const EpilogueChain &chain, hipStrea
   return launch_maybe_split("conv2d launch", v, a, chain, true, plan.x.dtype, plan.w_ncontig, plan.out.device, stream);
 }
 
+// A convolution whose operands the kernels cannot read in place -- input channels that are not a multiple of 8
+// (an RGB first layer), [R,S,C,K] filters with a ragged K, operands that do not start on 16 bytes -- runs from
+// copies with the channels padded to a multiple of 8 with zeros (they add nothing to any sum), activations
+// NHWC and filters [K,R,S,C], in the per-(device, stream) buffer of run_gemm's padded operands.  (The
+// reference's kernel reads such channels element by element: src/emitter/cuda/conv.rs:228-240.)
+TraceaStatus run_conv_maybe_padded(const ConvPlan &plan, const TraceaTensorView *tout_c, const TraceaConv2dParams &params,
+                                   const EpilogueChain &chain, hipStream_t stream) {
+  if (!plan.pad_c) return run_conv(plan, chain, stream);
+  const View &x = plan.x, &w = plan.w;
+  const long long N = x.shape[0], H = x.shape[1], W = x.shape[2], C = x.shape[3];
+  const long long K = w.shape[0], R = w.shape[1], S = w.shape[2];
+  const long long Cp = (C + 7) / 8 * 8;
+  const size_t x_bytes = (size_t)(N * H * W) * (size_t)Cp * 2, w_bytes = (size_t)(K * R * S) * (size_t)Cp * 2;
+  const size_t x_room = (x_bytes + 255) / 256 * 256;
+  DeviceScope scope(plan.out.device);
+  if (scope.err != hipSuccess) return hip_status("hipSetDevice", (int)scope.err);
+  unsigned char *buf = (unsigned char *)pad_scratch(plan.out.device, stream, x_room + w_bytes);
+  if (buf == nullptr)
+    return fail(TRACEA_UNSUPPORTED_CONFIG,
+                "tracea_conv2d: input channels (%lld) must be a multiple of 8 ([R,S,C,K] filters: output channels too) and x, "
+                "w 16-byte aligned where no buffer for padded copies can be had (stream under capture, or above 1 GiB)", C);
+  int e = launch_pad_copy(x.ptr, buf, 2, N * H * W, C, C, 1, N * H * W, Cp, stream);
+  if (e == 0) {
+    if (!plan.w_ncontig) e = launch_pad_copy(w.ptr, buf + x_room, 2, K * R * S, C, C, 1, K * R * S, Cp, stream);
+    else e = launch_pad_copy(w.ptr, buf + x_room, 2, K * R * S, C, 1, K, K * R * S, Cp, stream, R * S, C * K);
+  }
+  if (e != 0) return hip_status("operand copy launch", e);
+  const uint64_t xs[4] = {(uint64_t)N, (uint64_t)H, (uint64_t)W, (uint64_t)Cp}, ws[4] = {(uint64_t)K, (uint64_t)R, (uint64_t)S, (uint64_t)Cp};
+  TraceaTensorView tx{}, tw{};
+  tx.ptr = buf; tx.rank = 4; tx.shape = xs; tx.stride = nullptr; tx.dtype = (TraceaDType)x.dtype; tx.device_id = x.device;
+  tw.ptr = buf + x_room; tw.rank = 4; tw.shape = ws; tw.stride = nullptr; tw.dtype = (TraceaDType)w.dtype; tw.device_id = w.device;
+  TraceaTensorView tout = *tout_c;
+  ConvPlan padded;
+  const TraceaStatus st = conv_common(tx, tw, &tout, params, &padded);
+  if (st != TRACEA_SUCCESS) return st;
+  if (padded.pad_c) return fail(TRACEA_UNKNOWN_ERROR, "tracea_conv2d: padded operands still not readable");
+  return run_conv(padded, chain, stream);
+}
+
 }  // namespace
 
 TraceaStatus dispatch_conv2d_kind(const TraceaTensorView &tx, const TraceaTensorView &tw,
@@ -1937,7 +1973,7 @@ TraceaStatus dispatch_conv2d_kind(const TraceaTensorView &tx, const TraceaTensor
   EpilogueChain chain{};
   st = lower_chain("tracea_conv2d", ops, (uint32_t)n, plan.out.shape[3], plan.out.shape[3], &chain);
   if (st != TRACEA_SUCCESS) return st;
-  return run_conv(plan, chain, (hipStream_t)params.stream);
+  return run_conv_maybe_padded(plan, tout, params, chain, (hipStream_t)params.stream);
 }
 
 TraceaStatus dispatch_conv2d_ops(const TraceaTensorView &tx, const TraceaTensorView &tw,
@@ -1949,7 +1985,7 @@ TraceaStatus dispatch_conv2d_ops(const TraceaTensorView &tx, const TraceaTensorV
   EpilogueChain chain{};
   st = lower_chain("tracea_conv2d_ex", ops, n_ops, plan.out.shape[3], plan.out.shape[3], &chain);
   if (st != TRACEA_SUCCESS) return st;
-  return run_conv(plan, chain, (hipStream_t)params.stream);
+  return run_conv_maybe_padded(plan, tout, params, chain, (hipStream_t)params.stream);
 }
 
 // ---- ConvTranspose2d ---------------------------------------------------------------

@@ -450,25 +450,26 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(const GenericGemmArgs
 
 template <typename T>
 __global__ void __launch_bounds__(256) pad_copy_kernel(const T *src, T *dst, long long rows_src, long long cols_src, long long rs,
-                                                       long long cs, long long pitch, long long total) {
+                                                       long long cs, long long n1, long long s1, long long pitch, long long total) {
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
   const long long r = idx / pitch, c = idx - r * pitch;
-  dst[idx] = (r < rows_src && c < cols_src) ? src[r * rs + c * cs] : T(0);
+  const long long r0 = r / n1, r1 = r - r0 * n1;
+  dst[idx] = (r < rows_src && c < cols_src) ? src[r0 * rs + r1 * s1 + c * cs] : T(0);
 }
 
 int launch_pad_copy(const void *src, void *dst, int elt_bytes, long long rows_src, long long cols_src, long long rs,
-                    long long cs, long long rows_dst, long long pitch, hipStream_t stream) {
+                    long long cs, long long rows_dst, long long pitch, hipStream_t stream, long long n1, long long s1) {
   const long long total = rows_dst * pitch;
   if (total <= 0) return 0;
   const long long blocks = (total + 255) / 256;
-  if (blocks >= (1ll << 31) || (elt_bytes != 2 && elt_bytes != 4)) return (int)hipErrorInvalidValue;
+  if (blocks >= (1ll << 31) || (elt_bytes != 2 && elt_bytes != 4) || n1 < 1) return (int)hipErrorInvalidValue;
   if (elt_bytes == 2)
     hipLaunchKernelGGL(pad_copy_kernel<unsigned short>, dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned short *)src,
-                       (unsigned short *)dst, rows_src, cols_src, rs, cs, pitch, total);
+                       (unsigned short *)dst, rows_src, cols_src, rs, cs, n1, s1, pitch, total);
   else
     hipLaunchKernelGGL(pad_copy_kernel<unsigned>, dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned *)src, (unsigned *)dst,
-                       rows_src, cols_src, rs, cs, pitch, total);
+                       rows_src, cols_src, rs, cs, n1, s1, pitch, total);
   return (int)hipGetLastError();
 }
 

@@ -123,13 +123,13 @@ class TraceaConv2d(torch.nn.Conv2d):
     """Drop-in replacement for torch.nn.Conv2d (tracea-python/python/tracea/__init__.py:29-56):
     NCHW in, NCHW out.  groups != 1, dilation != (1,1), a padding mode other than "zeros" fall back
     to PyTorch as in the reference; so does what the convolution kernels here do not take: tensors
-    off the GPU, dtypes other than f16 / bf16, input channels not a multiple of 8, string padding."""
+    off the GPU, dtypes other than f16 / bf16, string padding.  (Input channels that are not a multiple of 8,
+    an RGB first layer, run from copies padded to 8 inside the library.)"""
 
     def _tracea_supported(self, x):
         return (self.groups == 1 and self.dilation == (1, 1) and self.padding_mode == "zeros"
                 and not isinstance(self.padding, str) and x.is_cuda and x.dim() == 4
-                and x.dtype in (torch.float16, torch.bfloat16) and self.weight.dtype == x.dtype
-                and self.in_channels % 8 == 0)
+                and x.dtype in (torch.float16, torch.bfloat16) and self.weight.dtype == x.dtype)
 
     def _tracea_weight(self):
         # [K,C,R,S] -> [K,R,S,C], once per weight version
