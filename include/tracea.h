@@ -197,7 +197,15 @@ TraceaStatus tracea_low_rank_mlp(TraceaTensorView x, TraceaTensorView a, TraceaT
                                  TraceaTensorView *c, TraceaGemmParams params);
 
 /* ---- FlashAttention-2 forward: reference include/tracea.hpp:147-149,
- * src/interface/c_bindings.rs:443-495.  q,k,v,o [B,H,S,D]. */
+ * src/interface/c_bindings.rs:443-495.  q,k,v,o [B,H,S,D], f16 or bf16, D <= 128.
+ * The kernels read D = 64 or 128 with a contiguous head dimension, other strides
+ * multiples of 8 elements and bases on 16 bytes in place.  Any other D from 1 to
+ * 128 (the reference compiles its kernel for the head dimension at hand:
+ * src/kernels/attention/cuda_emitter.rs:39-58) and any other strides or bases
+ * run from zero-padded copies of q, k and v in the padded road's per-(device,
+ * stream) buffer (four tensors of B*H*S rows of 64 or 128 elements, at most
+ * 1 GiB, not grown under capture), the result copied out to o; scale 0 stays
+ * 1/sqrt(D) of the true D. */
 TraceaStatus tracea_attention(TraceaTensorView q, TraceaTensorView k, TraceaTensorView v,
                               TraceaTensorView *o, TraceaAttentionParams params);
 

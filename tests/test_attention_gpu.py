@@ -228,7 +228,7 @@ def test_strided_views_and_error_paths(tracea_gpu):
     o = tracea_gpu.attention(q, k, v, causal=True)
     want = oracle.attention_bhsd(*[t.float().cpu().numpy() for t in (q, k, v)], 1.0 / 8.0, True)
     assert_close_scaled(o.float().cpu().numpy(), want, _tol(d, "f16"), "strided q/k/v")
-    bad = torch.zeros(1, 1, 8, 48, device="cuda", dtype=torch.float16)
+    bad = torch.zeros(1, 1, 8, 160, device="cuda", dtype=torch.float16)   # above the kernels' 128
     with pytest.raises(capi.TraceaError) as e:
         tracea_gpu.attention(bad, bad, bad)
     assert e.value.status == capi.UNSUPPORTED_CONFIG
@@ -240,3 +240,40 @@ def test_strided_views_and_error_paths(tracea_gpu):
     with pytest.raises(capi.TraceaError) as e:
         tracea_gpu.attention(a, a[:, :, :4], a)
     assert e.value.status == capi.INVALID_PARAMS
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_other_head_dimensions_and_unaligned_tensors_run_from_padded_copies(tracea_gpu, dtype):
+    """Head dimensions off 64 and 128 (the reference compiles its kernel per head dimension:
+    src/kernels/attention/cuda_emitter.rs:39-58), a strided head dimension, odd strides and bases off
+    16 bytes: padded copies, the caller's scale (1/sqrt of the true D by default), result copied out."""
+    tdt, rnd = (torch.bfloat16, round_bf16) if dtype == "bf16" else (torch.float16, round_f16)
+    for (b, h, s, d) in [(2, 3, 77, 32), (1, 2, 200, 80), (2, 2, 130, 96), (1, 1, 64, 8), (1, 2, 33, 1), (1, 2, 150, 127)]:
+        q, k, v = _inputs(b, h, s, d, 7 * s + d, rnd)
+        for causal in (False, True):
+            want = oracle.attention_bhsd(q, k, v, 1.0 / np.sqrt(d), causal)
+            got = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=causal)
+            assert got.shape == (b, h, s, d)
+            assert_close_scaled(got.float().cpu().numpy(), want, _tol(d, dtype), "D=%d S=%d causal=%s %s" % (d, s, causal, dtype))
+    # an explicit scale goes through as given
+    b, h, s, d = 1, 2, 90, 40
+    q, k, v = _inputs(b, h, s, d, 5, rnd)
+    got = tracea_gpu.attention(_dev(q, tdt), _dev(k, tdt), _dev(v, tdt), causal=True, scale=0.25)
+    assert_close_scaled(got.float().cpu().numpy(), oracle.attention_bhsd(q, k, v, 0.25, True), _tol(d, dtype), "explicit scale")
+    # D = 64 the kernels could read, but: head dimension strided (a [B,H,D,S] tensor seen transposed), a
+    # sequence stride of 65 elements, a base 2 bytes off
+    b, h, s, d = 2, 2, 100, 64
+    q, k, v = _inputs(b, h, s, d, 11, rnd)
+    want = oracle.attention_bhsd(q, k, v, 1.0 / 8.0, False)
+    qt = _dev(q.transpose(0, 1, 3, 2), tdt).permute(0, 1, 3, 2)
+    assert qt.stride(3) != 1
+    kw = torch.zeros(b, h, s, 65, device="cuda", dtype=tdt)
+    kw[..., :64] = _dev(k, tdt)
+    flat = torch.zeros(b * h * s * d + 8, device="cuda", dtype=tdt)
+    vo = flat[1:1 + b * h * s * d].view(b, h, s, d)
+    vo.copy_(_dev(v, tdt))
+    assert vo.data_ptr() % 16 != 0
+    out_wide = torch.full((b, h, s, 72), 7.0, device="cuda", dtype=tdt)
+    got = tracea_gpu.attention(qt, kw[..., :64], vo, causal=False, out=out_wide[..., 3:67])
+    assert_close_scaled(got.float().cpu().numpy(), want, _tol(d, dtype), "unaligned tensors")
+    assert (out_wide[..., :3] == 7.0).all() and (out_wide[..., 67:] == 7.0).all()   # nothing written beside the result

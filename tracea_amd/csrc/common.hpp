@@ -138,12 +138,15 @@ struct GenericGemmArgs {
   EpilogueChain epi;
 };
 int launch_gemm_generic(const GenericGemmArgs &args, hipStream_t stream);
-// dst[r][c] (rows_dst rows of `pitch` elements of elt_bytes = 2 or 4) = src[(r / n1) * rs + (r % n1) * s1 + c * cs]
-// for r < rows_src and c < cols_src, zero elsewhere: an operand as the tile kernels can read it (rows on 16
-// bytes, a whole number of 16-byte pieces, zeros behind the data), from any two strides (n1 = 1) or, with the
-// rows in two levels, three.
+// An operand as the tile kernels can read it: dst[r][c] (rows_dst rows of `pitch` elements of elt_bytes = 2 or 4)
+// = src[r0 * rs + r1 * s1 + r2 * s2 + c * cs] for r = (r0 * n1 + r1) * n2 + r2 < rows_src and c < cols_src, zero
+// elsewhere (rows on 16 bytes, a whole number of 16-byte pieces, zeros behind the data), from up to four strides.
 int launch_pad_copy(const void *src, void *dst, int elt_bytes, long long rows_src, long long cols_src, long long rs,
-                    long long cs, long long rows_dst, long long pitch, hipStream_t stream, long long n1 = 1, long long s1 = 0);
+                    long long cs, long long rows_dst, long long pitch, hipStream_t stream, long long n1 = 1, long long s1 = 0,
+                    long long n2 = 1, long long s2 = 0);
+// The way back for a result: dst[r0 * rs + r1 * s1 + r2 * s2 + c * cs] = src[r][c] for r < rows, c < cols.
+int launch_unpad_copy(const void *src, void *dst, int elt_bytes, long long rows, long long cols, long long rs, long long cs,
+                      long long pitch, hipStream_t stream, long long n1 = 1, long long s1 = 0, long long n2 = 1, long long s2 = 0);
 
 // Second stage of a split-K contraction: out[m, n] = chain(sum over z of partial[z][m][n]).
 struct SplitKReduceArgs {

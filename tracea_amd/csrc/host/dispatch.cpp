@@ -2431,22 +2431,59 @@ TraceaStatus dispatch_attention(const TraceaTensorView &tq, const TraceaTensorVi
     return fail(TRACEA_INVALID_PARAMS, "tracea_attention: operands live on different devices");
   const long long B = q.shape[0], H = q.shape[1], S = q.shape[2], D = q.shape[3];
   if (B == 0 || H == 0 || S == 0) return TRACEA_SUCCESS;
-  if (D != 64 && D != 128)
-    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: head dim %lld (64 or 128 supported)", D);
+  if (D < 1 || D > 128)
+    return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: head dim %lld (1 to 128 supported)", D);
   if (S >= (1ll << 31) || B * H * ((S + 127) / 128) >= (1ll << 31))
     return fail(TRACEA_UNSUPPORTED_CONFIG, "tracea_attention: problem too large");
-  const View *views[4] = {&q, &k, &v, &o};
-  for (const View *t : views) {
-    if (t->stride[3] != 1 || t->stride[2] % 8 != 0 || t->stride[1] % 8 != 0 || t->stride[0] % 8 != 0 ||
-        !aligned(t->ptr, 16))
-      return fail(TRACEA_UNSUPPORTED_CONFIG,
-                  "tracea_attention: head dim must be contiguous, other strides multiples of 8 "
-                  "elements, bases 16-byte aligned");
-  }
   float scale = params.scale;
   if (scale == 0.0f) scale = 1.0f / sqrtf((float)D);
   if (!(scale == scale) || std::isinf(scale))
     return fail(TRACEA_INVALID_PARAMS, "tracea_attention: scale is not finite");
+  const View *views[4] = {&q, &k, &v, &o};
+  bool in_place = D == 64 || D == 128;
+  for (const View *t : views)
+    if (t->stride[3] != 1 || t->stride[2] % 8 != 0 || t->stride[1] % 8 != 0 || t->stride[0] % 8 != 0 || !aligned(t->ptr, 16))
+      in_place = false;
+  if (!in_place) {
+    // Head dimensions other than 64 and 128 (the kernels' two), and tensors the kernels cannot read in place
+    // (head dimension strided, other strides off a multiple of 8 elements, bases off 16 bytes): Q, K and V are
+    // copied into dense [B,H,S,Dp] tensors, Dp = 64 or 128, zeros behind the data -- they add nothing to a score
+    // and give zero output columns -- the kernels run on those with the caller's scale, and the first D columns
+    // of the result are copied out.  In the per-(device, stream) buffer of the padded GEMM operands; where it
+    // cannot be had the call is refused.  (The reference compiles its kernel for the head dimension at hand:
+    // src/kernels/attention/cuda_emitter.rs:39-58.)
+    static thread_local bool in_padded = false;
+    const long long Dp = D <= 64 ? 64 : 128;
+    const size_t one = (size_t)(B * H * S) * (size_t)Dp * 2;
+    DeviceScope pad_scope(o.device);
+    if (pad_scope.err != hipSuccess) return hip_status("hipSetDevice", (int)pad_scope.err);
+    unsigned char *buf = in_padded ? nullptr : (unsigned char *)pad_scratch(o.device, (hipStream_t)params.stream, 4 * one);
+    if (buf == nullptr)
+      return fail(TRACEA_UNSUPPORTED_CONFIG,
+                  "tracea_attention: head dim %lld / these strides need padded copies, and no buffer for them can be had "
+                  "(stream under capture, or above 1 GiB); in place: head dim 64 or 128, contiguous, other strides "
+                  "multiples of 8 elements, bases 16-byte aligned", D);
+    hipStream_t stream = (hipStream_t)params.stream;
+    const View *src[3] = {&q, &k, &v};
+    for (int i = 0; i < 3; ++i) {
+      const int e = launch_pad_copy(src[i]->ptr, buf + i * one, 2, B * H * S, D, src[i]->stride[0], src[i]->stride[3], B * H * S, Dp,
+                                    stream, H, src[i]->stride[1], S, src[i]->stride[2]);
+      if (e != 0) return hip_status("operand copy launch", e);
+    }
+    const uint64_t shape[4] = {(uint64_t)B, (uint64_t)H, (uint64_t)S, (uint64_t)Dp};
+    TraceaTensorView pq = tq, pk = tk, pv = tv, po = *to;
+    pq.ptr = buf; pk.ptr = buf + one; pv.ptr = buf + 2 * one; po.ptr = buf + 3 * one;
+    pq.shape = pk.shape = pv.shape = po.shape = shape;
+    pq.stride = pk.stride = pv.stride = po.stride = nullptr;
+    TraceaAttentionParams pp = params;
+    pp.scale = scale;
+    in_padded = true;
+    st = dispatch_attention(pq, pk, pv, &po, pp);
+    in_padded = false;
+    if (st != TRACEA_SUCCESS) return st;
+    return hip_status("result copy launch", launch_unpad_copy(buf + 3 * one, o.ptr, 2, B * H * S, D, o.stride[0], o.stride[3], Dp, stream,
+                                                              H, o.stride[1], S, o.stride[2]));
+  }
 
   AttentionArgs a{};
   a.Q = q.ptr; a.K = k.ptr; a.V = v.ptr; a.O = o.ptr;

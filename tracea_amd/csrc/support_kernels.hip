@@ -448,28 +448,52 @@ __global__ void __launch_bounds__(256) gemm_generic_kernel(const GenericGemmArgs
   store_from_float<1>(a.C, a.c_dtype, (long long)m * a.scm + (long long)n * a.scn, 1, v);
 }
 
-template <typename T>
-__global__ void __launch_bounds__(256) pad_copy_kernel(const T *src, T *dst, long long rows_src, long long cols_src, long long rs,
-                                                       long long cs, long long n1, long long s1, long long pitch, long long total) {
+// (row r of the padded side = ((r0 * n1) + r1) * n2 + r2; its first element on the strided side lies at
+// r0 * rs + r1 * s1 + r2 * s2.  TO_PADDED: strided -> padded rows, zeros behind the data; else the way back,
+// data only.)
+template <typename T, bool TO_PADDED>
+__global__ void __launch_bounds__(256) pad_copy_kernel(const T *src, T *dst, long long rows, long long cols, long long rs, long long cs,
+                                                       long long n1, long long s1, long long n2, long long s2, long long pitch,
+                                                       long long total) {
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= total) return;
-  const long long r = idx / pitch, c = idx - r * pitch;
-  const long long r0 = r / n1, r1 = r - r0 * n1;
-  dst[idx] = (r < rows_src && c < cols_src) ? src[r0 * rs + r1 * s1 + c * cs] : T(0);
+  const long long width = TO_PADDED ? pitch : cols;
+  const long long r = idx / width, c = idx - r * width;
+  const long long r01 = r / n2, r2 = r - r01 * n2;
+  const long long r0 = r01 / n1, r1 = r01 - r0 * n1;
+  const long long strided = r0 * rs + r1 * s1 + r2 * s2 + c * cs;
+  if constexpr (TO_PADDED) dst[idx] = (r < rows && c < cols) ? src[strided] : T(0);
+  else dst[strided] = src[r * pitch + c];
 }
 
 int launch_pad_copy(const void *src, void *dst, int elt_bytes, long long rows_src, long long cols_src, long long rs,
-                    long long cs, long long rows_dst, long long pitch, hipStream_t stream, long long n1, long long s1) {
+                    long long cs, long long rows_dst, long long pitch, hipStream_t stream, long long n1, long long s1,
+                    long long n2, long long s2) {
   const long long total = rows_dst * pitch;
   if (total <= 0) return 0;
   const long long blocks = (total + 255) / 256;
-  if (blocks >= (1ll << 31) || (elt_bytes != 2 && elt_bytes != 4) || n1 < 1) return (int)hipErrorInvalidValue;
+  if (blocks >= (1ll << 31) || (elt_bytes != 2 && elt_bytes != 4) || n1 < 1 || n2 < 1) return (int)hipErrorInvalidValue;
   if (elt_bytes == 2)
-    hipLaunchKernelGGL(pad_copy_kernel<unsigned short>, dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned short *)src,
-                       (unsigned short *)dst, rows_src, cols_src, rs, cs, n1, s1, pitch, total);
+    hipLaunchKernelGGL((pad_copy_kernel<unsigned short, true>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       (const unsigned short *)src, (unsigned short *)dst, rows_src, cols_src, rs, cs, n1, s1, n2, s2, pitch, total);
   else
-    hipLaunchKernelGGL(pad_copy_kernel<unsigned>, dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned *)src, (unsigned *)dst,
-                       rows_src, cols_src, rs, cs, n1, s1, pitch, total);
+    hipLaunchKernelGGL((pad_copy_kernel<unsigned, true>), dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned *)src,
+                       (unsigned *)dst, rows_src, cols_src, rs, cs, n1, s1, n2, s2, pitch, total);
+  return (int)hipGetLastError();
+}
+
+int launch_unpad_copy(const void *src, void *dst, int elt_bytes, long long rows, long long cols, long long rs, long long cs,
+                      long long pitch, hipStream_t stream, long long n1, long long s1, long long n2, long long s2) {
+  const long long total = rows * cols;
+  if (total <= 0) return 0;
+  const long long blocks = (total + 255) / 256;
+  if (blocks >= (1ll << 31) || (elt_bytes != 2 && elt_bytes != 4) || n1 < 1 || n2 < 1) return (int)hipErrorInvalidValue;
+  if (elt_bytes == 2)
+    hipLaunchKernelGGL((pad_copy_kernel<unsigned short, false>), dim3((unsigned)blocks), dim3(256), 0, stream,
+                       (const unsigned short *)src, (unsigned short *)dst, rows, cols, rs, cs, n1, s1, n2, s2, pitch, total);
+  else
+    hipLaunchKernelGGL((pad_copy_kernel<unsigned, false>), dim3((unsigned)blocks), dim3(256), 0, stream, (const unsigned *)src,
+                       (unsigned *)dst, rows, cols, rs, cs, n1, s1, n2, s2, pitch, total);
   return (int)hipGetLastError();
 }
 
