@@ -284,21 +284,44 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   // prologue STAGES-1 tiles are in flight or landed beyond the one being read.
   constexpr int PER = 2 * T * KSUB;  // requests per thread and tile; the wait count is bits 3:0 of the immediate
   constexpr int WAIT_FIRST = 0x0f70 | ((STAGES - 1) * PER), WAIT_NEXT = 0x0f70 | ((STAGES - 2) * PER);
+  // The operand reads are written as instructions.  Through a pointer the compiler puts a vmcnt(0) in front
+  // of the first of them that follows a tile request (it cannot tell that the request writes another stage),
+  // so every K tile waited out the request issued a few instructions earlier and no number of stages covered
+  // anything.  As instructions they are outside its bookkeeping: operands_landed, in front of the MFMAs that
+  // take them, is the wait.
   auto read_operands = [&](const unsigned char *cur, f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8]) {
+    const unsigned base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)cur;
 #pragma unroll
     for (int u = 0; u < KSUB; ++u) {
 #pragma unroll
       for (int i = 0; i < T; ++i)
 #pragma unroll
-        for (int c = 0; c < 2; ++c) af[u][i][c] = *(const f32x4 *)(cur + u * SUB + a_off[i][c]);
+        for (int c = 0; c < 2; ++c)
+          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[u][i][c]) : "v"(base + a_off[i][c]), "i"(u * SUB));
 #pragma unroll
       for (int j = 0; j < T; ++j)
 #pragma unroll
-        for (int t = 0; t < 8; ++t) bf[u][j][t] = *(const float *)(cur + u * SUB + b_off[j] + t * B_PITCH);
+        for (int t = 0; t < 8; ++t)
+          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(bf[u][j][t]) : "v"(base + b_off[j]), "i"(u * SUB + t * B_PITCH));
     }
   };
-  auto step = [&](int kt, const f32x4 (&af)[KSUB][T][2], const float (&bf)[KSUB][T][8], f32x4 (&af_next)[KSUB][T][2],
+  auto operands_landed = [&](f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8]) {
+    asm volatile("s_waitcnt lgkmcnt(0)");
+#pragma unroll
+    for (int u = 0; u < KSUB; ++u) {
+#pragma unroll
+      for (int i = 0; i < T; ++i)
+#pragma unroll
+        for (int c = 0; c < 2; ++c) asm volatile("" : "+v"(af[u][i][c]));
+#pragma unroll
+      for (int j = 0; j < T; ++j)
+#pragma unroll
+        for (int t = 0; t < 8; ++t) asm volatile("" : "+v"(bf[u][j][t]));
+    }
+  };
+  auto step = [&](int kt, f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8], f32x4 (&af_next)[KSUB][T][2],
                   float (&bf_next)[KSUB][T][8]) {
+    operands_landed(af, bf);
     // first half of tile kt's MFMAs, then the barrier, the requests and the operand reads of tile
     // kt+1 spread between the MFMAs of the second half: with one wave per SIMD whatever is issued
     // between two barriers without an MFMA in flight is time the matrix pipe stands still
@@ -319,7 +342,11 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
 #pragma unroll
       for (int t = 0; t < 4; ++t) mfma(u, t);
     __builtin_amdgcn_s_waitcnt(WAIT_NEXT);  // tile kt+1 has landed (this wave's share)
-    __syncthreads();                        // ... everyone's, and everyone holds its operands of tile kt
+    // ... everyone's, and everyone holds its operands of tile kt.  The barrier alone: with the fences of
+    // __syncthreads() the compiler waits for every request in flight, those of the later tiles included.
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
     dma(smem + (kt % STAGES) * STAGE, (kt + STAGES) * BK);
     read_operands(smem + ((kt + 1) % STAGES) * STAGE, af_next, bf_next);
 #pragma unroll
@@ -345,8 +372,11 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
     step(kt, af0, bf0, af1, bf1);
     if (kt + 1 < nk) step(kt + 1, af1, bf1, af0, bf0);
   }
-  // requests past the end of K may still be writing zeros where the epilogue stages
-  __builtin_amdgcn_s_waitcnt(0x0f70);
+  // requests past the end of K may still be writing zeros where the epilogue stages, and the last operand reads
+  // (of a tile nobody multiplies) may still be writing their registers
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  operands_landed(af0, bf0);
+  operands_landed(af1, bf1);
   __syncthreads();
   if constexpr (T == 1) {
 #pragma unroll
