@@ -300,8 +300,8 @@ TraceaStatus tracea_linear(TraceaTensorView a, TraceaTensorView w, const TraceaT
 
 
 /* Split-K.  A gemm / conv2d launch with few output tiles and a long K (tiles * 2 <= 256 CUs,
- * at least 8 K tiles; the 64x64 tile of the fp32 GEMM: up to about four workgroups per CU, ranges of at least
- * 16 K tiles of 16) is split along K
+ * at least 8 K tiles; the 64x64 tile of the fp32 GEMM: one to four ranges of at least 16 K tiles of 16, at
+ * most 4.5 workgroups per CU, the count with the least estimated time) is split along K
  * over more workgroups; fp32 partial products go to a
  * scratch buffer the library keeps per (device, stream) (grown on demand up to 64 MiB, never
  * while the stream is being captured, never freed) and a second kernel sums them and applies

@@ -127,7 +127,7 @@ int contraction_variant_count();
 const ContractionVariant &contraction_variant(int i);
 
 // fp32 MFMA GEMM (row-major A [M,K], row-major B [K,N]).
-int launch_gemm_f32(const ContractionArgs &args, int tile, hipStream_t stream);  // tile: 128 or 64
+int launch_gemm_f32(const ContractionArgs &args, int tile, hipStream_t stream);  // tile: 128, 64 or 6432 (64x64 with K tiles of 32)
 // Any dtype/stride combination, no alignment requirement (VALU, slow).
 struct GenericGemmArgs {
   const void *A, *B;

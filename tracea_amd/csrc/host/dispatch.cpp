@@ -821,41 +821,53 @@ TraceaStatus run_gemm(const View &a, const View &b, const View &c, const Epilogu
     // Two tile shapes, 128x128x16 and (direct-to-LDS form only) 64x64x16.  A CU works through its
     // share of the tiles at one 128x128 tile per 4 units of time or one 64x64 tile per 1.06 units
     // (the small tile reads its operands from LDS twice as often): the shape whose busiest CU
-    // finishes first is taken.  Measured, 128 / 64, in us: 1024^3 32.5 / 27.0, 1536^3 104 / 79,
-    // 2304x2048x512 70 / 49, 3072^3 539 / 454, 2048^3 138 / 135, 4096^3 972 / 1027.
-    // Both split along K by the rule of the half kernels.
+    // finishes first is taken.  Measured, 128 / 64, in us: 1024^3 68 / 24.7, 1536^3 102 / 77,
+    // 3072^3 558 / 441, 2048^3 134.7 / 133.4, 4096^3 972 / 1033.  (A 128x64 tile was never the fastest:
+    // 477 at 3072^3, 1003 at 4096^3.)
     static const ContractionVariant f32_tile128 = {"f32_128x128x16", 128, 128, 16, 2, 2, 1, 0, 0, nullptr, 32};
-    static const ContractionVariant f32_tile64 = {"f32_64x64x16", 64, 64, 16, 2, 2, 1, 0, 0, nullptr, 32};
     const long long tiles128 = ((M + 127) / 128) * ((N + 127) / 128), tiles64 = ((M + 63) / 64) * ((N + 63) / 64);
     const long long ncu = device_limits().cus;
-    const int tile = args.a_bytes != 0 && (double)((tiles64 + ncu - 1) / ncu) * 1.06 < (double)((tiles128 + ncu - 1) / ncu) * 4.0 ? 64 : 128;
+    int tile = args.a_bytes != 0 && (double)((tiles64 + ncu - 1) / ncu) * 1.06 < (double)((tiles128 + ncu - 1) / ncu) * 4.0 ? 64 : 128;
     int k_split = 0, splits = 1;
     t_last_split_launches = 1;
     const bool can_fuse = args.a_bytes != 0 && !static_only && g_split_k_enabled.load() && g_split_k_one_launch.load();
     const int nk = (int)((K + 15) / 16);
-    if (tile == 64 && args.a_bytes != 0 && g_split_k_enabled.load()) {
+    if (tile == 64) {
       // (the same K ranges whether the sum then runs in the launch or, for the entry point that must not
       // allocate or with one-launch splits switched off, in a reduction kernel: the results are the same bits)
-      // The 64x64 tile splits in one launch (the tile's last workgroup sums, see the kernel), and it wants about
-      // four workgroups per CU: a workgroup is one wave per SIMD walking K alone, and the others' MFMAs run
-      // under its waits.  Ranges of at least 16 K tiles, at most four.  Measured (us, replayed graphs,
-      // unsplit -> split): 1024^3 30.3 -> 26.0, 1024x1024x2048 79.5 -> 44.4, 768x1024x1024 28.1 -> 22.6,
-      // 2048x1024x1024 55.5 -> 44.7, 1536^3 98.2 -> 95.3; 2048^3 (four tiles per CU as it is) stays unsplit.
-      long long want = (4 * ncu + tiles64 / 2) / tiles64;
-      if (want > kOneLaunchMaxSplits) want = kOneLaunchMaxSplits;
-      if (want > nk / 16) want = nk / 16;
-      if (want >= 2) {
-        const int per = (int)((nk + want - 1) / want);
+      // The 64x64 tile splits in one launch (the tile's last workgroup sums, see the kernel).  Up to four ranges
+      // of at least 16 K tiles, and no more than 4.5 workgroups per CU; among those the count with the least
+      // estimated time, in K tiles of one workgroup: rounds of workgroups over the CUs x K tiles per range,
+      // x 0.9 where at least two workgroups share a CU (one's MFMAs run under the other's waits), x 0.92 where
+      // there is at most one per CU (it then runs K tiles of 32: half the barriers, and the 64 KB of LDS
+      // displace nobody), + 3 for a split + 4 per range beyond two (partial tiles written and read again).
+      // Measured (us, replayed graphs, 1 / 2 / 4 ranges): 1024^3 24.7 (22.8 on K tiles of 32) / 23.9 / 26.8,
+      // 1024x1024x2048 42.5 (41.8) / 40.3 / 42.3, 768x1024x1024 23.5 / 23.5 / 20.1, 1536^3 76.9 / 67.7 / -,
+      // 2048^3 133.4 / 137.5 / -.
+      int best = 1;
+      if (g_split_k_enabled.load()) {
+        double best_cost = 0.0;
+        for (int s = 1; s <= kOneLaunchMaxSplits && (s == 1 || (s <= nk / 16 && tiles64 * s * 2 <= 9 * ncu)); ++s) {
+          const long long wgs = tiles64 * s;
+          const double share = wgs >= 2 * ncu ? 0.9 : wgs <= ncu ? 0.92 : 1.0;
+          const double cost = (double)((wgs + ncu - 1) / ncu) * (double)((nk + s - 1) / s) * share + (s > 1 ? 3.0 + 4.0 * (s - 2) : 0.0);
+          if (s == 1 || cost < best_cost) { best = s; best_cost = cost; }
+        }
+      }
+      if (tiles64 * best <= ncu) tile = 6432;
+      if (best >= 2) {
+        int per = (nk + best - 1) / best;
+        if (tile == 6432) per += per & 1;  // whole K tiles of 32
         k_split = per * 16;
         splits = (nk + per - 1) / per;
       }
     } else {
-      const ContractionVariant &f32_tile0 = tile == 64 ? f32_tile64 : f32_tile128;
-      splits = g_split_k_enabled.load() ? choose_split(f32_tile0, (int)M, (int)N, (int)K, &k_split, tile == 64 ? 16 : 4) : 1;
+      splits = g_split_k_enabled.load() ? choose_split(f32_tile128, (int)M, (int)N, (int)K, &k_split, 4) : 1;
     }
-    const long long tiles = tile == 64 ? tiles64 : tiles128;
+    const long long tiles = tile == 128 ? tiles128 : tiles64;
+    const size_t tile_elts = tile == 128 ? 128 * 128 : 64 * 64;
     if (can_fuse && splits > 1 && splits <= kOneLaunchMaxSplits && tiles <= kFuseTiles) {
-      void *fws = splitk_scratch(c.device, stream, (size_t)tiles * (size_t)splits * (size_t)(tile * tile) * 4);
+      void *fws = splitk_scratch(c.device, stream, (size_t)tiles * (size_t)splits * tile_elts * 4);
       unsigned *cnt = fws != nullptr ? fuse_counters(c.device, stream) : nullptr;
       if (cnt != nullptr) {
         args.epi = chain;

@@ -182,13 +182,13 @@ __global__ void __launch_bounds__(256) gemm_f32_kernel(const ContractionArgs arg
 // out of range (they write zeros to a stage nobody multiplies), so that the
 // count of outstanding requests a wave waits on is the same in every iteration.
 // ---------------------------------------------------------------------------
-template <int T, int STAGES, int KSUB>
+template <int TM, int TN, int STAGES, int KSUB, int FIRST_T = 1>
 __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs args) {
-  constexpr int BM = 64 * T, BN = 64 * T, BK = F32_BK * KSUB;  // a stage holds KSUB sub-tiles of 16 k, each [A][B]
+  constexpr int BM = 64 * TM, BN = 64 * TN, BK = F32_BK * KSUB;  // a stage holds KSUB sub-tiles of 16 k, each [A][B]
   constexpr int A_STAGE = BM * F32_BK * 4, B_STAGE = F32_BK * BN * 4, SUB = A_STAGE + B_STAGE, STAGE = KSUB * SUB;
   constexpr int B_PITCH = BN * 4, B_PIECES = BN / 4;  // bytes and 16-byte pieces per k row of B
-  static_assert(STAGES * STAGE >= 4 * 32 * 32 * T * 4, "the epilogue stages 32 rows per wave in the tile buffers");
-  static_assert((STAGES - 1) * 2 * T * KSUB < 16, "outstanding requests must fit the 4-bit wait count used here");
+  static_assert(STAGES * STAGE >= 4 * 32 * 32 * TN * 4, "the epilogue stages 32 rows per wave in the tile buffers");
+  static_assert((STAGES - 1) * (TM + TN) * KSUB < 64, "outstanding requests must fit the 6-bit wait count");
   __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * STAGE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
@@ -206,55 +206,59 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   constexpr unsigned OOB = 0x80000000u;
   __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void *)args.A, 0, (int)args.a_bytes, 0x00020000);
   __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc((void *)args.B, 0, (int)args.b_bytes, 0x00020000);
-  // T pieces of A and T of B per thread and K tile
-  unsigned a_voff[T], b_voff[T];
-  int a_kcol[T], b_krow[T];
+  // TM pieces of A and TN of B per thread and K tile
+  unsigned a_voff[TM], b_voff[TN];
+  int a_kcol[TM], b_krow[TN];
 #pragma unroll
-  for (int i = 0; i < T; ++i) {
+  for (int i = 0; i < TM; ++i) {
     const int q = tid + i * 256;
     const int row = q >> 2;
     int m = m0 + row;
     m = m < M ? m : M - 1;  // rows past the end re-read the last row; their results are never stored
     a_kcol[i] = ((q & 3) ^ ((row >> 2) & 3)) * 4;
     a_voff[i] = (unsigned)(((long long)m * args.lda + a_kcol[i]) * 4);
+  }
+#pragma unroll
+  for (int i = 0; i < TN; ++i) {
+    const int q = tid + i * 256;
     b_krow[i] = q / B_PIECES;
     const int n = n0 + (((q % B_PIECES) ^ ((b_krow[i] >> 3) << 3)) << 2);
     b_voff[i] = n < N ? (unsigned)(((long long)b_krow[i] * args.ldb + n) * 4) : OOB;
   }
-  auto dma_sub = [&](unsigned char *stage, int k0) {
-    k0 += kb;
+  // request r of a K tile: sub-tile r / (TM + TN), then TM pieces of A and TN of B
+  auto dma_nth = [&](unsigned char *stage, int k0, int r) __attribute__((always_inline)) {
+    const int u = r / (TM + TN), w = r % (TM + TN);
+    stage += u * SUB;
+    k0 += kb + u * F32_BK;
     const bool any = k0 < K;  // uniform: a tile wholly past K asks for nothing but zeros
-    const int so_a = any ? k0 * 4 : 0;
-    const int so_b = any ? (int)((long long)k0 * args.ldb * 4) : 0;
-#pragma unroll
-    for (int i = 0; i < T; ++i) {
-      unsigned char *dst = stage + (i * 256 + wave_u * 64) * 16;
-      const unsigned va = k0 + a_kcol[i] < K ? a_voff[i] : OOB;
+    if (w < TM) {
+      unsigned char *dst = stage + (w * 256 + wave_u * 64) * 16;
+      const unsigned va = k0 + a_kcol[w] < K ? a_voff[w] : OOB;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void *)dst, 16, (int)va,
-                                               so_a, 0, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < T; ++i) {
-      unsigned char *dst = stage + A_STAGE + (i * 256 + wave_u * 64) * 16;
-      const unsigned vb = k0 + b_krow[i] < K ? b_voff[i] : OOB;
+                                               any ? k0 * 4 : 0, 0, 0);
+    } else {
+      unsigned char *dst = stage + A_STAGE + ((w - TM) * 256 + wave_u * 64) * 16;
+      const unsigned vb = k0 + b_krow[w - TM] < K ? b_voff[w - TM] : OOB;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b, (__attribute__((address_space(3))) void *)dst, 16, (int)vb,
-                                               so_b, 0, 0);
+                                               any ? (int)((long long)k0 * args.ldb * 4) : 0, 0, 0);
     }
   };
+  constexpr int REQS = (TM + TN) * KSUB;  // requests per thread and K tile
   auto dma = [&](unsigned char *stage, int k0) {
 #pragma unroll
-    for (int u = 0; u < KSUB; ++u) dma_sub(stage + u * SUB, k0 + u * F32_BK);
+    for (int r = 0; r < REQS; ++r) dma_nth(stage, k0, r);
   };
 
-  f32x16 acc[T][T];
+  constexpr bool ONE = TM * TN == 1;
+  f32x16 acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < T; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < T; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  // With one 32x32 block per wave (T = 1) every MFMA would wait for the one before it, the same accumulator
+  // With one 32x32 block per wave (TM = TN = 1) every MFMA would wait for the one before it, the same accumulator
   // being its input: the odd k pairs of a tile go to a second accumulator, added in once at the end, and
   // the matrix pipe always has an independent MFMA to start.
   f32x16 acc_odd;
@@ -262,19 +266,19 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   for (int e = 0; e < 16; ++e) acc_odd[e] = 0.0f;
 
   const int lrow = lane & 31, lhalf = lane >> 5;
-  // A: row wm*32T + i*32 + lrow, 16-byte columns 2h and 2h+1 (k = 8h .. 8h+7)
-  int a_off[T][2];
+  // A: row wm*32TM + i*32 + lrow, 16-byte columns 2h and 2h+1 (k = 8h .. 8h+7)
+  int a_off[TM][2];
 #pragma unroll
-  for (int i = 0; i < T; ++i) {
-    const int row = wm * (32 * T) + i * 32 + lrow;
+  for (int i = 0; i < TM; ++i) {
+    const int row = wm * (32 * TM) + i * 32 + lrow;
 #pragma unroll
     for (int c = 0; c < 2; ++c) a_off[i][c] = row * 64 + (((2 * lhalf + c) ^ ((row >> 2) & 3)) << 4);
   }
-  // B: k row 8h + t, channel wn*32T + j*32 + lrow
-  int b_off[T];
+  // B: k row 8h + t, channel wn*32TN + j*32 + lrow
+  int b_off[TN];
 #pragma unroll
-  for (int j = 0; j < T; ++j) {
-    const int n = wn * (32 * T) + j * 32 + lrow;
+  for (int j = 0; j < TN; ++j) {
+    const int n = wn * (32 * TN) + j * 32 + lrow;
     b_off[j] = A_STAGE + (8 * lhalf) * B_PITCH + ((((n >> 2) ^ (lhalf << 3)) << 2) + (n & 3)) * 4;
   }
 
@@ -282,82 +286,93 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   // wave per SIMD nothing else would cover the latency of those reads).  Stage kt%STAGES is free
   // once every wave has its operands of tile kt, so tile kt+STAGES is requested into it: after the
   // prologue STAGES-1 tiles are in flight or landed beyond the one being read.
-  constexpr int PER = 2 * T * KSUB;  // requests per thread and tile; the wait count is bits 3:0 of the immediate
-  constexpr int WAIT_FIRST = 0x0f70 | ((STAGES - 1) * PER), WAIT_NEXT = 0x0f70 | ((STAGES - 2) * PER);
+  constexpr int PER = REQS;
+  constexpr auto vmcnt = [](int n) constexpr { return 0x0f70 | (n & 15) | ((n >> 4) << 14); };  // the count's bits 5:4 sit in 15:14
+  constexpr int WAIT_FIRST = vmcnt((STAGES - 1) * PER), WAIT_NEXT = vmcnt((STAGES - 2) * PER);
   // The operand reads are written as instructions.  Through a pointer the compiler puts a vmcnt(0) in front
   // of the first of them that follows a tile request (it cannot tell that the request writes another stage),
   // so every K tile waited out the request issued a few instructions earlier and no number of stages covered
   // anything.  As instructions they are outside its bookkeeping: operands_landed, in front of the MFMAs that
   // take them, is the wait.
-  auto read_operands = [&](const unsigned char *cur, f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8]) {
+  constexpr int READS_SUB = 2 * TM + 8 * TN, READS = KSUB * READS_SUB;  // operand reads per sub-tile and per K tile
+  auto read_nth = [&](unsigned base, f32x4 (&af)[KSUB][TM][2], float (&bf)[KSUB][TN][8], int r) __attribute__((always_inline)) {
+    const int u = r / READS_SUB, w = r % READS_SUB;
+    if (w < 2 * TM)
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[u][w >> 1][w & 1]) : "v"(base + a_off[w >> 1][w & 1]), "i"(u * SUB));
+    else
+      asm volatile("ds_read_b32 %0, %1 offset:%2"
+                   : "=v"(bf[u][(w - 2 * TM) >> 3][(w - 2 * TM) & 7])
+                   : "v"(base + b_off[(w - 2 * TM) >> 3]), "i"(u * SUB + ((w - 2 * TM) & 7) * B_PITCH));
+  };
+  auto read_operands = [&](const unsigned char *cur, f32x4 (&af)[KSUB][TM][2], float (&bf)[KSUB][TN][8]) {
     const unsigned base = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)cur;
 #pragma unroll
-    for (int u = 0; u < KSUB; ++u) {
-#pragma unroll
-      for (int i = 0; i < T; ++i)
-#pragma unroll
-        for (int c = 0; c < 2; ++c)
-          asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(af[u][i][c]) : "v"(base + a_off[i][c]), "i"(u * SUB));
-#pragma unroll
-      for (int j = 0; j < T; ++j)
-#pragma unroll
-        for (int t = 0; t < 8; ++t)
-          asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(bf[u][j][t]) : "v"(base + b_off[j]), "i"(u * SUB + t * B_PITCH));
-    }
+    for (int r = 0; r < READS; ++r) read_nth(base, af, bf, r);
   };
-  auto operands_landed = [&](f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8]) {
+  auto operands_landed = [&](f32x4 (&af)[KSUB][TM][2], float (&bf)[KSUB][TN][8]) {
     asm volatile("s_waitcnt lgkmcnt(0)");
 #pragma unroll
     for (int u = 0; u < KSUB; ++u) {
 #pragma unroll
-      for (int i = 0; i < T; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int c = 0; c < 2; ++c) asm volatile("" : "+v"(af[u][i][c]));
 #pragma unroll
-      for (int j = 0; j < T; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int t = 0; t < 8; ++t) asm volatile("" : "+v"(bf[u][j][t]));
     }
   };
-  auto step = [&](int kt, f32x4 (&af)[KSUB][T][2], float (&bf)[KSUB][T][8], f32x4 (&af_next)[KSUB][T][2],
-                  float (&bf_next)[KSUB][T][8]) {
+  auto step = [&](int kt, f32x4 (&af)[KSUB][TM][2], float (&bf)[KSUB][TN][8], f32x4 (&af_next)[KSUB][TM][2],
+                  float (&bf_next)[KSUB][TN][8]) {
     operands_landed(af, bf);
-    // first half of tile kt's MFMAs, then the barrier, the requests and the operand reads of tile
-    // kt+1 spread between the MFMAs of the second half: with one wave per SIMD whatever is issued
-    // between two barriers without an MFMA in flight is time the matrix pipe stands still
-    auto mfma = [&](int u, int t) {
-      if constexpr (T == 1) {
+    // A few of tile kt's MFMAs, then the barrier, then the rest with the requests of tile kt+STAGES and the
+    // operand reads of tile kt+1 between them: with one wave per SIMD whatever is issued without an MFMA in
+    // flight is time the matrix pipe stands still.  A request holds the wave for about 64 cycles (measured:
+    // two behind one MFMA cost the pipe 65 cycles, four behind two 220), so each goes behind an MFMA of its
+    // own; the reads, about 8 cycles each, follow at an even rate and leave the last MFMAs for their
+    // latency.  (The order is held with scheduling barriers: left alone the compiler puts every MFMA
+    // behind the barrier and the requests, and the matrix pipe drains while the workgroup gathers.)
+    auto mfma_nth = [&](int q) __attribute__((always_inline)) {
+      const int j = q % TN, i = (q / TN) % TM, t = (q / (TN * TM)) % 8, u = q / (TN * TM * 8);
+      if constexpr (ONE) {
         if (t & 1) acc_odd = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][0][t], af[u][0][t >> 2][t & 3], acc_odd, 0, 0, 0);
         else acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][0][t], af[u][0][t >> 2][t & 3], acc[0][0], 0, 0, 0);
       } else {
-#pragma unroll
-        for (int i = 0; i < T; ++i)
-#pragma unroll
-          for (int j = 0; j < T; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[u][j][t], af[u][i][t >> 2][t & 3], acc[i][j], 0, 0, 0);
       }
     };
+    constexpr int MFMAS = 8 * TM * TN * KSUB;   // of a K tile
+    constexpr int FIRST = FIRST_T * TM * TN;    // in front of the barrier: they cover the gathering of the workgroup
+    constexpr int LAND = ONE ? 1 : 2;           // the last ones, with nothing behind them
+    constexpr int READ_SLOTS = MFMAS - FIRST - REQS - LAND;
+    constexpr int PER_MFMA = (READS + READ_SLOTS - 1) / READ_SLOTS;
+    static_assert(READ_SLOTS > 0, "every request and read has its place");
 #pragma unroll
-    for (int u = 0; u < KSUB; ++u)
-#pragma unroll
-      for (int t = 0; t < 4; ++t) mfma(u, t);
+    for (int q = 0; q < FIRST; ++q) mfma_nth(q);
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt(WAIT_NEXT);  // tile kt+1 has landed (this wave's share)
     // ... everyone's, and everyone holds its operands of tile kt.  The barrier alone: with the fences of
     // __syncthreads() the compiler waits for every request in flight, those of the later tiles included.
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    dma(smem + (kt % STAGES) * STAGE, (kt + STAGES) * BK);
-    read_operands(smem + ((kt + 1) % STAGES) * STAGE, af_next, bf_next);
+    const unsigned next = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)(smem + ((kt + 1) % STAGES) * STAGE);
+    unsigned char *freed = smem + (kt % STAGES) * STAGE;
 #pragma unroll
-    for (int u = 0; u < KSUB; ++u)
+    for (int q = FIRST; q < MFMAS; ++q) {
+      mfma_nth(q);
+      const int slot = q - FIRST;
+      if (slot < REQS) {
+        dma_nth(freed, (kt + STAGES) * BK, slot);
+      } else {
 #pragma unroll
-      for (int t = 4; t < 8; ++t) mfma(u, t);
-    __builtin_amdgcn_sched_group_barrier(0x020, 2 * T * KSUB, 0);  // the requests first
-#pragma unroll
-    for (int q = 0; q < 4 * T * T * KSUB; ++q) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, T == 1 ? 3 : 2, 0);
+        for (int x = 0; x < PER_MFMA; ++x) {
+          const int r = (slot - REQS) * PER_MFMA + x;
+          if (r < READS) read_nth(next, af_next, bf_next, r);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   const int nk = (K - kb + BK - 1) / BK;
@@ -365,8 +380,8 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   for (int s = 0; s < STAGES; ++s) dma(smem + s * STAGE, s * BK);
   __builtin_amdgcn_s_waitcnt(WAIT_FIRST);
   __syncthreads();
-  f32x4 af0[KSUB][T][2], af1[KSUB][T][2];
-  float bf0[KSUB][T][8], bf1[KSUB][T][8];
+  f32x4 af0[KSUB][TM][2], af1[KSUB][TM][2];
+  float bf0[KSUB][TN][8], bf1[KSUB][TN][8];
   read_operands(smem, af0, bf0);
   for (int kt = 0; kt < nk; kt += 2) {
     step(kt, af0, bf0, af1, bf1);
@@ -378,7 +393,7 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
   operands_landed(af0, bf0);
   operands_landed(af1, bf1);
   __syncthreads();
-  if constexpr (T == 1) {
+  if constexpr (ONE) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[0][0][e] += acc_odd[e];
   }
@@ -396,13 +411,13 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
     const unsigned first = blockIdx.x * splits * TILE_BYTES + wave_u * WAVE_BYTES + lane * 16;
     const unsigned mine = first + blockIdx.y * TILE_BYTES;
 #pragma unroll
-    for (int i = 0; i < T; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < T; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const f32x4 v = {acc[i][j][g * 4 + 0], acc[i][j][g * 4 + 1], acc[i][j][g * 4 + 2], acc[i][j][g * 4 + 3]};
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_ws, (int)(mine + ((i * T + j) * 4 + g) * 1024), 0,
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rsrc_ws, (int)(mine + ((i * TN + j) * 4 + g) * 1024), 0,
                                                  DEVICE_SCOPE);
         }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): the stores are acknowledged
@@ -412,44 +427,46 @@ __global__ void __launch_bounds__(256) gemm_f32_dma_kernel(const ContractionArgs
     if (s_ticket != splits - 1) return;
     if (tid == 0) __hip_atomic_store(args.fuse_count + blockIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-    for (int i = 0; i < T; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
-      for (int j = 0; j < T; ++j)
+      for (int j = 0; j < TN; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 #pragma unroll 1
     for (unsigned z = 0; z < splits; ++z) {
 #pragma unroll
-      for (int i = 0; i < T; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < T; ++j)
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
             const f32x4 v = __builtin_bit_cast(
-                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_ws, (int)(first + z * TILE_BYTES + ((i * T + j) * 4 + g) * 1024), 0,
+                f32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc_ws, (int)(first + z * TILE_BYTES + ((i * TN + j) * 4 + g) * 1024), 0,
                                                            DEVICE_SCOPE));
 #pragma unroll
             for (int e = 0; e < 4; ++e) acc[i][j][g * 4 + e] += v[e];
           }
     }
   }
-  f32_tile_epilogue<32, T, T>(acc, (float *)smem + wave_u * (32 * 32 * T), args, m0 + wm * (32 * T), n0 + wn * (32 * T),
+  f32_tile_epilogue<32, TM, TN>(acc, (float *)smem + wave_u * (32 * 32 * TN), args, m0 + wm * (32 * TM), n0 + wn * (32 * TN),
                               zrow, lane);
 }
 
 int launch_gemm_f32(const ContractionArgs &a, int tile, hipStream_t stream) {
   ContractionArgs args = a;
-  // the 64x64 tile exists in the direct-to-LDS form only (operands below 2 GiB, a_bytes / b_bytes set by the dispatcher)
+  // the 64x64 tiles exist in the direct-to-LDS form only (operands below 2 GiB, a_bytes / b_bytes set by the dispatcher)
   const bool dma = a.a_bytes != 0 && a.b_bytes != 0;
-  if (tile != 64 || !dma) tile = 128;
-  args.grid_m = (a.M + tile - 1) / tile;
-  args.grid_n = (a.N + tile - 1) / tile;
+  if ((tile != 64 && tile != 6432) || !dma) tile = 128;
+  const int edge = tile == 128 ? 128 : 64;
+  args.grid_m = (a.M + edge - 1) / edge;
+  args.grid_n = (a.N + edge - 1) / edge;
   args.group_m = 4;
   const unsigned splits = a.k_split > 0 ? (unsigned)((a.K + a.k_split - 1) / a.k_split) : 1u;
   const dim3 grid((unsigned)(args.grid_m * args.grid_n), splits);
   if (!dma) hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, stream, args);
-  else if (tile == 64) hipLaunchKernelGGL((gemm_f32_dma_kernel<1, 4, 1>), grid, dim3(256), 0, stream, args);
-  else hipLaunchKernelGGL((gemm_f32_dma_kernel<2, 2, 1>), grid, dim3(256), 0, stream, args);
+  else if (tile == 64) hipLaunchKernelGGL((gemm_f32_dma_kernel<1, 1, 4, 1>), grid, dim3(256), 0, stream, args);
+  else if (tile == 6432) hipLaunchKernelGGL((gemm_f32_dma_kernel<1, 1, 4, 2>), grid, dim3(256), 0, stream, args);
+  else hipLaunchKernelGGL((gemm_f32_dma_kernel<2, 2, 2, 1>), grid, dim3(256), 0, stream, args);
   return (int)hipGetLastError();
 }
 
