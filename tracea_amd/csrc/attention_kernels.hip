@@ -753,20 +753,46 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     Interleave3<0, 2 * KS>::run();
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The transposed V operand of P.V step (kk, d): V rows kk*16.., head-dim block d.
-  auto read_v = [&](const unsigned char *sV, int kk, int d) __attribute__((always_inline)) -> u32x4 {
+  // The transposed V operand of P.V step (kk, d): V rows kk*16.., head-dim block d.  The two transposing reads
+  // of a fragment are written as instructions: through the builtin the compiler puts a vmcnt(0) in front of the
+  // first of them that follows a tile request (it cannot tell that the request writes another stage), and every
+  // iteration then waited in its middle for the K and V tiles it had asked for at its head.  As instructions they
+  // are outside its bookkeeping; v_landed, on the fragment, is the wait (LDS answers in order: lgkmcnt(N) says
+  // "all but the latest N").  v_lane[d]: the lane's part of the address, first row g*4 + (r>>2) of key block 0;
+  // the piece swizzle has a period of RP * WIN = 4 rows, so key block kk and the fragment's second half (8 rows
+  // on) are immediates.
+  static_assert(8 % (RP * WIN) == 0, "the V piece swizzle must repeat every 8 rows");
+  unsigned v_lane[DB];
+  {
     const int r = lane & 15;
-    const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
-    const int row_lo = kk * 16 + g * 4 + (r >> 2);
-    const int row_hi = row_lo + 8;
-    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_lo, col >> 3) + (col & 7) * 2));
-    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-        (__attribute__((address_space(3))) s16x4 *)(sV + v_piece(row_hi, col >> 3) + (col & 7) * 2));
-    const u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
-    u32x4 vf;
+#pragma unroll
+    for (int d = 0; d < DB; ++d) {
+      const int col = d * 32 + ((lane >> 4) & 1) * 16 + (r & 3) * 4;
+      v_lane[d] = (unsigned)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)sVbase +
+                  (unsigned)(v_piece(g * 4 + (r >> 2), col >> 3) + (col & 7) * 2);
+    }
+  }
+  // (va: v_lane plus whatever of the stage's offset is not in the immediate OFF)
+  auto issue_v = [&](const unsigned (&va)[DB], auto off_tag, int kk, int d, u32x4 &vf) __attribute__((always_inline)) {
+    constexpr int OFF = decltype(off_tag)::value;
+    u32x2 lo2, hi2;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo2) : "v"(va[d]), "i"(OFF + kk * 16 * ROW_BYTES));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi2) : "v"(va[d]), "i"(OFF + kk * 16 * ROW_BYTES + 8 * ROW_BYTES));
     vf[0] = lo2[0]; vf[1] = lo2[1]; vf[2] = hi2[0]; vf[3] = hi2[1];
-    return vf;
+  };
+  auto v_landed = [&](auto newer_tag, u32x4 &vf) __attribute__((always_inline)) {
+    constexpr int NEWER = decltype(newer_tag)::value;  // LDS instructions issued behind the fragment's two
+    static_assert(NEWER == 0 || NEWER == 2, "fragments in flight");
+    if constexpr (NEWER == 0) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(vf));
+    else asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(vf));
+  };
+  // a stage's offset as an immediate where the stage is a constant of the loop's copy and the offsets fit 16 bits
+  auto v_stage = [&](auto stage_tag, int stage, unsigned (&va)[DB]) __attribute__((always_inline)) {
+    constexpr int STG = decltype(stage_tag)::value;
+    constexpr bool IMM = STG >= 0 && STG * TILE_BYTES + 56 * ROW_BYTES < 65536;
+#pragma unroll
+    for (int d = 0; d < DB; ++d) va[d] = IMM ? v_lane[d] : v_lane[d] + (unsigned)(stage * TILE_BYTES);
+    return std::integral_constant<int, IMM ? STG * TILE_BYTES : 0>{};
   };
 
   // The barrier at the head of iteration t publishes K(t+1) and V(t) and retires K(t) and V(t-1),
@@ -837,7 +863,8 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // K and V fragments are loop invariants plus immediates instead of an addition per read group.
   auto iteration_on = [&](int t, auto edge_tag, f32x16 (&cur)[QB][2], f32x16 (&nxt)[QB][2], auto copy_tag, auto stage_tag) __attribute__((always_inline)) {
     constexpr int STG = decltype(stage_tag)::value;
-    const unsigned char *sV = sVbase + (STG >= 0 ? STG : (tb + t) % NSTG) * TILE_BYTES;
+    unsigned va[DB];
+    const auto v_off = v_stage(stage_tag, STG >= 0 ? STG : (tb + t) % NSTG, va);
     if constexpr (!EARLY_MAX) {
       const bool moved = take_max(t, edge_tag, s_cur);
       rescale(moved);
@@ -846,7 +873,12 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-        for (int d = 0; d < DB; ++d) o[0][d] = Mfma32<DT>::run(read_v(sV, kk, d), pf[0][kk], o[0][d]);
+        for (int d = 0; d < DB; ++d) {
+          u32x4 vf;
+          issue_v(va, v_off, kk, d, vf);
+          v_landed(std::integral_constant<int, 0>{}, vf);
+          o[0][d] = Mfma32<DT>::run(vf, pf[0][kk], o[0][d]);
+        }
     } else {
       // Both phases are written as short chunks -- a few MFMAs and their share of
       // the vector-ALU work -- each closed by a full scheduling fence: MFMA issue
@@ -921,16 +953,21 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       float mx[QB];
 #pragma unroll
       for (int qi = 0; qi < QB; ++qi) mx[qi] = -INFINITY;
-      u32x4 vf = read_v(sV, 0, 0);
+      u32x4 vr[2];  // the fragment being multiplied and the one on its way
+      issue_v(va, v_off, 0, 0, vr[0]);
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk) {
 #pragma unroll
         for (int d = 0; d < DB; ++d) {
-          const int nxt = kk * DB + d + 1;
-          const u32x4 vn = nxt < 4 * DB ? read_v(sV, nxt / DB, nxt % DB) : vf;
+          const int idx = kk * DB + d;
+          if (idx + 1 < 4 * DB) {
+            issue_v(va, v_off, (idx + 1) / DB, (idx + 1) % DB, vr[(idx + 1) & 1]);
+            v_landed(std::integral_constant<int, 2>{}, vr[idx & 1]);
+          } else {
+            v_landed(std::integral_constant<int, 0>{}, vr[idx & 1]);
+          }
 #pragma unroll
-          for (int qi = 0; qi < QB; ++qi) o[qi][d] = Mfma32<DT>::run(vf, pf[qi][kk], o[qi][d]);
-          vf = vn;
+          for (int qi = 0; qi < QB; ++qi) o[qi][d] = Mfma32<DT>::run(vr[idx & 1], pf[qi][kk], o[qi][d]);
         }
 #pragma unroll
         for (int qi = 0; qi < QB; ++qi)
@@ -970,7 +1007,8 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
   // The iteration of the last tile any query of the wave may keep: its exponentials and its P.V product.
   // The tile after it has no key for this wave: no score product and no maximum.
   auto last_live_iteration = [&](int t) __attribute__((always_inline)) {
-    const unsigned char *sV = sVbase + ((tb + t) % NSTG) * TILE_BYTES;
+    unsigned va[DB];
+    const auto v_off = v_stage(std::integral_constant<int, -1>{}, (tb + t) % NSTG, va);
 #pragma unroll
     for (int qi = 0; qi < QB; ++qi) {
       float lsum = 0.0f;
@@ -992,7 +1030,9 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
       for (int d = 0; d < DB; ++d) {
-        const u32x4 vf = read_v(sV, kk, d);
+        u32x4 vf;
+        issue_v(va, v_off, kk, d, vf);
+        v_landed(std::integral_constant<int, 0>{}, vf);
 #pragma unroll
         for (int qi = 0; qi < QB; ++qi) o[qi][d] = Mfma32<DT>::run(vf, pf[qi][kk], o[qi][d]);
       }
