@@ -1366,7 +1366,10 @@ __global__ void __launch_bounds__(WM *WN * 64) contraction_kernel(const Contract
         __builtin_amdgcn_sched_barrier(0);
       }
       __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // tile kt+1 has landed; newer requests stay in flight
-      __syncthreads();
+      // (the barrier alone: with the fences of __syncthreads() the compiler waits for every request in flight)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
       dma(fill, fill + A_STAGE, tile_f * BK, ((KS - 1) * L) / KS, L);
       read_operands(0, nxt, nxt + A_STAGE, 0);
       mma((KS - 1) & 1);

@@ -225,7 +225,11 @@ __global__ void __launch_bounds__(WM *WN * 64) conv_patch_kernel(const Contracti
         mma(ks & 1);
       }
       __builtin_amdgcn_s_waitcnt(WAIT_TILE);  // tile kt+1 has landed; newer requests stay in flight
-      __syncthreads();
+      // (the barrier alone: with the fences of __syncthreads() the compiler waits for every request in flight,
+      // and the ring is no deeper than one tile)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
       // the last k-step of the tile runs behind the barrier, together with the first
       // operand reads of the next tile
       read_operands(0, ring + nxt_i * B_STAGE, 0);
