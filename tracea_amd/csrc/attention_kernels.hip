@@ -828,7 +828,9 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     } else if constexpr (PAIR_SYNC) {
       if ((tt & 1) == 0) {
         __builtin_amdgcn_s_waitcnt(WAIT_TILES);
-        __syncthreads();
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         load_k(tt + 3, sKbase + ((tt + 3) % NSTG) * TILE_BYTES);
         load_v(tt + 2, sVbase + ((tt + 2) % NSTG) * TILE_BYTES);
         load_k(tt + 4, sKbase + ((tt + 4) % NSTG) * TILE_BYTES);
@@ -836,7 +838,11 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
       }
     } else {
       __builtin_amdgcn_s_waitcnt(WAIT_TILES);  // K(tt+1) and V(tt), requested NSTG-1 iterations ago
-      __syncthreads();
+      // (the barrier alone: with the fences of __syncthreads() the compiler waits for every request in flight,
+      // and a ring of three or four stages is no deeper than two)
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
       load_k(ahead(tt + NSTG), sKbase + ((tb + tt) % NSTG) * TILE_BYTES);
       load_v(ahead(tt + NSTG - 1), sVbase + ((tb + tt + NSTG - 1) % NSTG) * TILE_BYTES);
     }
