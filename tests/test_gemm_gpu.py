@@ -38,8 +38,11 @@ def test_fp32_1024_matches_cpu_packed_path(tracea_gpu):
 # fp32 kernels by shape: the 64x64 tile (few large tiles: the first two, (200, 300, 1000) split three
 # ways along K, (1000, 1000, 40) with a ragged last K tile and an odd tile count), the 128x128 tile
 # (2047 x 2044: 256 large tiles, one per CU), the any-layout kernel (N not a multiple of 4)
+# (K tiles of 32 for launches of at most one workgroup per CU: (512, 512, 1040) with half a K tile at the
+# end and four K ranges of an odd number of 16-wide tiles, (1024, 1024, 1072) unsplit, (320, 256, 2064) split)
 @pytest.mark.parametrize("shape", [(64, 64, 64), (100, 36, 52), (129, 257, 200), (5, 4, 8), (200, 300, 1000),
-                                   (1000, 1000, 40), (2047, 2044, 72), (192, 64, 16), (65, 68, 4)])
+                                   (1000, 1000, 40), (2047, 2044, 72), (192, 64, 16), (65, 68, 4),
+                                   (512, 512, 1040), (1024, 1024, 1072), (320, 256, 2064), (768, 1024, 1040)])
 def test_fp32_edges_and_fallback(tracea_gpu, shape):
     m, n, k = shape
     rng = np.random.default_rng(m * 7 + n)
