@@ -856,6 +856,36 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     }
   };
 
+  // DEFER: the requests of an iteration are not issued in a block behind its barrier, where they hold every wave
+  // of the workgroup at once (a request holds its wave for some 130 cycles, and the matrix pipes stand still),
+  // but one by one behind the MFMAs of the first k-steps of phase A.
+  constexpr bool DEFER = EARLY_MAX && !PP && !PAIR_SYNC;
+  auto head_wait = [&](int tt) __attribute__((always_inline)) {
+    if constexpr (DEFER) {
+      __builtin_amdgcn_s_waitcnt(WAIT_TILES);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    } else {
+      head_of(tt);
+    }
+  };
+  // request r of iteration tt: r < NI a piece of K(tt+NSTG), else a piece of V(tt+NSTG-1)
+  auto request_nth = [&](int tt, int r) __attribute__((always_inline)) {
+    if (r < NI) {
+      const unsigned adv = (unsigned)ahead(tt + NSTG) * (unsigned)(FA_BKV * 2) * (unsigned)a.k_ss;
+      unsigned char *dst = sKbase + ((tb + tt) % NSTG) * TILE_BYTES;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_k, (__attribute__((address_space(3))) void *)(dst + (r * WAVES + wave_u) * RPI * ROW_BYTES), 16, (int)(k_voff[r] + adv), 0, 0, 0);
+    } else {
+      const unsigned adv = (unsigned)ahead(tt + NSTG - 1) * (unsigned)(FA_BKV * 2) * (unsigned)a.v_ss;
+      unsigned char *dst = sVbase + ((tb + tt + NSTG - 1) % NSTG) * TILE_BYTES;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_v, (__attribute__((address_space(3))) void *)(dst + ((r - NI) * WAVES + wave_u) * RPI * ROW_BYTES), 16,
+          (int)(v_voff[r - NI] + adv), 0, 0, 0);
+    }
+  };
+
   // One iteration, compiled twice: EDGE tiles (sequence end or causal diagonal)
   // mask scores with selects, interior tiles do not test at all.  Either body is
   // branch-free up to the optional rescale, so MFMAs and vector-ALU work can be
@@ -925,6 +955,12 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
           // (SHIFT: from -m, and the shift of the whole block costs no instruction)
           nxt[qi][0] = Mfma32<DT>::run(kf0, qf[qi][ks], ks == 0 ? (SHIFT ? negm[SHIFT ? qi : 0] : zero16) : nxt[qi][0]);
           nxt[qi][1] = Mfma32<DT>::run(kf1, qf[qi][ks], ks == 0 ? (SHIFT ? negm[SHIFT ? qi : 0] : zero16) : nxt[qi][1]);
+        }
+        if constexpr (DEFER) {
+          constexpr int PER_CHUNK = (2 * NI + KS - 1) / KS;
+#pragma unroll
+          for (int x = 0; x < PER_CHUNK; ++x)
+            if (ks * PER_CHUNK + x < 2 * NI) request_nth(t, ks * PER_CHUNK + x);
         }
 #pragma unroll
         for (int j = 0; j < EPC; ++j) {
@@ -1118,24 +1154,24 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     constexpr bool CONST_STAGES = NSTG == 2 && ITEMS == 1;
     constexpr int S0 = CONST_STAGES ? 0 : -1, S1 = CONST_STAGES ? 1 : -1;
     if (CONST_STAGES && t < interior_end && ((tb + t) & 1)) {
-      head_of(t);
+      head_wait(t);
       iteration(t, std::false_type{});
       ++t;
     }
     for (; t + 1 < interior_end; t += 2) {
-      head_of(t);
+      head_wait(t);
       iteration_on(t, std::false_type{}, s_cur, s_nxt, std::false_type{}, std::integral_constant<int, S0>{});
-      head_of(t + 1);
+      head_wait(t + 1);
       iteration_on(t + 1, std::false_type{}, s_nxt, s_cur, std::false_type{}, std::integral_constant<int, S1>{});
     }
     if (t < interior_end) {
-      head_of(t);
+      head_wait(t);
       iteration(t, std::false_type{});
       ++t;
     }
   } else {
     for (; t < interior_end; ++t) {
-      head_of(t);
+      head_wait(t);
       iteration(t, std::false_type{});
     }
   }
@@ -1147,7 +1183,7 @@ fa2_fwd_pipe_kernel(const AttentionArgs a) {
     // causal mask that is one and a half iterations of two of the four waves and half an iteration of the others.)
     const int last_live = wave_last_key / FA_BKV;
     for (; t < last_live; ++t) {
-      head_of(t);
+      head_wait(t);
       iteration(t, std::true_type{});
     }
     head_of(t);
